@@ -1,0 +1,80 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions, wave64 reductions,
+// and the error channel of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace kvcm {
+
+constexpr int kWave = 64;
+
+// Storage types.  bf16 is kept as raw bits so that loads can be vectorised freely.
+struct bf16_t { uint16_t bits; };
+
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest, ties to even
+  return static_cast<uint16_t>(u >> 16);
+}
+
+template <class T> __device__ __forceinline__ float load_f(const T* p);
+template <> __device__ __forceinline__ float load_f<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_f<bf16_t>(const bf16_t* p) { return bf16_bits_to_float(p->bits); }
+
+template <class T> __device__ __forceinline__ void store_f(T* p, float v);
+template <> __device__ __forceinline__ void store_f<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_f<bf16_t>(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
+
+// Value after one trip through the storage type (identity for float).
+template <class T> __device__ __forceinline__ float round_to(float v);
+template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_to<bf16_t>(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Sum over a block of THREADS threads (a multiple of 64); every thread gets the result.  The
+// order of additions depends on THREADS only.
+template <int THREADS>
+__device__ __forceinline__ float block_sum(float v, float* scratch /* THREADS/64 + 1 floats */) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < THREADS / kWave; ++w) s += scratch[w];
+    scratch[THREADS / kWave] = s;
+  }
+  __syncthreads();
+  const float r = scratch[THREADS / kWave];
+  __syncthreads();
+  return r;
+}
+
+// ---- host side ------------------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int launch_status(const char* what);
+
+}  // namespace kvcm
+
+#define KVCM_REQUIRE(cond, ...)          \
+  do {                                   \
+    if (!(cond)) {                       \
+      kvcm::set_error(__VA_ARGS__);      \
+      return -1;                         \
+    }                                    \
+  } while (0)

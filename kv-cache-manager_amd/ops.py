@@ -1,0 +1,210 @@
+"""Calls into libkvcm_hip.so.  Every function takes torch tensors that live on the GPU, checks on
+the host that their shapes and dtypes are what the kernel assumes, and launches on torch's
+current stream.  There is no fallback: without the library (or without a GPU) these raise.
+"""
+import ctypes as C
+import threading
+
+import torch
+
+from .csrc import build as _build
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _declare(lib):
+    vp, i, f = C.c_void_p, C.c_int, C.c_float
+
+    def fn(name, *args):
+        g = getattr(lib, name)
+        g.restype = C.c_int
+        g.argtypes = list(args)
+
+    lib.kvcm_hip_last_error.restype = C.c_char_p
+    fn("kvcm_embed", vp, vp, i, vp, i, i, i, vp)
+    fn("kvcm_rmsnorm", vp, vp, i, vp, vp, i, vp, i, i, i, f, i, vp)
+    fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
+    fn("kvcm_swiglu", vp, vp, i, i, i, vp)
+    fn("kvcm_add_residual", vp, vp, i, C.c_longlong, vp)
+    fn("kvcm_gemm_f32", vp, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_gemm_bf16", vp, vp, vp, i, i, i, i, i, i, i, vp)
+    fn("kvcm_attention_generic", vp, i, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp)
+    fn("kvcm_sample", vp, i, vp, vp, vp, vp, vp, i, i, vp)
+
+
+def lib():
+    global _lib
+    with _lock:
+        if _lib is None:
+            loaded = C.CDLL(_build.build_hip())
+            _declare(loaded)
+            _lib = loaded
+    return _lib
+
+
+def library_path():
+    lib()
+    return _lib._name
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(rc):
+    if rc != 0:
+        raise KernelError(lib().kvcm_hip_last_error().decode())
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _need(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must live on the GPU")
+
+
+def _i32(t, name, n=None):
+    if t is None:
+        return
+    _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be a contiguous int32 tensor")
+    if n is not None:
+        _need(t.numel() >= n, f"{name} holds {t.numel()} entries, {n} are needed")
+
+
+def _rows2d(t, name):
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-d with unit inner stride")
+
+
+# --------------------------------------------------------------------------------------------
+def embed(ids, table, out):
+    """out[t, :] = float(table[ids[t], :]);  out is the 32-bit residual stream [T, H]."""
+    _dev(ids, table, out)
+    T, H = out.shape
+    _i32(ids, "ids", T)
+    _need(table.dim() == 2 and table.shape[1] == H and table.is_contiguous(), "embedding table must be [V, H]")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "residual stream must be contiguous float32")
+    _check(lib().kvcm_embed(_ptr(ids), _ptr(table), _DT[table.dtype], _ptr(out), T, H, table.shape[0], _stream()))
+
+
+def rmsnorm(x, weight, out, eps, add=None, rows=None, write_back=True):
+    """v = x[src] (+ add[src]); x[src] = v when write_back; out[r] = weight * round(v * rsqrt(mean v^2 + eps)).
+    src = rows[r] if rows is given, else r."""
+    _dev(x, weight, out, add, rows)
+    R, H = out.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == H, "x must be contiguous float32 [T, H]")
+    _need(weight.numel() == H and weight.is_contiguous(), "norm weight must have H entries")
+    _need(out.is_contiguous(), "norm output must be contiguous")
+    if rows is None:
+        _need(x.shape[0] >= R, "x has fewer rows than the output")
+    else:
+        _i32(rows, "rows", R)
+    if add is not None:
+        _need(add.shape == x.shape and add.is_contiguous(), "add must match x")
+    wb = bool(write_back) and add is not None and rows is None
+    _check(lib().kvcm_rmsnorm(_ptr(x), _ptr(add), _DT[add.dtype] if add is not None else 0, _ptr(rows), _ptr(weight),
+                              _DT[weight.dtype], _ptr(out), _DT[out.dtype], R, H, float(eps), int(wb), _stream()))
+
+
+def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcache=None, vcache=None,
+               block_size=0, rows=None):
+    """Rotates the q and k heads of the fused rows in place (inv_freq given) and copies k (rotated)
+    and v to the paged cache (slots given).  Cache layout [pages, nkv, block_size, hd]."""
+    _dev(qkv, positions, inv_freq, slots, kcache, vcache)
+    _rows2d(qkv, "qkv")
+    T = qkv.shape[0] if rows is None else rows
+    _need(qkv.shape[1] >= (nh + 2 * nkv) * hd, "qkv rows are too short for the head layout")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == hd // 2 and inv_freq.is_contiguous(),
+              "inv_freq must hold head_dim/2 float32 values")
+        _i32(positions, "positions", T)
+        _need(positions is not None, "rotation needs positions")
+    if slots is not None:
+        _i32(slots, "slots", T)
+        for c in (kcache, vcache):
+            _need(c is not None and c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
+                  and tuple(c.shape[1:]) == (nkv, block_size, hd), "cache must be [pages, nkv, block_size, hd]")
+    _check(lib().kvcm_rope_cache(_ptr(qkv), _DT[qkv.dtype], qkv.stride(0), _ptr(positions), _ptr(inv_freq),
+                                 _ptr(slots), _ptr(kcache), _ptr(vcache), T, nh, nkv, hd, block_size, _stream()))
+
+
+def swiglu(gate_up, out):
+    _dev(gate_up, out)
+    T, I = out.shape
+    _need(gate_up.shape == (T, 2 * I) and gate_up.is_contiguous() and out.is_contiguous()
+          and gate_up.dtype == out.dtype, "swiglu needs [T, 2I] -> [T, I] of one dtype")
+    _check(lib().kvcm_swiglu(_ptr(gate_up), _ptr(out), _DT[out.dtype], T, I, _stream()))
+
+
+def add_residual(x, y):
+    _dev(x, y)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape,
+          "add_residual needs a float32 x and a y of the same shape")
+    _check(lib().kvcm_add_residual(_ptr(x), _ptr(y), _DT[y.dtype], x.numel(), _stream()))
+
+
+def gemm(x, w, out):
+    """out[M, N] = x[M, K] @ w[N, K]^T.  float32 x float32 -> float32 (plain FMA), or
+    bfloat16 x bfloat16 -> bfloat16 | float32 (MFMA, 32-bit accumulation)."""
+    _dev(x, w, out)
+    for t, n in ((x, "x"), (w, "w"), (out, "out")):
+        _rows2d(t, n)
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K and out.shape == (M, N), f"gemm shapes do not agree: {tuple(x.shape)} {tuple(w.shape)} {tuple(out.shape)}")
+    if x.dtype == torch.float32:
+        _need(w.dtype == torch.float32 and out.dtype == torch.float32, "a float32 gemm needs float32 operands")
+        _check(lib().kvcm_gemm_f32(_ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0), _stream()))
+    else:
+        _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm operands must both be bfloat16")
+        _check(lib().kvcm_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, x.stride(0), w.stride(0),
+                                    out.stride(0), _stream()))
+
+
+def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, nh, nkv, hd, scale, window=0,
+              rows=None):
+    """out[r, h, :] = softmax(scale * q[r, h] . K[0:ctx_r]) V[0:ctx_r] over the paged cache."""
+    _dev(q, out, kcache, vcache, tables, row_seq, ctx_lens)
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    T = q.shape[0] if rows is None else rows
+    _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype, "attention operands must share one dtype")
+    _need(kcache.dim() == 4 and kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape == vcache.shape
+          and kcache.shape[1] == nkv and kcache.shape[3] == hd, "cache must be [pages, nkv, block_size, hd]")
+    _i32(row_seq, "row_seq", T)
+    _i32(ctx_lens, "ctx_lens", T)
+    _i32(tables, "tables")
+    _check(lib().kvcm_attention_generic(_ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache),
+                                        _ptr(vcache), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh,
+                                        nkv, hd, kcache.shape[2], float(scale), int(window), _stream()))
+
+
+def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_index=None):
+    """out[r] = argmax of row r, or a Gumbel-max draw where temperature[r] > 0."""
+    _dev(logits, out, temperature, seeds, request_ids, token_index)
+    _rows2d(logits, "logits")
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "logits must be float32")
+    _i32(out, "out", R)
+    if temperature is not None:
+        _need(temperature.dtype == torch.float32 and temperature.numel() >= R, "temperature must be float32 [R]")
+        _need(seeds is not None and seeds.dtype in (torch.int64, torch.uint64) and seeds.numel() >= R, "seeds must be 64-bit [R]")
+        _need(request_ids is not None and request_ids.dtype == torch.int64 and request_ids.numel() >= R, "request ids must be int64 [R]")
+        _i32(token_index, "token_index", R)
+    _check(lib().kvcm_sample(_ptr(logits), logits.stride(0), _ptr(temperature), _ptr(seeds), _ptr(request_ids),
+                             _ptr(token_index), _ptr(out), R, V, _stream()))

@@ -145,7 +145,7 @@ def gumbel_uniforms(seed, request_id, token_index, vocab):
     h = _mix64(h ^ ((token_index * 0xBF58476D1CE4E5B9) & _M64))
     out = np.empty(vocab, dtype=np.float64)
     for j in range(vocab):
-        out[j] = ((_mix64((h + j) & _M64) >> 40) + 0.5) / float(1 << 24)
+        out[j] = ((_mix64((h + j) & _M64) >> 41) + 0.5) / float(1 << 23)
     return out
 
 

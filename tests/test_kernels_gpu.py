@@ -1,0 +1,478 @@
+"""Each HIP kernel alone against the plain NumPy function of the same formula, at sizes the tiny
+models do not use.  Held vectors of the reference's own kernel tests are restated where they exist
+(tests/test_kernels.cu, tests/test_paged_attention.cu)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from kvcm_amd import ops as _ops
+    _ops.lib()
+    return _ops
+
+
+def _t(a, dtype):
+    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+def _bf16_grid(a):
+    return plain.round_bf16(a)
+
+
+# ------------------------------------------------------------------------------- embedding
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding_gathers_rows(ops, dtype):
+    rng = np.random.default_rng(0)
+    V, H = 387, 100
+    table = _bf16_grid(rng.normal(size=(V, H)))
+    ids = np.array([0, 386, 5, 5, 17], dtype=np.int32)
+    out = torch.zeros(len(ids), H, dtype=torch.float32, device=DEV)
+    ops.embed(_t(ids, torch.int32), _t(table, dtype), out)
+    np.testing.assert_array_equal(_np(out), plain.embedding(table, ids))
+
+
+# -------------------------------------------------------------------------------- RMS norm
+def test_rmsnorm_with_row_gather_reference_vector(ops):
+    # tests/test_kernels.cu:25-49: R=5, H=2048, rows {4,0,2}, x ~ 3 N(0,1), w ~ 1 + 0.1 N, eps 1e-5
+    rng = np.random.default_rng(1)
+    R, H = 5, 2048
+    x = (rng.normal(size=(R, H)) * 3).astype(np.float32)
+    w = _bf16_grid(1 + 0.1 * rng.normal(size=H))
+    rows = np.array([4, 0, 2], dtype=np.int32)
+    out = torch.zeros(3, H, dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(_t(x, torch.float32), _t(w, torch.bfloat16), out, 1e-5, rows=_t(rows, torch.int32))
+    ref = plain.rms_norm(x[rows], w, 1e-5, plain.round_bf16)
+    got = _np(out)
+    # one bfloat16 step at most (a product that lands on a rounding tie in one of the two)
+    assert np.max(np.abs(got - ref) / np.maximum(1.0, np.abs(ref))) <= 2 ** -7
+    assert np.mean(got == ref) > 0.995
+    out32 = torch.zeros(3, H, dtype=torch.float32, device=DEV)
+    ops.rmsnorm(_t(x, torch.float32), _t(w, torch.float32), out32, 1e-5, rows=_t(rows, torch.int32))
+    np.testing.assert_allclose(_np(out32), plain.rms_norm(x[rows], w, 1e-5), rtol=2e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("H", [96, 1000, 4099])
+def test_rmsnorm_fused_add_updates_the_stream(ops, H):
+    rng = np.random.default_rng(2)
+    T = 7
+    x = rng.normal(size=(T, H)).astype(np.float32)
+    y = rng.normal(size=(T, H)).astype(np.float32)
+    w = rng.normal(size=H).astype(np.float32)
+    xt = _t(x, torch.float32)
+    out = torch.zeros(T, H, dtype=torch.float32, device=DEV)
+    ops.rmsnorm(xt, _t(w, torch.float32), out, 1e-6, add=_t(y, torch.float32))
+    np.testing.assert_array_equal(_np(xt), (x + y).astype(np.float64))
+    np.testing.assert_allclose(_np(out), plain.rms_norm((x + y).astype(np.float64), w, 1e-6), rtol=3e-6, atol=1e-6)
+    # gathered add: the stream is left alone
+    xt = _t(x, torch.float32)
+    rows = _t([6, 1], torch.int32)
+    out = torch.zeros(2, H, dtype=torch.float32, device=DEV)
+    ops.rmsnorm(xt, _t(w, torch.float32), out, 1e-6, add=_t(y, torch.float32), rows=rows)
+    np.testing.assert_array_equal(_np(xt), x.astype(np.float64))
+    np.testing.assert_allclose(_np(out), plain.rms_norm((x + y)[[6, 1]].astype(np.float64), w, 1e-6), rtol=3e-6, atol=1e-6)
+
+
+def test_rmsnorm_eps_is_inside_the_root(ops):
+    # x = c * ones, w = 1  ->  c / sqrt(c^2 + eps); with eps as large as c^2 a misplaced eps shows
+    H, c, eps = 64, 0.01, 1e-4
+    out = torch.zeros(1, H, dtype=torch.float32, device=DEV)
+    ops.rmsnorm(torch.full((1, H), c, device=DEV), torch.ones(H, device=DEV), out, eps)
+    np.testing.assert_allclose(_np(out), c / math.sqrt(c * c + eps), rtol=1e-6)
+
+
+# ---------------------------------------------------------------------------------- rotary
+def _inv_freq(hd, theta):
+    j = np.arange(hd // 2, dtype=np.float32)
+    return (np.float32(1.0) / np.power(np.float32(theta), (np.float32(2.0) * j) / np.float32(hd))).astype(np.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_matches_rotate_half_reference_vector(ops, dtype):
+    # tests/test_kernels.cu:51-78: T=3, NH=4, NKV=2, HD=64, positions {0,7,1999}, theta 1e4
+    rng = np.random.default_rng(3)
+    T, NH, NKV, HD = 3, 4, 2, 64
+    qkv = _bf16_grid(rng.normal(size=(T, (NH + 2 * NKV) * HD)))
+    pos = np.array([0, 7, 1999], dtype=np.int32)
+    t = _t(qkv, dtype)
+    ops.rope_cache(t, NH, NKV, HD, positions=_t(pos, torch.int32), inv_freq=_t(_inv_freq(HD, 1e4), torch.float32))
+    got = _np(t).reshape(T, NH + 2 * NKV, HD)
+    src = qkv.reshape(T, NH + 2 * NKV, HD)
+    r16 = plain.round_bf16 if dtype == torch.bfloat16 else None
+    ref = plain.rotary(src[:, :NH + NKV], pos, 1e4, r16)
+    tol = 2 ** -5 if dtype == torch.bfloat16 else 1e-5     # |values| < 8: one bfloat16 step there
+    np.testing.assert_allclose(got[:, :NH + NKV], ref, atol=tol, rtol=0)
+    np.testing.assert_array_equal(got[:, NH + NKV:], src[:, NH + NKV:])        # v heads untouched
+    np.testing.assert_array_equal(got[0], src[0])                               # position 0 is the identity
+    # each (j, j + hd/2) pair keeps its length
+    n0 = src[:, :NH + NKV, :HD // 2] ** 2 + src[:, :NH + NKV, HD // 2:] ** 2
+    n1 = got[:, :NH + NKV, :HD // 2] ** 2 + got[:, :NH + NKV, HD // 2:] ** 2
+    np.testing.assert_allclose(n1, n0, rtol=3e-2 if dtype == torch.bfloat16 else 1e-5, atol=1e-3 if dtype == torch.bfloat16 else 1e-6)
+
+
+def test_rope_dot_products_depend_on_distance_only(ops):
+    rng = np.random.default_rng(4)
+    HD = 48
+    q = rng.normal(size=(1, HD)).astype(np.float32)
+    k = rng.normal(size=(1, HD)).astype(np.float32)
+    inv = _t(_inv_freq(HD, 5e5), torch.float32)
+
+    def dot(pq, pk):
+        row = _t(np.concatenate([q, k, k], axis=1), torch.float32)   # one q head, one k head, one v head
+        rows = torch.cat([row, row])
+        ops.rope_cache(rows, 1, 1, HD, positions=_t([pq, pk], torch.int32), inv_freq=inv)
+        a = _np(rows)
+        return float(a[0, :HD] @ a[1, HD:2 * HD])
+
+    base = dot(5, 2)
+    assert abs(dot(105, 102) - base) < 1e-4 and abs(dot(17, 14) - base) < 1e-4
+    assert abs(dot(5, 3) - base) > 1e-3
+
+
+# ------------------------------------------------------------------------------- KV write
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reshape_and_cache_scatters_to_slots(ops, dtype):
+    # tests/test_paged_attention.cu:230-265: T=37, KVH=4, HD=64, B=16, NB=10, padded stride,
+    # random slot permutation, slot -1 skipped and its natural slot stays zero
+    rng = np.random.default_rng(5)
+    T, KVH, HD, B, NB, NH = 37, 4, 64, 16, 10, 4
+    stride = (NH + 2 * KVH) * HD + 24
+    rows = _bf16_grid(rng.normal(size=(T, stride)))
+    slots = rng.permutation(NB * B)[:T].astype(np.int32)
+    skipped = 11
+    natural = slots[skipped]
+    slots[skipped] = -1
+    kc = torch.zeros(NB, KVH, B, HD, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    buf = _t(rows, dtype)
+    ops.rope_cache(buf[:, :stride], NH, KVH, HD, slots=_t(slots, torch.int32), kcache=kc, vcache=vc, block_size=B)
+    K, V = _np(kc), _np(vc)
+    for t in range(T):
+        k_src = rows[t, NH * HD:(NH + KVH) * HD].reshape(KVH, HD)
+        v_src = rows[t, (NH + KVH) * HD:(NH + 2 * KVH) * HD].reshape(KVH, HD)
+        if slots[t] < 0:
+            assert not K[natural // B, :, natural % B].any() and not V[natural // B, :, natural % B].any()
+            continue
+        np.testing.assert_array_equal(K[slots[t] // B, :, slots[t] % B], k_src)
+        np.testing.assert_array_equal(V[slots[t] // B, :, slots[t] % B], v_src)
+    assert np.count_nonzero(K.any(axis=(1, 3))) == T - 1            # nothing else was touched
+
+
+def test_fused_rope_and_cache_write_stores_rotated_keys(ops):
+    rng = np.random.default_rng(6)
+    T, NH, KVH, HD, B = 5, 6, 2, 32, 8
+    rows = rng.normal(size=(T, (NH + 2 * KVH) * HD)).astype(np.float32)
+    pos = np.array([3, 4, 5, 40, 41], dtype=np.int32)
+    slots = np.array([8, 9, 10, 0, 1], dtype=np.int32)
+    kc = torch.zeros(3, KVH, B, HD, device=DEV)
+    vc = torch.zeros_like(kc)
+    buf = _t(rows, torch.float32)
+    ops.rope_cache(buf, NH, KVH, HD, positions=_t(pos, torch.int32), inv_freq=_t(_inv_freq(HD, 1e4), torch.float32),
+                   slots=_t(slots, torch.int32), kcache=kc, vcache=vc, block_size=B)
+    k_ref = plain.rotary(rows[:, NH * HD:(NH + KVH) * HD].reshape(T, KVH, HD), pos, 1e4)
+    K, V = _np(kc), _np(vc)
+    for t in range(T):
+        np.testing.assert_allclose(K[slots[t] // B, :, slots[t] % B], k_ref[t], atol=1e-5)
+        np.testing.assert_array_equal(V[slots[t] // B, :, slots[t] % B],
+                                      rows[t, (NH + KVH) * HD:].reshape(KVH, HD).astype(np.float64))
+
+
+# ---------------------------------------------------------------------------------- SwiGLU
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(ops, dtype):
+    # tests/test_kernels.cu:80-94: T=2, I=300
+    rng = np.random.default_rng(7)
+    T, I = 2, 300
+    gu = _bf16_grid(rng.normal(size=(T, 2 * I)))
+    gu[0, :3] = [0.0, 30.0, -30.0]          # silu(0) = 0, silu(x) -> x, silu(-x) -> 0
+    out = torch.zeros(T, I, dtype=dtype, device=DEV)
+    ops.swiglu(_t(gu, dtype), out)
+    r16 = plain.round_bf16 if dtype == torch.bfloat16 else None
+    ref = plain.swiglu(gu, r16)
+    got = _np(out)
+    np.testing.assert_allclose(got, ref, rtol=2 ** -7 if r16 else 2e-6, atol=1e-7)
+    assert got[0, 0] == 0.0
+    np.testing.assert_allclose(got[0, 1], 30.0 * gu[0, I + 1], rtol=2 ** -7)
+    assert abs(got[0, 2]) < 1e-10
+
+
+# -------------------------------------------------------------------------------- residual
+def test_add_residual(ops):
+    rng = np.random.default_rng(8)
+    x = rng.normal(size=(3, 1001)).astype(np.float32)
+    y = _bf16_grid(rng.normal(size=(3, 1001)))
+    xt = _t(x, torch.float32)
+    ops.add_residual(xt, _t(y, torch.bfloat16))
+    np.testing.assert_array_equal(_np(xt), (x + y.astype(np.float32)).astype(np.float64))
+
+
+# ------------------------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (3, 130, 96), (70, 176, 64), (129, 65, 1000), (16, 64, 16), (33, 300, 177)])
+def test_gemm_f32_equals_x_wT(ops, M, N, K):
+    rng = np.random.default_rng(M * 1000 + N)
+    x = rng.normal(size=(M, K)).astype(np.float32)
+    w = rng.normal(size=(N, K)).astype(np.float32)
+    out = torch.zeros(M, N, device=DEV)
+    ops.gemm(_t(x, torch.float32), _t(w, torch.float32), out)
+    ref = plain.linear(x, w)
+    np.testing.assert_allclose(_np(out), ref, rtol=0, atol=2e-6 * math.sqrt(K) * 4)
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch(ops):
+    rng = np.random.default_rng(9)
+    K, N = 333, 200
+    x = rng.normal(size=(150, K)).astype(np.float32)
+    w = _t(rng.normal(size=(N, K)).astype(np.float32), torch.float32)
+    full = torch.zeros(150, N, device=DEV)
+    ops.gemm(_t(x, torch.float32), w, full)
+    for lo, hi in [(0, 1), (17, 19), (60, 100), (149, 150)]:
+        part = torch.zeros(hi - lo, N, device=DEV)
+        ops.gemm(_t(x[lo:hi], torch.float32), w, part)
+        assert torch.equal(part, full[lo:hi]), "a row's sum changed with the rows beside it"
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 32), (5, 100, 96), (64, 64, 64), (70, 176, 200), (200, 333, 1024), (3, 50, 20)])
+def test_gemm_bf16_equals_x_wT(ops, M, N, K, out_dtype):
+    rng = np.random.default_rng(M * 1000 + N)
+    x = _bf16_grid(rng.normal(size=(M, K)))
+    w = _bf16_grid(rng.normal(size=(N, K)))
+    out = torch.zeros(M, N, dtype=out_dtype, device=DEV)
+    ops.gemm(_t(x, torch.bfloat16), _t(w, torch.bfloat16), out)
+    ref = plain.linear(x, w)
+    if out_dtype == torch.bfloat16:
+        np.testing.assert_allclose(_np(out), ref, rtol=2 ** -7, atol=1e-4 * math.sqrt(K))
+    else:
+        np.testing.assert_allclose(_np(out), ref, rtol=0, atol=3e-6 * math.sqrt(K) * 4)
+
+
+def test_gemm_bf16_fused_projection_equals_separate_ones(ops):
+    # the fused QKV product is the three products stacked
+    rng = np.random.default_rng(10)
+    x = _t(_bf16_grid(rng.normal(size=(9, 96))), torch.bfloat16)
+    ws = [_bf16_grid(rng.normal(size=(n, 96))) for n in (96, 32, 32)]
+    fused = torch.zeros(9, 160, dtype=torch.float32, device=DEV)
+    ops.gemm(x, _t(np.concatenate(ws), torch.bfloat16), fused)
+    col = 0
+    for w in ws:
+        part = torch.zeros(9, w.shape[0], dtype=torch.float32, device=DEV)
+        ops.gemm(x, _t(w, torch.bfloat16), part)
+        np.testing.assert_allclose(_np(fused[:, col:col + w.shape[0]]), _np(part), atol=1e-5)
+        col += w.shape[0]
+
+
+# ------------------------------------------------------------------------------- attention
+def _paged_problem(rng, ctx_lens, nh, nkv, hd, B, all_rows, shuffle=True, spare=7, dtype=torch.float32):
+    """Random Q/K/V on the bfloat16 grid, block tables over shuffled pages with unused spares
+    (tests/test_paged_attention.cu:41,53-64)."""
+    S = len(ctx_lens)
+    max_blocks = max((c + B - 1) // B for c in ctx_lens)
+    total = sum((c + B - 1) // B for c in ctx_lens)
+    nb = total + spare
+    phys = np.arange(nb)
+    if shuffle:
+        np.random.default_rng(77).shuffle(phys)
+    Kl = [_bf16_grid(rng.normal(size=(c, nkv, hd))) for c in ctx_lens]
+    Vl = [_bf16_grid(rng.normal(size=(c, nkv, hd))) for c in ctx_lens]
+    tables = np.zeros((S, max_blocks), dtype=np.int32)
+    Kc = np.zeros((nb, nkv, B, hd))
+    Vc = np.zeros((nb, nkv, B, hd))
+    nxt = 0
+    for s, c in enumerate(ctx_lens):
+        for b in range((c + B - 1) // B):
+            tables[s, b] = phys[nxt]
+            nxt += 1
+        for t in range(c):
+            Kc[tables[s, t // B], :, t % B] = Kl[s][t]
+            Vc[tables[s, t // B], :, t % B] = Vl[s][t]
+    row_seq, ctx = [], []
+    for s, c in enumerate(ctx_lens):
+        if all_rows:
+            row_seq += [s] * c
+            ctx += list(range(1, c + 1))
+        else:
+            row_seq.append(s)
+            ctx.append(c)
+    R = len(row_seq)
+    Q = _bf16_grid(rng.normal(size=(R, nh, hd)))
+    return dict(Q=Q, Kl=Kl, Vl=Vl, Kc=Kc, Vc=Vc, tables=tables, row_seq=np.array(row_seq, np.int32),
+                ctx=np.array(ctx, np.int32), S=S, R=R, max_blocks=max_blocks)
+
+
+def _run_attention(ops, P, nh, nkv, hd, dtype, window=0, scale=None):
+    out = torch.zeros(P["R"], nh * hd, dtype=dtype, device=DEV)
+    ops.attention(_t(P["Q"].reshape(P["R"], nh * hd), dtype), out, _t(P["Kc"], dtype), _t(P["Vc"], dtype),
+                  _t(P["tables"], torch.int32), P["max_blocks"], _t(P["row_seq"], torch.int32), _t(P["ctx"], torch.int32),
+                  nh, nkv, hd, scale if scale is not None else 1.0 / math.sqrt(hd), window)
+    return _np(out).reshape(P["R"], nh, hd)
+
+
+def _ref_attention(P, nh, nkv, hd, window=0, scale=None, r16=None):
+    ref = np.zeros((P["R"], nh, hd))
+    sc = scale if scale is not None else 1.0 / math.sqrt(hd)
+    for r in range(P["R"]):
+        s, c = P["row_seq"][r], P["ctx"][r]
+        ref[r] = plain.attention(P["Q"][r:r + 1], P["Kl"][s][:c], P["Vl"][s][:c], [c - 1], np.arange(c), sc, window, r16)[0]
+    return ref
+
+
+@pytest.mark.parametrize("B", [8, 16, 32, 64])
+@pytest.mark.parametrize("ctx", [1, 15, 16, 17, 2047])
+def test_paged_attention_decode_rows(ops, B, ctx):
+    # tests/test_paged_attention.cu:160-175: four sequences {ctx, ctx/2, 1, min(ctx+3, 2047)}
+    rng = np.random.default_rng(B * 10000 + ctx)
+    lens = [ctx, max(1, ctx // 2), 1, min(ctx + 3, 2047)]
+    P = _paged_problem(rng, lens, 8, 2, 64, B, all_rows=False)
+    got = _run_attention(ops, P, 8, 2, 64, torch.float32)
+    np.testing.assert_allclose(got, _ref_attention(P, 8, 2, 64), atol=2e-5, rtol=0)
+    got16 = _run_attention(ops, P, 8, 2, 64, torch.bfloat16)
+    np.testing.assert_allclose(got16, _ref_attention(P, 8, 2, 64), atol=1e-2, rtol=0)   # the reference's bound
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 8, 64), (16, 4, 128), (32, 4, 128), (3, 1, 32), (4, 2, 16), (6, 3, 48), (2, 1, 256), (5, 5, 80)])
+def test_paged_attention_head_shapes_prefill_rows_causal(ops, nh, nkv, hd):
+    # one row per position (tests/test_paged_attention.cu:177-185), head shapes of l.196-206 and more
+    rng = np.random.default_rng(nh * 100 + hd)
+    P = _paged_problem(rng, [33, 70, 5], nh, nkv, hd, 16, all_rows=True)
+    got = _run_attention(ops, P, nh, nkv, hd, torch.float32)
+    np.testing.assert_allclose(got, _ref_attention(P, nh, nkv, hd), atol=2e-5, rtol=0)
+
+
+def test_paged_attention_refuses_unsupported_head_dim(ops):
+    P = _paged_problem(np.random.default_rng(0), [4], 2, 1, 20, 4, all_rows=False)
+    with pytest.raises(ops.KernelError, match="head_dim"):
+        _run_attention(ops, P, 2, 1, 20, torch.float32)
+
+
+def test_paged_attention_shuffled_layout_is_bit_identical(ops):
+    # tests/test_paged_attention.cu:208-219
+    a = _paged_problem(np.random.default_rng(11), [200, 37, 64], 8, 2, 64, 16, all_rows=False, shuffle=True)
+    b = _paged_problem(np.random.default_rng(11), [200, 37, 64], 8, 2, 64, 16, all_rows=False, shuffle=False)
+    assert not np.array_equal(a["tables"], b["tables"])
+    for dt in (torch.float32, torch.bfloat16):
+        np.testing.assert_array_equal(_run_attention(ops, a, 8, 2, 64, dt), _run_attention(ops, b, 8, 2, 64, dt))
+
+
+def test_paged_attention_special_cases(ops):
+    rng = np.random.default_rng(12)
+    nh, nkv, hd, B = 4, 2, 32, 8
+    P = _paged_problem(rng, [1, 40], nh, nkv, hd, B, all_rows=False)
+    got = _run_attention(ops, P, nh, nkv, hd, torch.float32)
+    # one key: the output is that key's value, for each head's own KV head
+    for h in range(nh):
+        np.testing.assert_allclose(got[0, h], P["Vl"][0][0, h // 2], atol=1e-6)
+    # all keys equal: the output is the mean of the values
+    P["Kc"][:] = 0.25
+    P["Kl"] = [np.full_like(k, 0.25) for k in P["Kl"]]
+    got = _run_attention(ops, P, nh, nkv, hd, torch.float32)
+    for h in range(nh):
+        np.testing.assert_allclose(got[1, h], P["Vl"][1][:, h // 2].mean(0), atol=1e-6)
+
+
+def test_paged_attention_equals_dense_library_attention(ops):
+    # plain attention without rotation: a library routine with K/V repeated per group
+    rng = np.random.default_rng(13)
+    nh, nkv, hd, B, n = 6, 2, 64, 16, 50
+    P = _paged_problem(rng, [n], nh, nkv, hd, B, all_rows=True)
+    got = _run_attention(ops, P, nh, nkv, hd, torch.float32)
+    q = torch.tensor(P["Q"]).permute(1, 0, 2)[None]
+    k = torch.tensor(P["Kl"][0]).permute(1, 0, 2).repeat_interleave(nh // nkv, 0)[None]
+    v = torch.tensor(P["Vl"][0]).permute(1, 0, 2).repeat_interleave(nh // nkv, 0)[None]
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)[0].permute(1, 0, 2).numpy()
+    np.testing.assert_allclose(got, ref, atol=2e-5)
+
+
+def test_paged_attention_finds_a_far_key_among_hundreds(ops):
+    # one key far back (and across a page edge) is made to dominate; a lost page or a wrong
+    # table row would miss it
+    rng = np.random.default_rng(14)
+    nh, nkv, hd, B = 4, 1, 64, 16
+    for far in (0, 15, 16, 31, 500, 1023):
+        P = _paged_problem(rng, [1024], nh, nkv, hd, B, all_rows=False)
+        P["Q"][0, 2] = 0.0
+        P["Q"][0, 2, 5] = 40.0
+        kvec = np.zeros(hd)
+        kvec[5] = 40.0
+        P["Kl"][0][far, 0] = kvec
+        P["Kc"][P["tables"][0, far // B], 0, far % B] = kvec
+        got = _run_attention(ops, P, nh, nkv, hd, torch.float32, scale=1.0)
+        np.testing.assert_allclose(got[0, 2], P["Vl"][0][far, 0], atol=1e-5)
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 64, 100])
+def test_paged_attention_window_edge(ops, window):
+    rng = np.random.default_rng(15 + window)
+    nh, nkv, hd, B = 2, 1, 32, 8
+    P = _paged_problem(rng, [130], nh, nkv, hd, B, all_rows=True)
+    got = _run_attention(ops, P, nh, nkv, hd, torch.float32, window=window)
+    np.testing.assert_allclose(got, _ref_attention(P, nh, nkv, hd, window=window), atol=2e-5)
+    # the key just outside the window must be invisible: make it huge for the last row
+    r, edge = P["R"] - 1, 130 - 1 - window
+    if edge >= 0:
+        P["Q"][r, 0] = 0
+        P["Q"][r, 0, 3] = 30.0
+        kvec = np.zeros(hd)
+        kvec[3] = 30.0
+        P["Kl"][0][edge, 0] = kvec
+        P["Kc"][P["tables"][0, edge // B], 0, edge % B] = kvec
+        got = _run_attention(ops, P, nh, nkv, hd, torch.float32, window=window, scale=1.0)
+        ref = _ref_attention(P, nh, nkv, hd, window=window, scale=1.0)
+        np.testing.assert_allclose(got[r], ref[r], atol=2e-5)
+        assert np.abs(got[r, 0] - P["Vl"][0][edge, 0]).max() > 0.1
+
+
+# -------------------------------------------------------------------------------- sampling
+def test_argmax_reference_vector(ops):
+    # tests/test_kernels.cu:96-109
+    rng = np.random.default_rng(16)
+    R, V = 3, 32000
+    logits = rng.normal(size=(R, V)).astype(np.float32)
+    logits[0, 31999] = 50
+    logits[1, 7] = 50
+    logits[1, 9] = 50
+    logits[2, 12345] = 50
+    out = torch.zeros(R, dtype=torch.int32, device=DEV)
+    ops.sample(_t(logits, torch.float32), out)
+    assert out.tolist() == [31999, 7, 12345]
+
+
+def test_temperature_sampling_matches_the_plain_draw(ops):
+    rng = np.random.default_rng(17)
+    R, V = 6, 1000
+    logits = rng.normal(size=(R, V)).astype(np.float32)
+    temps = np.array([0.0, 0.8, 0.8, 1.5, 0.1, 0.8], dtype=np.float32)
+    seeds = np.array([5, 5, 5, 99, 99, 6], dtype=np.int64)
+    reqs = np.array([0, 0, 1, 3, 3, 0], dtype=np.int64)
+    idx = np.array([0, 0, 0, 7, 8, 0], dtype=np.int32)
+    out = torch.zeros(R, dtype=torch.int32, device=DEV)
+    ops.sample(_t(logits, torch.float32), out, _t(temps, torch.float32), _t(seeds, torch.int64), _t(reqs, torch.int64),
+               _t(idx, torch.int32))
+    got = out.tolist()
+    for r in range(R):
+        want, margin = plain.sample_row(logits[r], float(temps[r]), int(seeds[r]), int(reqs[r]), int(idx[r]))
+        assert got[r] == want or (margin is not None and margin < 1e-5)
+    assert got[1] != got[2] or got[1] != got[5]          # request id and seed enter the draw
+
+
+def test_temperature_sampling_follows_softmax(ops):
+    logits = np.log(np.array([[0.1, 0.2, 0.3, 0.4]], dtype=np.float64)).astype(np.float32)
+    N = 4000
+    rows = _t(np.repeat(logits, N, axis=0), torch.float32)
+    out = torch.zeros(N, dtype=torch.int32, device=DEV)
+    ops.sample(rows, out, torch.full((N,), 1.0, device=DEV), torch.arange(N, device=DEV, dtype=torch.int64),
+               torch.zeros(N, dtype=torch.int64, device=DEV), torch.zeros(N, dtype=torch.int32, device=DEV))
+    freq = np.bincount(out.cpu().numpy(), minlength=4) / N
+    np.testing.assert_allclose(freq, [0.1, 0.2, 0.3, 0.4], atol=0.03)
