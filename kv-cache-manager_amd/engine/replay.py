@@ -1,0 +1,119 @@
+"""Trace replay: given token ids are fed through the model step by step and logits are written
+out.  Nothing is sampled.  It drives the same model, step function, cache manager and kernels
+that generation uses.  The nearest thing in the reference is Engine::score, which scores one
+whole sequence in one step through the real manager (src/engine/engine.cpp:92-108).
+
+A step is a JSON object  {"step": k, "entries": [{"id": .., "tokens": [..], "want": [..]}], "end": [..]}:
+all entries are one batch; a request's tokens continue where its last entry stopped; ``want``
+are places among this entry's tokens whose logits are asked for; ``end`` lists requests whose
+pages are given back after the step.
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+from ..config.engine_config import EngineConfig
+from .build import build_runner
+
+
+class ReplayError(RuntimeError):
+    pass
+
+
+class TraceReplayer:
+    def __init__(self, model_dir, dtype="bfloat16", max_tokens=4096, block_size=16, device="cuda:0",
+                 max_live=8, attn="auto"):
+        pages = (max_tokens + block_size - 1) // block_size
+        span = max(pages * block_size, block_size)
+        ec = EngineConfig(policy="paged", block_size=block_size, max_seq_len=span, num_blocks=max(pages, 1),
+                          watermark_blocks=0, max_num_seqs=max_live, max_batched_tokens=span,
+                          max_logit_rows=min(span, 1024), dtype=dtype, attn=attn, use_graphs=False)
+        self.runner, self.core, self.model, self.model_config = build_runner(model_dir, ec, device=device)
+        self.vocab_size = self.model.spec.vocab_size
+        self._ids = {}          # external id -> integer id
+        self._next = 0
+        self._computed = {}     # integer id -> tokens already run
+
+    def _sid(self, ext, create):
+        key = json.dumps(ext)
+        if key not in self._ids:
+            if not create:
+                raise ReplayError(f"request {ext!r} is not live")
+            self._ids[key] = self._next
+            self._next += 1
+        return self._ids[key]
+
+    def step(self, record):
+        """Runs one step; returns float32 logits [wanted, vocab] or None when nothing is wanted."""
+        entries, seen = [], set()
+        for e in record.get("entries", []):
+            tokens = [int(t) for t in e["tokens"]]
+            want = [int(w) for w in e.get("want", [])]
+            if not tokens:
+                raise ReplayError(f"request {e['id']!r}: an entry needs at least one token")
+            if any(t < 0 or t >= self.vocab_size for t in tokens):
+                raise ReplayError(f"request {e['id']!r}: token id outside the vocabulary of {self.vocab_size}")
+            if any(w < 0 or w >= len(tokens) for w in want):
+                raise ReplayError(f"request {e['id']!r}: a wanted place lies outside its {len(tokens)} tokens")
+            fresh = json.dumps(e["id"]) not in self._ids
+            sid = self._sid(e["id"], create=True)
+            if sid in seen:
+                raise ReplayError(f"request {e['id']!r} appears twice in one step")
+            seen.add(sid)
+            if fresh:
+                self.core.seq_new(sid, tokens)
+                if not self.core.can_admit(sid):
+                    self.core.seq_delete(sid)
+                    del self._ids[json.dumps(e["id"])]
+                    raise ReplayError(f"request {e['id']!r} does not fit the cache pool (--max-tokens is too small)")
+                self.core.admit(sid)
+                self._computed[sid] = 0
+            else:
+                self.core.seq_push_tokens(sid, tokens)
+                if not self.core.append_slot(sid):
+                    raise ReplayError(f"out of cache pages while extending request {e['id']!r} (--max-tokens is too small)")
+            entries.append((sid, self._computed[sid], len(tokens), want))
+        logits = None
+        if entries:
+            layout = self.core.build_batch(entries, self.runner.host_buffer())
+            logits = self.runner.execute_to_host(layout)
+            for sid, start, count, _ in entries:
+                self._computed[sid] = start + count
+                self.core.set_computed(sid, start + count)
+                self.core.commit(sid)
+        for ext in record.get("end", []):
+            sid = self._sid(ext, create=False)
+            self.core.release(sid)
+            self.core.seq_delete(sid)
+            del self._ids[json.dumps(ext)]
+            del self._computed[sid]
+        return logits
+
+
+def main(argv=None):
+    import argparse
+    ap = argparse.ArgumentParser(prog="trace_run", description="replay given token ids step by step and write logits")
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--attn", default="auto", choices=["v1", "v2", "auto"])
+    args = ap.parse_args(argv)
+    os.makedirs(args.out, exist_ok=True)
+    print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
+    rp = TraceReplayer(args.model, args.dtype, args.max_tokens, args.block_size, attn=args.attn)
+    print("[trace_run] ready", file=sys.stderr, flush=True)
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        record = json.loads(line)
+        logits = rp.step(record)
+        if logits is not None:
+            np.ascontiguousarray(logits, dtype="<f4").tofile(os.path.join(args.out, f"{record['step']}.f32"))
+        print(f"done {record['step']}", flush=True)
+    return 0

@@ -1,0 +1,217 @@
+"""The step function: one batch of (request, its next tokens) in, logits at the wanted places out.
+
+``ModelRunner`` owns the model, the device side of the cache, the work buffers and the packed
+metadata buffers.  ``execute`` runs exactly the rows it is given, prompt portions beside single
+decoded tokens, from what earlier steps left in the cache.  The reference's step is
+LlamaModel::forward (src/model/llama.cpp:54-141): one packed upload of integers, the layer loop,
+the head on the wanted rows only.
+"""
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import numpy as np
+import torch
+
+from ..cache.manager import BatchLayout, CacheGroupSpec, HostCore
+from ..cache.storage import KVStorage, StateStorage, bytes_per_block
+from ..parts.base import BuildContext, KVCacheNeed, StateNeed
+from ..parts.model import Model
+
+
+@dataclass
+class ModelLimits:
+    """Largest step the work buffers are made for (src/model/llama.h:35-41, engine.cpp:38-45)."""
+    max_tokens: int
+    max_seqs: int
+    max_logit_rows: int
+    max_blocks_per_seq: int
+    max_context_len: int
+
+
+class Workspace:
+    """Named device buffers with fixed capacity, reused by every step (stable addresses)."""
+
+    def __init__(self, device, default_dtype, limits: ModelLimits):
+        self.device, self.default_dtype, self.limits = device, default_dtype, limits
+        self.buffers: Dict[str, torch.Tensor] = {}
+        self.row_caps = {"head_in": limits.max_logit_rows, "logits": limits.max_logit_rows}
+
+    def get(self, name, shape, dtype=None):
+        dtype = dtype or self.default_dtype
+        rows, cols = shape
+        cap = self.row_caps.get(name, self.limits.max_tokens)
+        if rows > cap:
+            raise RuntimeError(f"step: batch exceeds model limits ({name}: {rows} rows > {cap})")
+        key = (name, cols, dtype)
+        buf = self.buffers.get(key)
+        if buf is None:
+            buf = torch.empty(cap, cols, dtype=dtype, device=self.device)
+            self.buffers[key] = buf
+        return buf[:rows]
+
+    def bytes(self):
+        return sum(b.numel() * b.element_size() for b in self.buffers.values())
+
+
+class StepContext:
+    """What the parts see of one step: where each array of the packed metadata lies on the device
+    and on the host, the work buffers, and the attention entry point."""
+
+    def __init__(self, runner, layout: BatchLayout):
+        self.runner, self.layout = runner, layout
+        L = layout
+        self.rows, self.real_rows = L.rows_padded, L.rows
+        self.seqs, self.real_seqs = L.seqs_padded, L.seqs
+        self.logit_rows_padded, self.logit_rows = L.logit_rows_padded, L.logit_rows
+        self.max_context, self.max_run = L.max_context, L.max_run
+        d, h = runner.meta_dev, runner.meta_host
+        T, S, R = self.rows, self.seqs, self.logit_rows_padded
+        self.tokens = d[L.tokens:L.tokens + T]
+        self.positions = d[L.positions:L.positions + T]
+        self.ctx_lens = d[L.context_lens:L.context_lens + T]
+        self.row_seq = d[L.row_seq:L.row_seq + T]
+        self.run_start = d[L.run_start:L.run_start + S + 1]
+        self.seq_start = d[L.seq_start:L.seq_start + S]
+        self.seq_end = d[L.seq_end:L.seq_end + S]
+        self.logit_row_index = d[L.logit_row_index:L.logit_row_index + R]
+        self.state_slots = d[L.state_slots:L.state_slots + S]
+        # the same arrays on the host, for parts that loop over sequences in Python
+        self.host_positions = h[L.positions:L.positions + T]
+        self.host_run_start = h[L.run_start:L.run_start + S + 1]
+        self.host_seq_start = h[L.seq_start:L.seq_start + S]
+        self.host_seq_end = h[L.seq_end:L.seq_end + S]
+        self.host_state_slots = h[L.state_slots:L.state_slots + S]
+
+    def slots(self, g):
+        L = self.layout
+        return self.runner.meta_dev[L.slots[g]:L.slots[g] + self.rows]
+
+    def tables(self, g):
+        L = self.layout
+        return self.runner.meta_dev[L.tables[g]:L.tables[g] + self.seqs * L.table_stride[g]]
+
+    def table_stride(self, g):
+        return self.layout.table_stride[g]
+
+    def ws(self, name, shape, dtype=None):
+        return self.runner.workspace.get(name, shape, dtype)
+
+    def attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window=0):
+        self.runner.attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window)
+
+
+class ModelRunner:
+    def __init__(self, model: Model, core: HostCore, storages, limits: ModelLimits, dtype, device, attn="auto"):
+        self.model, self.core, self.storages, self.limits = model, core, storages, limits
+        self.dtype, self.device, self.attn = dtype, device, attn
+        self.ops = model.ctx.ops
+        self.workspace = Workspace(device, dtype, limits)
+        G = core.num_groups
+        ints = (4 * limits.max_tokens + 4 * limits.max_seqs + 1 + limits.max_logit_rows
+                + G * (limits.max_tokens + limits.max_seqs * limits.max_blocks_per_seq) + 64)
+        self._pinned = torch.empty(ints, dtype=torch.int32, pin_memory=True)
+        self.meta_host = self._pinned.numpy()
+        self.meta_dev = torch.zeros(ints, dtype=torch.int32, device=device)
+        self.vocab_size = model.spec.vocab_size
+        self._upload_done = torch.cuda.Event()
+        self._upload_pending = False
+        model.attach_caches(storages)
+
+    def host_buffer(self) -> np.ndarray:
+        """The pinned metadata buffer, once the previous step's upload no longer reads it."""
+        if self._upload_pending:
+            self._upload_done.synchronize()
+            self._upload_pending = False
+        return self.meta_host
+
+    # ------------------------------------------------------------------------- attention
+    def attention(self, step, q, out, kcache, vcache, g, nh, nkv, hd, scale, window):
+        self.ops.attention(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
+                           step.ctx_lens, nh, nkv, hd, scale, window, rows=step.rows)
+
+    # ------------------------------------------------------------------------------ steps
+    def _check(self, layout: BatchLayout):
+        lim = self.limits
+        if (layout.rows_padded > lim.max_tokens or layout.seqs_padded > lim.max_seqs
+                or layout.logit_rows_padded > lim.max_logit_rows or layout.max_context > lim.max_context_len
+                or max(layout.table_stride + [0]) > lim.max_blocks_per_seq):
+            raise RuntimeError(
+                f"step: batch exceeds model limits (rows {layout.rows_padded}/{lim.max_tokens}, sequences "
+                f"{layout.seqs_padded}/{lim.max_seqs}, logit rows {layout.logit_rows_padded}/{lim.max_logit_rows}, "
+                f"context {layout.max_context}/{lim.max_context_len})")
+        toks = self.meta_host[layout.tokens:layout.tokens + layout.rows]
+        if layout.rows and (toks.min() < 0 or toks.max() >= self.vocab_size):
+            raise ValueError(f"step: token id outside the vocabulary of {self.vocab_size}")
+
+    def _begin(self, layout: BatchLayout) -> StepContext:
+        self._check(layout)
+        n = layout.total
+        self.meta_dev[:n].copy_(self._pinned[:n], non_blocking=True)
+        self._upload_done.record()
+        self._upload_pending = True
+        return StepContext(self, layout)
+
+    def execute(self, layout: BatchLayout) -> Optional[torch.Tensor]:
+        """Runs the batch whose metadata build_batch left in the host buffer.  Returns the logits
+        [layout.logit_rows, vocab] (a view of a work buffer, valid until the next step), or None
+        when no logits were asked for (the rows still run: their keys must reach the cache)."""
+        if layout.rows == 0:
+            return None
+        if layout.logit_rows_padded > self.limits.max_logit_rows:
+            raise RuntimeError(f"step: {layout.logit_rows_padded} logit rows exceed the limit of "
+                               f"{self.limits.max_logit_rows} (use execute_to_host)")
+        step = self._begin(layout)
+        x, pending = self.model.run_layers(step)
+        if layout.logit_rows_padded == 0:
+            return None
+        return self.model.head_logits(step, x, pending, step.logit_row_index)[:layout.logit_rows]
+
+    def execute_to_host(self, layout: BatchLayout) -> Optional[np.ndarray]:
+        """As ``execute``, for any number of wanted rows: the head runs over them in portions of
+        at most max_logit_rows and the logits are gathered in host memory [logit_rows, vocab]."""
+        if layout.rows == 0:
+            return None
+        step = self._begin(layout)
+        x, pending = self.model.run_layers(step)
+        R = layout.logit_rows
+        if R == 0:
+            torch.cuda.current_stream().synchronize()
+            return None
+        out = np.empty((R, self.vocab_size), dtype=np.float32)
+        cap = self.limits.max_logit_rows
+        for lo in range(0, R, cap):
+            hi = min(R, lo + cap)
+            logits = self.model.head_logits(step, x, pending, step.logit_row_index[lo:hi])
+            out[lo:hi] = logits.cpu().numpy()
+        return out
+
+    def run_entries(self, entries, **pad) -> Optional[torch.Tensor]:
+        """entries: (sequence id, start, count, want) as HostCore.build_batch takes them."""
+        layout = self.core.build_batch(entries, self.host_buffer(), **pad)
+        return self.execute(layout)
+
+
+# --------------------------------------------------------------------------------- building
+def plan_groups(model: Model, num_blocks: int, max_num_seqs: int) -> List[CacheGroupSpec]:
+    groups = []
+    for plan in model.groups:
+        if isinstance(plan.need, KVCacheNeed):
+            groups.append(CacheGroupSpec("window" if plan.need.window > 0 else "full", plan.need.window, num_blocks))
+        else:
+            groups.append(CacheGroupSpec("state", 0, 0))
+    return groups
+
+
+def make_storages(model: Model, num_blocks: int, block_size: int, max_num_seqs: int, dtype, device):
+    out = []
+    for g, plan in enumerate(model.groups):
+        if isinstance(plan.need, KVCacheNeed):
+            out.append(KVStorage(g, plan.need, len(plan.layers), num_blocks, block_size, dtype, device))
+        else:
+            out.append(StateStorage(g, plan.need, len(plan.layers), max_num_seqs, device))
+    return out
+
+
+def kv_bytes_per_block(model: Model, block_size: int, dtype) -> int:
+    return sum(bytes_per_block(p.need, len(p.layers), block_size, dtype)
+               for p in model.groups if isinstance(p.need, KVCacheNeed))

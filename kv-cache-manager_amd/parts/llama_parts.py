@@ -1,0 +1,172 @@
+"""The parts a Llama-style decoder is made of: RMS norm, rotary positions, grouped-query attention
+over the paged cache, SwiGLU feed-forward, token embedding, output head, and the pre-norm residual
+arrangement.  Formulas and rounding points follow the reference step (src/model/llama.cpp:84-128)
+and its kernels (src/cuda/kernels.cu, src/cuda/paged_attention.cu); every size and constant is a
+parameter.
+"""
+import math
+
+import torch
+
+from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS
+from .base import (Block, Embedding, FeedForward, Head, KVCacheNeed, Mixer, Norm, ParamSpec, PositionEncoding)
+
+
+def _linear(ctx, x, w, out):
+    ctx.ops.gemm(x, w, out)
+    return out
+
+
+@NORMS.register("rmsnorm")
+class RMSNorm(Norm):
+    """out = weight * round(x / sqrt(mean(x^2) + eps)); eps inside the root, no mean removed, the
+    weight a plain multiplier (src/cuda/kernels.cu:34-49).  params: size, eps."""
+
+    def param_specs(self):
+        return [ParamSpec("weight", ((self.prefix + "weight", (self.params["size"],)),), role="vector")]
+
+    def forward(self, x, out, add=None, rows=None):
+        self.ctx.ops.rmsnorm(x, self.w["weight"], out, self.params["eps"], add=add, rows=rows)
+        return out
+
+
+@POSITIONS.register("rotary")
+class Rotary(PositionEncoding):
+    """Rotate-half rotary positions over the first ``dim`` (= head_dim) entries of every q and k
+    head: pairs (j, j + dim/2), inv_freq_j = theta^(-2j/dim), angle = position * inv_freq_j in
+    32-bit (src/cuda/kernels.cu:51-70).  params: theta, dim."""
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        dim = params["dim"]
+        j = torch.arange(0, dim, 2, dtype=torch.float32)
+        self.inv_freq = (1.0 / torch.pow(torch.tensor(float(params["theta"]), dtype=torch.float32), j / dim)).to(ctx.device)
+
+    def ignorable_tensors(self):
+        return (self.prefix + "rotary_emb.inv_freq",)
+
+    def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None):
+        if head_dim != self.params["dim"]:
+            raise ValueError("rotary: this kernel rotates the whole head (dim must equal head_dim)")
+        k, v = cache if cache is not None else (None, None)
+        self.ctx.ops.rope_cache(qkv, num_heads, num_kv_heads, head_dim, positions=step.positions,
+                                inv_freq=self.inv_freq, slots=slots, kcache=k, vcache=v,
+                                block_size=self.ctx.block_size, rows=step.rows)
+        return cache is not None
+
+
+@POSITIONS.register("none")
+class NoPosition(PositionEncoding):
+    def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None):
+        return False
+
+
+@MIXERS.register("gqa_attention")
+class GQAAttention(Mixer):
+    """Grouped-query attention over the paged cache.  One fused projection [q | k | v]
+    (src/model/llama.cpp:108), positions applied to q and k, k and v stored to the pages of this
+    step's rows before attention reads them (llama.cpp:111-115), so a portion of a prompt attends
+    to itself through the cache; causality is context length = position + 1.
+    params: num_heads, num_kv_heads, head_dim, scale, window (0 = all keys), position (PartSpec)."""
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        p = params
+        self.nh, self.nkv, self.hd = p["num_heads"], p["num_kv_heads"], p["head_dim"]
+        self.scale = p.get("scale", 1.0 / math.sqrt(self.hd))
+        self.window = p.get("window", 0)
+        pos = p["position"]
+        self.position = POSITIONS.get(pos.kind)(pos.params, prefix, ctx)
+        self.q_dim, self.kv_dim = self.nh * self.hd, self.nkv * self.hd
+
+    def param_specs(self):
+        H, pre = self.ctx.hidden_size, self.prefix
+        return [ParamSpec("wqkv", ((pre + "q_proj.weight", (self.q_dim, H)), (pre + "k_proj.weight", (self.kv_dim, H)),
+                                   (pre + "v_proj.weight", (self.kv_dim, H)))),
+                ParamSpec("wo", ((pre + "o_proj.weight", (H, self.q_dim)),))]
+
+    def ignorable_tensors(self):
+        return self.position.ignorable_tensors()
+
+    def cache_need(self):
+        return KVCacheNeed(self.nkv, self.hd, self.window)
+
+    def forward(self, step, h):
+        ops = self.ctx.ops
+        g = self.cache.group
+        kc, vc = self.cache.k(self.cache_index), self.cache.v(self.cache_index)
+        qkv = step.ws("qkv", (step.rows, self.q_dim + 2 * self.kv_dim))
+        _linear(self.ctx, h, self.w["wqkv"], qkv)
+        slots = step.slots(g) if self.cache_owner else None
+        stored = self.position.apply(step, qkv, self.nh, self.nkv, self.hd,
+                                     cache=(kc, vc) if self.cache_owner else None, slots=slots)
+        if self.cache_owner and not stored:
+            ops.rope_cache(qkv, self.nh, self.nkv, self.hd, slots=slots, kcache=kc, vcache=vc,
+                           block_size=self.ctx.block_size, rows=step.rows)
+        attn = step.ws("attn", (step.rows, self.q_dim))
+        step.attention(qkv, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window)
+        return _linear(self.ctx, attn, self.w["wo"], step.ws("mixer_out", (step.rows, self.ctx.hidden_size)))
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(FeedForward):
+    """down( round(silu(gate(h))) * up(h) ) with gate and up as one fused projection
+    (src/model/llama.cpp:119-122, src/cuda/kernels.cu:72-82).  params: intermediate_size."""
+
+    def param_specs(self):
+        H, I, pre = self.ctx.hidden_size, self.params["intermediate_size"], self.prefix
+        return [ParamSpec("w_gate_up", ((pre + "gate_proj.weight", (I, H)), (pre + "up_proj.weight", (I, H)))),
+                ParamSpec("w_down", ((pre + "down_proj.weight", (H, I)),))]
+
+    def forward(self, step, h):
+        I = self.params["intermediate_size"]
+        gu = _linear(self.ctx, h, self.w["w_gate_up"], step.ws("gate_up", (step.rows, 2 * I)))
+        act = step.ws("act", (step.rows, I))
+        self.ctx.ops.swiglu(gu, act)
+        return _linear(self.ctx, act, self.w["w_down"], step.ws("ffn_out", (step.rows, self.ctx.hidden_size)))
+
+
+@EMBEDDINGS.register("token_embedding")
+class TokenEmbedding(Embedding):
+    """x = float(table[token]); nothing scaled or added (src/cuda/kernels.cu:27-32).
+    params: vocab_size."""
+
+    def param_specs(self):
+        return [ParamSpec("table", ((self.prefix + "weight", (self.params["vocab_size"], self.ctx.hidden_size)),),
+                          role="table")]
+
+    def forward(self, step, out):
+        self.ctx.ops.embed(step.tokens, self.w["table"], out)
+        return out
+
+
+@HEADS.register("linear_head")
+class LinearHead(Head):
+    """logits = h @ table^T in 32-bit, only for the rows that are asked for
+    (src/model/llama.cpp:126-128).  params: vocab_size, tied (use the embedding's table)."""
+
+    def param_specs(self):
+        if self.params.get("tied"):
+            return []
+        return [ParamSpec("table", ((self.prefix + "weight", (self.params["vocab_size"], self.ctx.hidden_size)),),
+                          role="table")]
+
+    def ignorable_tensors(self):
+        # a tied checkpoint may still carry a copy of the shared table
+        return (self.prefix + "weight",) if self.params.get("tied") else ()
+
+    def forward(self, step, h, out):
+        return _linear(self.ctx, h, self.w["table"], out)
+
+
+@BLOCKS.register("prenorm_residual")
+class PreNormResidual(Block):
+    """x += mixer(norm_mixer(x)); x += ffn(norm_ffn(x))  (src/model/llama.cpp:104-124).  Each
+    addition is done by the norm that follows it."""
+
+    def forward(self, step, x, pending):
+        h = step.ws("normed", (step.rows, x.shape[1]))
+        self.parts["norm_mixer"].forward(x, h, add=pending)
+        a = self.parts["mixer"].forward(step, h)
+        self.parts["norm_ffn"].forward(x, h, add=a)
+        return self.parts["ffn"].forward(step, h)
