@@ -1,0 +1,159 @@
+"""Decode and prefill throughput of the engine at TinyLlama-1.1B sizes with random weights.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512] [--layers L]
+
+A "step" is one decode step of the whole engine (schedule, batch metadata, upload, model step on
+the GPU, sampling, download, update).  W untimed steps, then exactly K timed steps between two
+device synchronisations.  One JSON line is printed: decoded tokens a second at the default batch,
+the same at batch 1 and 64, a 2,048-token prefill, and the decode step's memory roofline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+
+# BASELINE.json configs[2]: TinyLlama-1.1B sizes
+SIZES = dict(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_hidden_layers=22,
+             num_attention_heads=32, num_key_value_heads=4, head_dim=64, max_position_embeddings=2048,
+             rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+
+
+def build_engine(cfg, dtype, max_num_seqs, max_batched_tokens, tensors):
+    from kvcm_amd.config.engine_config import EngineConfig
+    from kvcm_amd.engine.engine import Engine
+    ec = EngineConfig(block_size=16, max_seq_len=2048, num_blocks=max_num_seqs * 2048 // 16,
+                      max_num_seqs=max_num_seqs, max_batched_tokens=max_batched_tokens, dtype=dtype,
+                      max_logit_rows=max(max_num_seqs, 64))
+    return Engine(config=ec, architecture="LlamaForCausalLM", model_config=cfg, tensors=tensors)
+
+
+def decode_run(eng, batch, prompt_len, steps, warmup, vocab, seed=1):
+    """-> (seconds for `steps` decode steps, mean context length during them)."""
+    import numpy as np
+    import torch
+    rng = np.random.default_rng(seed)
+    for _ in range(batch):
+        eng.add_request(rng.integers(3, vocab, size=prompt_len).tolist(), max_new_tokens=warmup + steps + 24)
+    extra = 0
+    while True:                                 # prompts, whole, as many per step as the budget takes
+        info = eng.step()
+        if info.prefill_tokens == 0 and eng.core.num_waiting() == 0:
+            break
+        extra += 1
+    for _ in range(warmup):
+        eng.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        info = eng.step()
+        assert info.decode_seqs == batch and info.prefill_tokens == 0, "a timed step was not a pure decode step"
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx = prompt_len + 2 + extra / 2.0 + warmup + (steps - 1) / 2.0
+    # drain
+    while not eng.idle():
+        eng.step()
+    eng.take_finished()
+    return dt, ctx
+
+
+def prefill_run(eng, tokens, vocab, reps=3):
+    import numpy as np
+    import torch
+    rng = np.random.default_rng(7)
+    times = []
+    for r in range(reps + 1):
+        eng.add_request(rng.integers(3, vocab, size=tokens).tolist(), max_new_tokens=1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        info = eng.step()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        assert info.prefill_tokens == tokens
+        eng.take_finished()
+    return sorted(times[1:])[len(times[1:]) // 2]     # median, first one is warm-up
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this engine runs on one GPU; --gpus N with N > 1 is not supported")
+        sys.exit(2)
+
+    import torch
+    from kvcm_amd.config.model_config import LlamaConfig
+    from kvcm_amd.weights.random_init import random_tensors
+
+    sizes = dict(SIZES)
+    full_layers = sizes["num_hidden_layers"]
+    if args.layers:
+        sizes["num_hidden_layers"] = args.layers
+    cfg = LlamaConfig.from_dict(sizes)
+    dt = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    tensors = random_tensors("LlamaForCausalLM", cfg, seed=0, dtype=dt, device="cuda:0")
+    esize = 2 if args.dtype == "bfloat16" else 4
+    key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    layer_params = cfg.qkv_dim * H + H * cfg.q_dim + 3 * I * H + 2 * H
+    kv_bytes_per_token = 2 * L * cfg.kv_dim * esize
+
+    def roofline(batch, seconds_per_step, ctx):
+        weights = (L * layer_params + H + V * H + batch * H) * esize
+        cache = batch * ctx * kv_bytes_per_token
+        achieved = (weights + cache) / seconds_per_step / 1e9
+        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_GBS, 4)}
+
+    eng = build_engine(cfg, args.dtype, max_num_seqs=64, max_batched_tokens=4096, tensors=tensors)
+    del tensors
+    torch.cuda.empty_cache()
+
+    seconds, ctx = decode_run(eng, args.batch, args.prompt_len, args.steps, args.warmup, V)
+    value = args.batch * args.steps / seconds
+    out = {
+        "metric": "decode tok/s at batch 8 (TinyLlama-1.1B sizes, 512-token prompts)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(1e3 * seconds / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": key, "data": "synthetic",
+        "config": {"model": "TinyLlama-1.1B sizes, random weights N(0,0.02)", "global_batch": args.batch,
+                   "seq_len": args.prompt_len, "parallelism": "single GPU", "layers": L, "layers_full": full_layers,
+                   "hidden": H, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate": I, "vocab": V, "kv_block": 16,
+                   "context_limit": 2048, "generated": args.warmup + args.steps},
+        "roofline": roofline(args.batch, seconds / args.steps, ctx),
+    }
+    if not args.no_points:
+        points = {}
+        for b, k in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
+            s, c = decode_run(eng, b, args.prompt_len, k, min(args.warmup, 8), V, seed=10 + b)
+            points[f"decode_b{b}"] = round(b * k / s, 1)
+            points[f"decode_b{b}_ms"] = round(1e3 * s / k, 4)
+            points[f"decode_b{b}_hbm_frac"] = roofline(b, s / k, c)["frac"]
+        out["points"] = points
+        T = 2048
+        sec = prefill_run(eng, T, V)
+        flops = 2.0 * T * (L * (layer_params - 2 * H)) + 2.0 * V * H + L * 4.0 * (T * (T + 1) / 2) * cfg.head_dim * cfg.num_attention_heads
+        out["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
+                          "frac": round(flops / sec / PEAK_FLOPS[key], 4)}
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
