@@ -1,0 +1,332 @@
+"""The engine as a user meets it: generation through the entry point (greedy and with a
+temperature), the scheduler under page pressure with real logits, prefix caching, paged against
+contiguous, graphs against eager steps, and each part of a layer on its own."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_llama as plain
+
+pytestmark = pytest.mark.gpu
+
+
+def _engine(d, **kw):
+    from kvcm_amd import Engine, EngineConfig
+    base = dict(block_size=16, num_blocks=64, max_seq_len=256, max_num_seqs=8, max_batched_tokens=256, dtype="float32")
+    base.update(kw)
+    return Engine(d, EngineConfig(**base))
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name in ("A", "B"):
+        for dtype in ("float32", "bfloat16"):
+            d = str(tmp_path_factory.mktemp(f"gen_{name}_{dtype}"))
+            H.make_model_dir(d, H.CONFIGS[name], H.WEIGHT_SEED[name], torch.float32 if dtype == "float32" else torch.bfloat16)
+            out[(name, dtype)] = (d, plain.load_model_dir(d, plain.round_bf16 if dtype == "bfloat16" else None))
+    return out
+
+
+def _prompts(raw, lengths, seed):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, raw["vocab_size"], size=n).tolist() for n in lengths]
+
+
+def _same_up_to_near_ties(got, want, margins, tie):
+    """Token lists agree; the first difference, if any, sits where the plain model's two best
+    scores are closer than ``tie`` (after it the continuations legitimately differ)."""
+    for k, (g, w) in enumerate(zip(got, want)):
+        if g != w:
+            return margins[k] < tie
+    return len(got) == len(want)
+
+
+# ------------------------------------------------------------------------------ generation
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_config_a(models, dtype):
+    """Tiny A: three requests with prompts of 7, 13 and 5 ids, 8 greedy tokens each."""
+    d, pm = models[("A", dtype)]
+    prompts = _prompts(H.TINY_A, [7, 13, 5], seed=1)
+    eng = _engine(d, dtype=dtype)
+    got = eng.generate(prompts, max_new_tokens=8)
+    for p, g in zip(prompts, got):
+        want, margins = pm.generate(p, 8)
+        assert _same_up_to_near_ties(g, want, margins, 1e-4 if dtype == "float32" else 5e-2), (g, want, margins)
+    assert eng.core.blocks_in_use() == 0 and eng.idle()
+    solo = [_engine(d, dtype=dtype, use_graphs=False).generate([p], 8)[0] for p in prompts]
+    assert solo == got, "a request's tokens changed with the batch it ran in"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_temperature_generation_config_b_chunked(models, dtype):
+    """Tiny B: prompts of 1, 9, 17, 33 and 40 ids, prefill in portions of 16 mixed with decodes,
+    12 tokens each at temperature 0.8 under a fixed sampler seed."""
+    d, pm = models[("B", dtype)]
+    prompts = _prompts(H.TINY_B, [1, 9, 17, 33, 40], seed=3)
+    eng = _engine(d, dtype=dtype, block_size=8, num_blocks=40, prefill_chunk=16, max_batched_tokens=24)
+    ids = [eng.add_request(p, 12, temperature=0.8, seed=1234) for p in prompts]
+    mixed = 0
+    done = {}
+    while not eng.idle():
+        plan_before = eng.core.num_running()
+        info = eng.step()
+        mixed += info.prefill_tokens > 0 and info.decode_seqs > 0
+        for f in eng.take_finished():
+            done[f.id] = f.generated
+    assert mixed > 0, "no step mixed a prompt portion with decoded tokens"
+    for rid, p in zip(ids, prompts):
+        want, margins = pm.generate(p, 12, temperature=0.8, seed=1234, request_id=rid)
+        assert _same_up_to_near_ties(done[rid], want, margins, 1e-4 if dtype == "float32" else 5e-2), (done[rid], want)
+    # the same requests, whole prompts, other batch order: the draw depends on (seed, request, index) only
+    eng2 = _engine(d, dtype=dtype, block_size=8, num_blocks=40)
+    for rid, p in reversed(list(zip(ids, prompts))):
+        eng2.add_request(p, 12, temperature=0.8, seed=1234, request_id=rid)
+    again = {f.id: f.generated for f in eng2.run_until_idle()}
+    if dtype == "float32":
+        assert again == done
+
+
+def test_preemption_recomputes_and_gives_the_same_tokens(models):
+    d, pm = models[("A", "float32")]
+    prompts = _prompts(H.TINY_A, [20, 25, 18, 30, 22, 19], seed=5)
+    roomy = _engine(d, num_blocks=64).generate(prompts, 24)
+    tight = _engine(d, num_blocks=9, watermark_blocks=0)       # 144 slots for 6 x (about 45) tokens
+    got = tight.generate(prompts, 24)
+    assert tight.core.counters()["preemptions"] > 0
+    assert got == roomy
+    assert tight.core.blocks_in_use() == 0
+
+
+def test_impossible_request_is_rejected_and_the_rest_served(models):
+    d, pm = models[("A", "float32")]
+    eng = _engine(d, num_blocks=4)
+    prompts = _prompts(H.TINY_A, [100, 10], seed=6)
+    out = eng.generate(prompts, 4)
+    assert out[0] == [] and len(out[1]) == 4 and eng.core.counters()["rejected"] == 1
+
+
+def test_paged_equals_contiguous_and_prefix_cache_changes_nothing(models):
+    d, pm = models[("B", "float32")]
+    rng = np.random.default_rng(7)
+    shared = rng.integers(0, 384, size=40).tolist()
+    prompts = [shared + rng.integers(0, 384, size=n).tolist() for n in (5, 9, 3)]
+    base = [_engine(d, block_size=8, num_blocks=64).generate([p], 10)[0] for p in prompts]
+    contiguous = _engine(d, block_size=8, num_blocks=128, policy="contiguous", max_seq_len=128)
+    assert [contiguous.generate([p], 10)[0] for p in prompts] == base
+    cached = _engine(d, block_size=8, num_blocks=64, prefix_caching=True)
+    got = [cached.generate([p], 10)[0] for p in prompts]
+    st = cached.core.prefix_stats()
+    assert st["hit_blocks"] >= 2 * 5 and cached.core.counters()["prefill_tokens_saved"] >= 80
+    assert got == base
+    assert cached.generate([prompts[0]], 10)[0] == base[0]        # a full re-run hits its own pages
+    with pytest.raises(RuntimeError, match="prefix caching"):
+        cached.score(prompts[0])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_score_gives_teacher_forced_logits(models, dtype):
+    d, pm = models[("A", dtype)]
+    toks = _prompts(H.TINY_A, [90], seed=8)[0]
+    eng = _engine(d, dtype=dtype)
+    got = eng.score(toks)
+    ref = pm.logits(toks)
+    tol = (1e-5 if dtype == "float32" else 1e-2) * max(1.0, np.abs(ref).max())
+    assert np.abs(got - ref).max() <= tol
+    assert eng.core.blocks_in_use() == 0
+
+
+def test_limits_and_bad_tokens_are_refused(models):
+    d, _ = models[("A", "float32")]
+    eng = _engine(d)
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([1, 2, 256], 4)
+    with pytest.raises(ValueError, match="at least one token"):
+        eng.add_request([], 4)
+    small = _engine(d, max_batched_tokens=16, max_num_seqs=2, max_seq_len=64)
+    with pytest.raises(RuntimeError, match="exceeds model limits"):
+        small.runner.run_entries([])  # nothing to run is fine ...
+        small.core.seq_new(99, list(range(100)))
+        small.core.admit(99)
+        small.runner.run_entries([(99, 0, 100, None)])            # ... more rows than the buffers hold is not
+
+
+# ---------------------------------------------------------------------------------- graphs
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(models, dtype):
+    """Decode steps replayed from a captured graph, several times with eager work and
+    synchronisations in between, give the tokens of eager decoding."""
+    d, pm = models[("A", dtype)]
+    prompts = _prompts(H.TINY_A, [9, 30, 4, 17, 12], seed=9)
+    eager = _engine(d, dtype=dtype, use_graphs=False).generate(prompts, 20)
+    eng = _engine(d, dtype=dtype, use_graphs=True)
+    ids = [eng.add_request(p, 20) for p in prompts[:3]]
+    done = {}
+    step = 0
+    while not eng.idle():
+        eng.step()
+        step += 1
+        if step == 4:                                             # eager work between replays: new prompts arrive
+            ids += [eng.add_request(p, 20) for p in prompts[3:]]
+        if step % 5 == 0:
+            eng.score(prompts[1])                                 # an eager step through the same buffers
+            torch.cuda.synchronize()
+        for f in eng.take_finished():
+            done[f.id] = f.generated
+    assert eng.decode_graphs.graphs, "no graph was captured"
+    assert [done[i] for i in ids] == eager
+
+
+# -------------------------------------------------------------------------- parts, alone
+def _ctx(dtype, hidden):
+    from kvcm_amd import ops
+    from kvcm_amd.parts.base import BuildContext
+    return BuildContext(dtype, torch.device("cuda:0"), hidden, 8, ops)
+
+
+class _Step:
+    """The little of a step that a part needs when it is run on its own."""
+
+    def __init__(self, rows, positions=None):
+        self.rows = rows
+        self.positions = None if positions is None else torch.tensor(positions, dtype=torch.int32, device="cuda:0")
+        self.tokens = None
+        self._bufs = {}
+
+    def ws(self, name, shape, dtype=None):
+        key = (name, tuple(shape), dtype)
+        if key not in self._bufs:
+            self._bufs[key] = torch.zeros(*shape, dtype=dtype or self.default, device="cuda:0")
+        return self._bufs[key]
+
+
+def _dev(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a), dtype=dtype, device="cuda:0")
+
+
+def test_part_rmsnorm_alone():
+    from kvcm_amd.registry import NORMS
+    rng = np.random.default_rng(20)
+    H_, T = 200, 5
+    part = NORMS.get("rmsnorm")({"size": H_, "eps": 3e-6}, "n.", _ctx(torch.float32, H_))
+    w = rng.normal(size=H_)
+    part.bind({"weight": _dev(w)})
+    x = rng.normal(size=(T, H_)).astype(np.float32)
+    out = torch.zeros(T, H_, device="cuda:0")
+    part.forward(_dev(x), out)
+    np.testing.assert_allclose(out.cpu().numpy(), plain.rms_norm(x, w, 3e-6), rtol=3e-6, atol=1e-6)
+    assert [s.sources[0][0] for s in part.param_specs()] == ["n.weight"]
+
+
+def test_part_rotary_alone():
+    from kvcm_amd.registry import POSITIONS
+    rng = np.random.default_rng(21)
+    nh, nkv, hd, T = 3, 1, 24, 4
+    part = POSITIONS.get("rotary")({"theta": 77777.0, "dim": hd}, "", _ctx(torch.float32, 64))
+    qkv = rng.normal(size=(T, (nh + 2 * nkv) * hd)).astype(np.float32)
+    pos = [0, 3, 50, 51]
+    t = _dev(qkv)
+    step = _Step(T, pos)
+    assert part.apply(step, t, nh, nkv, hd) is False              # nothing stored without a cache
+    got = t.cpu().numpy().reshape(T, nh + 2 * nkv, hd)
+    ref = plain.rotary(qkv.reshape(T, nh + 2 * nkv, hd)[:, :nh + nkv], pos, 77777.0)
+    np.testing.assert_allclose(got[:, :nh + nkv], ref, atol=2e-6)
+    np.testing.assert_array_equal(got[:, nh + nkv:], qkv.reshape(T, -1, hd)[:, nh + nkv:])
+
+
+def test_part_swiglu_alone():
+    from kvcm_amd.registry import FEED_FORWARDS
+    rng = np.random.default_rng(22)
+    H_, I, T = 40, 72, 6
+    part = FEED_FORWARDS.get("swiglu")({"intermediate_size": I}, "mlp.", _ctx(torch.float32, H_))
+    wg, wu, wd = rng.normal(size=(I, H_)), rng.normal(size=(I, H_)), rng.normal(size=(H_, I))
+    part.bind({"w_gate_up": _dev(np.concatenate([wg, wu])), "w_down": _dev(wd)})
+    h = rng.normal(size=(T, H_)).astype(np.float32) * 0.3
+    step = _Step(T)
+    step.default = torch.float32
+    out = part.forward(step, _dev(h))
+    gu = np.concatenate([plain.linear(h, wg), plain.linear(h, wu)], axis=-1)
+    np.testing.assert_allclose(out.cpu().numpy(), plain.linear(plain.swiglu(gu), wd), rtol=1e-4, atol=1e-4)
+    names = [n for s in part.param_specs() for n, _ in s.sources]
+    assert names == ["mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight"]
+
+
+def test_part_attention_mixer_alone_through_the_cache():
+    """The mixer on its own: one expert of everything else is the identity.  A prompt portion,
+    then single tokens, against plain attention over the whole sequence."""
+    from kvcm_amd.cache.storage import KVStorage
+    from kvcm_amd.parts.base import KVCacheNeed, PartSpec
+    from kvcm_amd.registry import MIXERS
+    rng = np.random.default_rng(23)
+    Hh, nh, nkv, hd, B, n = 48, 4, 2, 16, 8, 21
+    ctx = _ctx(torch.float32, Hh)
+    part = MIXERS.get("gqa_attention")({"num_heads": nh, "num_kv_heads": nkv, "head_dim": hd, "scale": 0.3, "window": 0,
+                                       "position": PartSpec("rotary", {"theta": 1e4, "dim": hd})}, "a.", ctx)
+    wq, wk, wv, wo = (rng.normal(size=s) * 0.3 for s in ((nh * hd, Hh), (nkv * hd, Hh), (nkv * hd, Hh), (Hh, nh * hd)))
+    part.bind({"wqkv": _dev(np.concatenate([wq, wk, wv])), "wo": _dev(wo)})
+    assert part.cache_need() == KVCacheNeed(nkv, hd, 0)
+    store = KVStorage(0, part.cache_need(), 1, 6, B, torch.float32, "cuda:0")
+    part.attach_cache(store, 0)
+    h = rng.normal(size=(n, Hh)).astype(np.float32)
+    table = [4, 1, 5]                                             # scattered pages
+
+    class Step(_Step):
+        default = torch.float32
+
+        def __init__(self, lo, hi):
+            super().__init__(hi - lo, list(range(lo, hi)))
+            self.lo, self.hi = lo, hi
+
+        def slots(self, g):
+            return _dev([table[p // B] * B + p % B for p in range(self.lo, self.hi)], torch.int32)
+
+        def attention(self, q, out, kc, vc, g, nh_, nkv_, hd_, scale, window=0):
+            ctx.ops.attention(q, out, kc, vc, _dev(table, torch.int32), 3, _dev([0] * self.rows, torch.int32),
+                              _dev([p + 1 for p in range(self.lo, self.hi)], torch.int32), nh_, nkv_, hd_, scale, window)
+
+    outs = []
+    for lo, hi in [(0, 13), (13, 14), (14, 19), (19, 20), (20, 21)]:
+        outs.append(part.forward(Step(lo, hi), _dev(h[lo:hi])).cpu().numpy().copy())
+    got = np.concatenate(outs)
+    pos = np.arange(n)
+    q = plain.rotary(plain.linear(h, wq).reshape(n, nh, hd), pos, 1e4)
+    k = plain.rotary(plain.linear(h, wk).reshape(n, nkv, hd), pos, 1e4)
+    v = plain.linear(h, wv).reshape(n, nkv, hd)
+    ref = plain.linear(plain.attention(q, k, v, pos, pos, 0.3).reshape(n, nh * hd), wo)
+    np.testing.assert_allclose(got, ref, atol=2e-4, rtol=1e-4)
+
+
+def test_block_arrangement_alone():
+    """pre-norm residual with stand-in parts: x + mixer(norm(x)) then + ffn(norm(.)), the last
+    addition left pending."""
+    from kvcm_amd.registry import BLOCKS
+    from kvcm_amd.parts.base import FeedForward, Mixer, Norm
+
+    class Twice(Norm):
+        def forward(self, x, out, add=None, rows=None):
+            if add is not None:
+                x += add
+            out.copy_(2 * x)
+            return out
+
+    class PlusOne(Mixer):
+        def forward(self, step, h):
+            return h + 1
+
+    class Negate(FeedForward):
+        def forward(self, step, h):
+            return -h
+
+    ctx = _ctx(torch.float32, 4)
+    block = BLOCKS.get("prenorm_residual")({"norm_mixer": Twice({}, "", ctx), "mixer": PlusOne({}, "", ctx),
+                                            "norm_ffn": Twice({}, "", ctx), "ffn": Negate({}, "", ctx)})
+    step = _Step(2)
+    step.default = torch.float32
+    x = torch.ones(2, 4, device="cuda:0")
+    pending = block.forward(step, x, torch.full((2, 4), 0.5, device="cuda:0"))
+    # x = 1 + 0.5 = 1.5; mixer(2x) = 4; x = 5.5; ffn(2x) = -11 pending
+    assert torch.equal(x, torch.full((2, 4), 5.5, device="cuda:0"))
+    assert torch.equal(pending, torch.full((2, 4), -11.0, device="cuda:0"))
