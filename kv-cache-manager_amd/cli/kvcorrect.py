@@ -1,0 +1,190 @@
+"""kvcorrect: end-to-end correctness gate.
+
+The reference's kvcorrect compares against outputs of another framework computed with real
+weights (src/main_correct.cpp:1-9).  Here the yardstick is the engine's own 32-bit path of the
+same model (every kernel in true float32), which the test suite in turn pins to a plain
+implementation.  With --refs FILE the reference's KVPR file format is read instead
+(main_correct.cpp:34-59).  Checks, as in the reference:
+  1. greedy output of each prompt alone equals the yardstick's; a divergence is tolerated only
+     where the yardstick's two best logits are closer than --tie-margin;
+  2. teacher-forced top-1 agreement >= 98 %, top-5 logit error reported;
+  3. paged and contiguous policies give identical tokens (scattered physical pages);
+  4. all prompts in one batch give the tokens of the solo runs;
+  5. prefix caching on: hits happen and outputs stay identical.
+Exit code 0 all pass, 2 some fail, 1 error.
+"""
+import struct
+import sys
+
+import numpy as np
+
+from .args import Args
+from .common import engine_config_from_args, make_engine
+
+
+def load_refs(path):
+    with open(path, "rb") as f:
+        magic, n, steps, topk = struct.unpack("<4s3i", f.read(16))
+        if magic != b"KVPR":
+            raise ValueError("bad refs magic")
+        out = []
+        for _ in range(n):
+            (ln,) = struct.unpack("<i", f.read(4))
+            prompt = np.frombuffer(f.read(4 * ln), dtype="<i4").tolist()
+            greedy = np.frombuffer(f.read(4 * steps), dtype="<i4").tolist()
+            top_ids = np.frombuffer(f.read(4 * steps * topk), dtype="<i4").reshape(steps, topk)
+            top_logits = np.frombuffer(f.read(4 * steps * topk), dtype="<f4").reshape(steps, topk)
+            out.append(dict(prompt=prompt, greedy=greedy, top_ids=top_ids, top_logits=top_logits))
+    return out, steps, topk
+
+
+def synthetic_prompts(vocab, n=8, shared=48, seed=11):
+    """Prompts that share a leading run of tokens (like a system prompt) and then differ."""
+    rng = np.random.default_rng(seed)
+    head = rng.integers(3, vocab, size=shared).tolist()
+    return [head + rng.integers(3, vocab, size=int(k)).tolist() for k in rng.integers(5, 40, size=n)]
+
+
+def yardstick(a, base_ec, prompts, steps, topk=5):
+    """Greedy continuations and per-step top-k logits from the 32-bit path."""
+    ec = type(base_ec)(**{**base_ec.__dict__, "dtype": "float32", "policy": "paged", "prefix_caching": False,
+                          "use_graphs": False})
+    eng = make_engine(a, ec)
+    refs = []
+    for p in prompts:
+        out = eng.generate([p], steps)[0]
+        logits = eng.score(p + out[:-1])[len(p) - 1:]
+        top = np.argsort(-logits, axis=1, kind="stable")[:, :topk]
+        refs.append(dict(prompt=p, greedy=out, top_ids=top, top_logits=np.take_along_axis(logits, top, axis=1)))
+    del eng
+    return refs
+
+
+def fragment_pool(core, n=200):
+    """Admits dummy sequences and releases every other one, so that real requests get scattered,
+    non-consecutive page tables (src/main_correct.cpp:100-116).  Returns the ids still held."""
+    made = []
+    for i in range(n):
+        sid = -1000 - i
+        core.seq_new(sid, [7] * (1 + (i * 37) % 50))
+        if not core.can_admit(sid):
+            core.seq_delete(sid)
+            break
+        core.admit(sid)
+        made.append(sid)
+    held = []
+    for k, sid in enumerate(made):
+        if k % 2:
+            core.release(sid)
+            core.seq_delete(sid)
+        else:
+            held.append(sid)
+    return held
+
+
+def first_mismatch(ref, got, steps, tie_margin):
+    for k in range(steps):
+        if k >= len(got) or got[k] != ref["greedy"][k]:
+            margin = float(ref["top_logits"][k][0] - ref["top_logits"][k][1])
+            return k, margin, margin < tie_margin
+    return -1, 0.0, True
+
+
+def main(argv=None):
+    try:
+        a = Args(sys.argv[1:] if argv is None else argv)
+        tie_margin = a.f64("tie-margin", 0.5)
+        steps = a.i32("steps", 0)
+        refs_path = a.str("refs", "")
+        base = engine_config_from_args(a, max_seq_len=a.i32("max-seq-len", 512), pool_gb=a.f64("pool-gb", 0.25),
+                                       max_num_seqs=a.i32("max-num-seqs", 16), max_batched_tokens=a.i32("max-batched-tokens", 2048))
+        ok_all = True
+
+        def check(cond, what):
+            nonlocal ok_all
+            print(f"{'[PASS]' if cond else '[FAIL]'}  {what}")
+            ok_all &= bool(cond)
+
+        mk = lambda **kw: make_engine(a, type(base)(**{**base.__dict__, **kw}))
+        probe = mk(policy="paged", prefix_caching=False)
+        vocab = probe.model.spec.vocab_size
+        if refs_path:
+            refs, ref_steps, topk = load_refs(refs_path)
+            steps = ref_steps if steps <= 0 or steps > ref_steps else steps
+        else:
+            steps = steps if steps > 0 else 32
+            topk = 5
+            refs = yardstick(a, base, synthetic_prompts(vocab), steps, topk)
+        a.warn_unused()
+        N = len(refs)
+        print(f"{N} reference prompts, {steps} steps, top-{topk}")
+
+        solo = {}
+        for policy in ("paged", "contiguous"):
+            eng = probe if policy == "paged" else mk(policy="contiguous", prefix_caching=False)
+            held = fragment_pool(eng.core) if policy == "paged" else []
+            print(f"\n== {policy}: each prompt alone ({'scattered' if policy == 'paged' else 'consecutive'} pages)")
+            ok, exact, outs = True, 0, []
+            for i, r in enumerate(refs):
+                out = eng.generate([r["prompt"]], steps)[0]
+                k, margin, fine = first_mismatch(r, out, steps, tie_margin)
+                exact += k < 0
+                if k >= 0:
+                    print(f"  prompt {i} ({len(r['prompt'])} tok): first divergence at step {k} (margin {margin:.3f}) -> "
+                          f"{'near-tie, tolerated' if fine else 'REAL MISMATCH'}")
+                ok &= fine
+                outs.append(out)
+            print(f"  {exact}/{N} prompts exact over {steps} steps")
+            check(ok, f"{policy}: greedy matches the reference (alone)")
+            solo[policy] = outs
+            if policy == "paged":
+                print("\n== paged: teacher-forced logits")
+                agree = total = 0
+                errs = []
+                for r in refs:
+                    toks = r["prompt"] + r["greedy"][:steps - 1]
+                    logits = eng.score(toks)
+                    for k in range(steps):
+                        row = logits[len(r["prompt"]) - 1 + k]
+                        agree += int(np.argmax(row)) == int(r["top_ids"][k][0])
+                        total += 1
+                        errs.extend(np.abs(row[r["top_ids"][k]] - r["top_logits"][k]).tolist())
+                print(f"  top-1 agreement {agree}/{total} ({100.0 * agree / total:.2f}%), top-{topk} logit |err| "
+                      f"mean {np.mean(errs):.4f} max {np.max(errs):.4f}")
+                check(agree >= 0.98 * total, "teacher-forced top-1 agreement >= 98%")
+                print(f"\n== paged: all {N} prompts in one batch")
+                outs = eng.generate([r["prompt"] for r in refs], steps)
+                same = sum(o == s for o, s in zip(outs, solo["paged"]))
+                bok = all(first_mismatch(r, o, steps, tie_margin)[2] for r, o in zip(refs, outs))
+                print(f"  {same}/{N} batched outputs identical to solo runs")
+                check(bok, "batched greedy matches the reference (no cross-contamination)")
+                for sid in held:
+                    eng.core.release(sid)
+                    eng.core.seq_delete(sid)
+        print("\n== paged vs contiguous")
+        same = sum(x == y for x, y in zip(solo["paged"], solo["contiguous"]))
+        print(f"  {same}/{N} prompts identical")
+        check(same == N, "paged and contiguous produce identical tokens")
+
+        print("\n== paged + prefix caching (shared leading tokens)")
+        eng = mk(policy="paged", prefix_caching=True)
+        outs = [eng.generate([r["prompt"]], steps)[0] for r in refs]
+        again = eng.generate([refs[0]["prompt"]], steps)[0]
+        st, c = eng.core.prefix_stats(), eng.core.counters()
+        print(f"  block hits {st['hit_blocks']} / {st['queried_blocks']} queried, prefill tokens computed "
+              f"{c['prefill_tokens']}, saved {c['prefill_tokens_saved']}")
+        same = sum(o == s for o, s in zip(outs, solo["paged"]))
+        print(f"  {same}/{N} outputs identical to prefix-off runs; re-run of prompt 0 "
+              f"{'identical' if again == solo['paged'][0] else 'differs'}")
+        check(st["hit_blocks"] > 0 and c["prefill_tokens_saved"] > 0, "prefix cache produces hits")
+        check(all(first_mismatch(r, o, steps, tie_margin)[2] for r, o in zip(refs, outs))
+              and first_mismatch(refs[0], again, steps, tie_margin)[2], "prefix-cached greedy matches the reference")
+        print("\nALL CHECKS PASSED" if ok_all else "\nSOME CHECKS FAILED")
+        return 0 if ok_all else 2
+    except Exception as e:  # noqa: BLE001
+        print(f"error: {e}", file=sys.stderr)
+        return 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())
