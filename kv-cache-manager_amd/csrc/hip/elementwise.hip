@@ -46,22 +46,34 @@ __global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__
 
 // -------------------------------------------------------------------------------- RMS norm
 // v = x[src] (+ add[src]); optionally x[src] = v; out[r] = w * round(v * inv)  with
-// inv = 1/sqrt(mean(v^2) + eps).  src = rows ? rows[r] : r.
+// inv = 1/sqrt(mean(v^2) + eps).  src = rows ? rows[r] : r.  The added term is a tensor, or the
+// split-K partial sums of the product that made it ([S][T][H] floats, added in split order and
+// rounded to the storage type as the stored product would have been).
 constexpr int kNormThreads = 256;
 template <class TA, class TW, class TO>
 __global__ void __launch_bounds__(kNormThreads)
-    rmsnorm_kernel(float* __restrict__ x, const TA* __restrict__ add, const int* __restrict__ rows,
-                   const TW* __restrict__ w, TO* __restrict__ out, int H, float eps, int write_back) {
+    rmsnorm_kernel(float* __restrict__ x, const TA* __restrict__ add, const float* __restrict__ partials, int S,
+                   int T, const int* __restrict__ rows, const TW* __restrict__ w, TO* __restrict__ out, int H,
+                   float eps, int write_back) {
   __shared__ float scratch[kNormThreads / kWave + 1];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   float* xr = x + size_t(src) * H;
   const TA* ar = add ? add + size_t(src) * H : nullptr;
+  const float* pr = partials ? partials + size_t(src) * H : nullptr;
+  const size_t pstride = size_t(T) * H;
+  const bool adds = ar || pr;
+  auto added = [&](int i) {
+    if (ar) return load_f(ar + i);
+    float a = 0.f;
+    for (int s = 0; s < S; ++s) a += pr[s * pstride + i];
+    return round_to<TO>(a);
+  };
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += kNormThreads) {
     float v = xr[i];
-    if (ar) {
-      v += load_f(ar + i);
+    if (adds) {
+      v += added(i);
       if (write_back) xr[i] = v;
     }
     ss += v * v;
@@ -71,7 +83,7 @@ __global__ void __launch_bounds__(kNormThreads)
   TO* o = out + size_t(r) * H;
   for (int i = threadIdx.x; i < H; i += kNormThreads) {
     float v = xr[i];
-    if (ar && !write_back) v += load_f(ar + i);
+    if (adds && !write_back) v += added(i);
     store_f(o + i, load_f(w + i) * round_to<TO>(v * inv));
   }
 }
@@ -81,13 +93,26 @@ __global__ void __launch_bounds__(kNormThreads)
 // (pairs (j, j + hd/2), angle = float(pos) * inv_freq[j] in 32-bit); rotated k and plain v are
 // copied to the paged cache at slot = page * B + offset, layout [page][kv_head][B][hd].
 // inv_freq == null: no rotation.  slots == null or slot < 0: no cache write.
+// partials != null: the fused rows do not exist yet; they are the split-K sums [S][rows][width]
+// of the projection that makes them (added in split order, rounded to the storage type), and only
+// what a later kernel reads is stored: q to the fused rows, k and v to the cache.
 template <class T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, const int* __restrict__ slots,
-                                  T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int hd, int B) {
+                                  T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int hd, int B,
+                                  const float* __restrict__ partials, int S) {
   const int t = blockIdx.x;
   T* row = qkv + size_t(t) * row_stride;
   const int half = hd / 2;
+  const int width = (nh + 2 * nkv) * hd;
+  const float* prow = partials ? partials + size_t(t) * width : nullptr;
+  const size_t pstride = size_t(gridDim.x) * width;
+  auto value = [&](int c) {
+    if (!prow) return load_f(row + c);
+    float a = 0.f;
+    for (int s = 0; s < S; ++s) a += prow[s * pstride + c];
+    return round_to<T>(a);
+  };
   const int slot = slots ? slots[t] : -1;
   const size_t page = slot >= 0 ? slot / B : 0;
   const int off = slot >= 0 ? slot % B : 0;
@@ -98,26 +123,29 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
       const int h = i / half, j = i % half;
       float sn, cs;
       sincosf(pos * inv_freq[j], &sn, &cs);
-      T* base = row + size_t(h) * hd;
-      const float a = load_f(base + j), b = load_f(base + j + half);
+      const int c = h * hd + j;
+      const float a = value(c), b = value(c + half);
       const float ra = a * cs - b * sn, rb = b * cs + a * sn;
-      store_f(base + j, ra);
-      store_f(base + j + half, rb);
+      if (!prow || h < nh) {
+        store_f(row + c, ra);
+        store_f(row + c + half, rb);
+      }
       if (slot >= 0 && h >= nh) {
         T* dst = kcache + ((page * nkv + (h - nh)) * B + off) * hd;
         store_f(dst + j, ra);
         store_f(dst + j + half, rb);
       }
     }
+  } else if (prow) {
+    for (int i = threadIdx.x; i < nh * hd; i += blockDim.x) store_f(row + i, value(i));
   }
   if (slot < 0) return;
-  const T* ksrc = row + size_t(nh) * hd;
-  const T* vsrc = row + size_t(nh + nkv) * hd;
+  const int koff = nh * hd, voff = (nh + nkv) * hd;
   for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
     const int h = i / hd, d = i % hd;
     const size_t dst = ((page * nkv + h) * B + off) * hd + d;
-    if (!inv_freq) kcache[dst] = ksrc[i];
-    vcache[dst] = vsrc[i];
+    if (!inv_freq) store_f(kcache + dst, value(koff + i));
+    store_f(vcache + dst, value(voff + i));
   }
 }
 
@@ -161,13 +189,17 @@ int kvcm_embed(const int* ids, const void* table, int table_dtype, float* x, int
   return launch_status("embed");
 }
 
-int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const int* rows, const void* w, int w_dtype, void* out,
-                 int out_dtype, int R, int H, float eps, int write_back, hipStream_t s) {
+// add: a tensor of x's shape, or null.  partials: split-K sums [S][T][H] (T = rows of x), or null.
+int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const float* partials, int S, int T, const int* rows,
+                 const void* w, int w_dtype, void* out, int out_dtype, int R, int H, float eps, int write_back,
+                 hipStream_t s) {
   if (R == 0) return 0;
   KVCM_REQUIRE(R > 0 && H > 0, "rmsnorm: bad sizes R=%d H=%d", R, H);
-  KVCM_REQUIRE(!(rows && add && write_back), "rmsnorm: a gathered add cannot write back");
-#define KVCM_NORM(TA, TW, TO)                                                                      \
-  rmsnorm_kernel<TA, TW, TO><<<R, kNormThreads, 0, s>>>(x, static_cast<const TA*>(add), rows,       \
+  KVCM_REQUIRE(!(rows && (add || partials) && write_back), "rmsnorm: a gathered add cannot write back");
+  KVCM_REQUIRE(!(add && partials), "rmsnorm: the added term is a tensor or partial sums, not both");
+  KVCM_REQUIRE(!partials || (S >= 1 && T >= 1), "rmsnorm: partial sums need their split count and row count");
+#define KVCM_NORM(TA, TW, TO)                                                                              \
+  rmsnorm_kernel<TA, TW, TO><<<R, kNormThreads, 0, s>>>(x, static_cast<const TA*>(add), partials, S, T, rows, \
                                                         static_cast<const TW*>(w), static_cast<TO*>(out), H, eps, write_back)
   const int key = ((add ? add_dtype : out_dtype) << 2) | (w_dtype << 1) | out_dtype;
   switch (key) {
@@ -184,20 +216,23 @@ int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const int* rows, cons
 
 int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, const float* inv_freq,
                     const int* slots, void* kcache, void* vcache, int T, int nh, int nkv, int hd, int B,
-                    hipStream_t s) {
+                    const float* partials, int S, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(hd > 0 && hd % 2 == 0, "rope: head_dim %d must be even", hd);
   KVCM_REQUIRE(nh >= 0 && nkv >= 0 && row_stride >= (nh + 2 * nkv) * hd, "rope: row stride %d too small", row_stride);
   KVCM_REQUIRE(!slots || (kcache && vcache && B > 0), "rope: cache write without a cache");
   KVCM_REQUIRE(!inv_freq || positions, "rope: rotation without positions");
+  KVCM_REQUIRE(!partials || S >= 1, "rope: partial sums need their split count");
   const int work = (nh + nkv) * hd / 2;
   const int threads = work >= 256 ? 256 : work >= 128 ? 128 : 64;
   if (dtype == kF32)
     rope_cache_kernel<float><<<T, threads, 0, s>>>(static_cast<float*>(qkv), row_stride, positions, inv_freq, slots,
-                                                  static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, hd, B);
+                                                  static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, hd, B,
+                                                  partials, S);
   else if (dtype == kBF16)
     rope_cache_kernel<bf16_t><<<T, threads, 0, s>>>(static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots,
-                                                   static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, hd, B);
+                                                   static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, hd, B,
+                                                   partials, S);
   else KVCM_REQUIRE(false, "rope: unknown dtype %d", dtype);
   return launch_status("rope_cache");
 }

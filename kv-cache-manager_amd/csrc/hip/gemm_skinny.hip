@@ -1,0 +1,180 @@
+// Decode-shaped products: Y[M,N] = X[M,K] * W[N,K]^T with few rows (M <= 64) and a weight matrix
+// that has to be streamed from HBM once.  The reference leaves these to cuBLAS
+// (src/model/llama.cpp:45-52); here the point is to keep enough weight bytes in flight on 256 CUs.
+//
+// One workgroup (4 waves) owns 16 output columns and one slice of K ("split"); its waves divide
+// the slice among themselves, each streaming its rows of W straight from global memory into
+// MFMA operand registers (every lane 32 contiguous bytes, four lanes one 128-byte line) and
+// multiplying with the matching pieces of X (v_mfma_f32_16x16x32_bf16).  The four waves' sums
+// are added through LDS in a fixed order.  With one split the result is stored; with S splits the
+// 32-bit partial sums go to scratch [S][M][N] and the consumer adds them in split order:
+// reduce_store below, or the fused consumers (residual add + RMS norm, SwiGLU, rotary + cache
+// write) in elementwise.hip.  No atomics: the result is the same on every run.
+#include "common.h"
+
+namespace kvcm {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int kUnit = 64;  // k elements per unit: 4 lanes x 16 elements = one 128-byte line per row
+
+union Frag {
+  uint4 u;
+  bf16x8 v;
+};
+
+template <int MT, class TO>
+__global__ void __launch_bounds__(256)
+    gemm_skinny_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ partials,
+                       TO* __restrict__ out, int M, int N, int K, int ldx, int ldw, int ldo, int S) {
+  __shared__ f32x4 red[4][MT][kWave];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int r = lane % 16, kq = lane / 16;
+  const int n0 = blockIdx.x * 16;
+  const int s = blockIdx.y;
+  const int units = K / kUnit;
+  const int u_lo = int((long long)units * s / S), u_hi = int((long long)units * (s + 1) / S);
+  const int span = u_hi - u_lo;
+  const int w_lo = u_lo + span * wave / 4, w_hi = u_lo + span * (wave + 1) / 4;
+
+  const uint16_t* wrow = W + size_t(n0 + r) * ldw + kq * 16;
+  const uint16_t* xrow[MT];
+  bool live[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + r;
+    live[t] = m < M;
+    xrow[t] = X + size_t(live[t] ? m : 0) * ldx + kq * 16;
+  }
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  int u = w_lo;
+  for (; u + 2 <= w_hi; u += 2) {  // two units per trip: four weight loads in flight per lane
+    Frag b[4];
+    const uint16_t* p = wrow + size_t(u) * kUnit;
+    b[0].u = *reinterpret_cast<const uint4*>(p);
+    b[1].u = *reinterpret_cast<const uint4*>(p + 8);
+    b[2].u = *reinterpret_cast<const uint4*>(p + kUnit);
+    b[3].u = *reinterpret_cast<const uint4*>(p + kUnit + 8);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      Frag a[4];
+      const uint16_t* q = xrow[t] + size_t(u) * kUnit;
+      const uint4 zero = {0u, 0u, 0u, 0u};
+      a[0].u = live[t] ? *reinterpret_cast<const uint4*>(q) : zero;
+      a[1].u = live[t] ? *reinterpret_cast<const uint4*>(q + 8) : zero;
+      a[2].u = live[t] ? *reinterpret_cast<const uint4*>(q + kUnit) : zero;
+      a[3].u = live[t] ? *reinterpret_cast<const uint4*>(q + kUnit + 8) : zero;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[i].v, acc[t], 0, 0, 0);
+    }
+  }
+  for (; u < w_hi; ++u) {
+    Frag b[2];
+    const uint16_t* p = wrow + size_t(u) * kUnit;
+    b[0].u = *reinterpret_cast<const uint4*>(p);
+    b[1].u = *reinterpret_cast<const uint4*>(p + 8);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      Frag a[2];
+      const uint16_t* q = xrow[t] + size_t(u) * kUnit;
+      const uint4 zero = {0u, 0u, 0u, 0u};
+      a[0].u = live[t] ? *reinterpret_cast<const uint4*>(q) : zero;
+      a[1].u = live[t] ? *reinterpret_cast<const uint4*>(q + 8) : zero;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[i].v, acc[t], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
+  __syncthreads();
+  for (int item = threadIdx.x; item < MT * kWave; item += 256) {
+    const int t = item / kWave, l = item % kWave;
+    f32x4 v = red[0][t][l];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const f32x4 o = red[w][t][l];
+      v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3];
+    }
+    const int n = n0 + l % 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = t * 16 + (l / 16) * 4 + i;
+      if (m >= M) continue;
+      if (S > 1) partials[(size_t(s) * M + m) * N + n] = v[i];
+      else store_f(out + size_t(m) * ldo + n, v[i]);
+    }
+  }
+}
+
+// out[m][n] = sum over splits, in split order.
+template <class TO>
+__global__ void reduce_store_kernel(const float* __restrict__ partials, TO* __restrict__ out, int M, int N, int ldo, int S) {
+  const size_t i = blockIdx.x * size_t(blockDim.x) + threadIdx.x;
+  if (i >= size_t(M) * N) return;
+  float v = 0.f;
+  for (int s = 0; s < S; ++s) v += partials[size_t(s) * M * N + i];
+  store_f(out + (i / N) * ldo + i % N, v);
+}
+
+}  // namespace kvcm
+
+using namespace kvcm;
+
+extern "C" {
+
+// How many splits of K a launch of this shape uses (0: the shape is not supported by this kernel).
+int kvcm_gemm_skinny_splits(int M, int N, int K) {
+  if (M <= 0 || M > 64 || N % 16 != 0 || K % kUnit != 0 || N <= 0 || K <= 0) return 0;
+  const int tiles = N / 16, units = K / kUnit;
+  int S = (640 + tiles - 1) / tiles;           // aim at >= 640 workgroups (2.5 per CU)
+  if (S > units / 2) S = units / 2;            // at least two units per split ...
+  if (S < 1) S = 1;
+  if (S > 16) S = 16;
+  return S;
+}
+
+// S == 1: the result is stored to `out` (bfloat16 or float32).  S > 1: partial sums are written to
+// `partials` [S][M][N]; `out` is not touched (pass S from kvcm_gemm_skinny_splits).
+int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, int out_dtype, int M, int N, int K,
+                     int ldx, int ldw, int ldo, int S, hipStream_t st) {
+  KVCM_REQUIRE(kvcm_gemm_skinny_splits(M, N, K) > 0, "gemm_skinny: unsupported shape M=%d N=%d K=%d", M, N, K);
+  KVCM_REQUIRE(S >= 1 && S <= K / kUnit, "gemm_skinny: bad split count %d", S);
+  KVCM_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0 && reinterpret_cast<uintptr_t>(X) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(W) % 16 == 0,
+               "gemm_skinny: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
+  KVCM_REQUIRE(ldx >= K && ldw >= K, "gemm_skinny: leading dimensions too small");
+  KVCM_REQUIRE(S == 1 ? (out != nullptr && ldo >= N) : partials != nullptr, "gemm_skinny: missing output buffer");
+  const dim3 grid(N / 16, S);
+  const uint16_t* x = static_cast<const uint16_t*>(X);
+  const uint16_t* w = static_cast<const uint16_t*>(W);
+  const int mt = (M + 15) / 16;
+#define KVCM_SKINNY(MT, TO) \
+  gemm_skinny_kernel<MT, TO><<<grid, 256, 0, st>>>(x, w, partials, static_cast<TO*>(out), M, N, K, ldx, ldw, ldo, S)
+  if (out_dtype == kBF16) {
+    if (mt == 1) KVCM_SKINNY(1, bf16_t); else if (mt == 2) KVCM_SKINNY(2, bf16_t); else if (mt == 3) KVCM_SKINNY(3, bf16_t); else KVCM_SKINNY(4, bf16_t);
+  } else if (out_dtype == kF32) {
+    if (mt == 1) KVCM_SKINNY(1, float); else if (mt == 2) KVCM_SKINNY(2, float); else if (mt == 3) KVCM_SKINNY(3, float); else KVCM_SKINNY(4, float);
+  } else {
+    KVCM_REQUIRE(false, "gemm_skinny: unknown output dtype %d", out_dtype);
+  }
+#undef KVCM_SKINNY
+  return launch_status("gemm_skinny");
+}
+
+int kvcm_reduce_store(const float* partials, void* out, int out_dtype, int M, int N, int ldo, int S, hipStream_t st) {
+  if (M == 0 || N == 0) return 0;
+  KVCM_REQUIRE(M > 0 && N > 0 && S >= 1 && ldo >= N, "reduce_store: bad sizes");
+  const size_t n = size_t(M) * N;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  if (out_dtype == kBF16) reduce_store_kernel<bf16_t><<<blocks, 256, 0, st>>>(partials, static_cast<bf16_t*>(out), M, N, ldo, S);
+  else if (out_dtype == kF32) reduce_store_kernel<float><<<blocks, 256, 0, st>>>(partials, static_cast<float*>(out), M, N, ldo, S);
+  else KVCM_REQUIRE(false, "reduce_store: unknown output dtype %d", out_dtype);
+  return launch_status("reduce_store");
+}
+
+}  // extern "C"

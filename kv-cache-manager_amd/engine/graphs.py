@@ -43,6 +43,16 @@ class DecodeGraphs:
         raise RuntimeError("no bucket")
 
     def _forward(self, layout, bucket):
+        """Only kernels of this package inside a graph: a library product may record nodes that
+        clear memory, which do not replay reliably."""
+        ops = self.runner.ops
+        keep, ops.LIBRARY_GEMM_MIN_ROWS = ops.LIBRARY_GEMM_MIN_ROWS, 0
+        try:
+            self._forward_inner(layout, bucket)
+        finally:
+            ops.LIBRARY_GEMM_MIN_ROWS = keep
+
+    def _forward_inner(self, layout, bucket):
         step = StepContext(self.runner, layout)
         logits = self.runner.model.forward(step)
         s = self.sampler

@@ -31,8 +31,8 @@ class ModelLimits:
 class Workspace:
     """Named device buffers with fixed capacity, reused by every step (stable addresses)."""
 
-    def __init__(self, device, default_dtype, limits: ModelLimits):
-        self.device, self.default_dtype, self.limits = device, default_dtype, limits
+    def __init__(self, device, default_dtype, limits: ModelLimits, ops=None):
+        self.device, self.default_dtype, self.limits, self.ops = device, default_dtype, limits, ops
         self.buffers: Dict[str, torch.Tensor] = {}
         self.row_caps = {"head_in": limits.max_logit_rows, "logits": limits.max_logit_rows}
 
@@ -49,8 +49,18 @@ class Workspace:
             self.buffers[key] = buf
         return buf[:rows]
 
+    def scratch(self, name, rows, n, k):
+        """Float32 scratch for the partial sums of a split-K product [rows, k] x [n, k], or None
+        when that shape is not split.  Sized once for the most rows the split kernel takes."""
+        key = ("scratch", name, n, k)
+        if key not in self.buffers:
+            splits = self.ops.skinny_splits(min(64, max(rows, 1)), n, k) if self.ops is not None else 0
+            self.buffers[key] = (torch.empty(splits * 64 * n, dtype=torch.float32, device=self.device)
+                                 if splits > 1 else None)
+        return self.buffers[key]
+
     def bytes(self):
-        return sum(b.numel() * b.element_size() for b in self.buffers.values())
+        return sum(b.numel() * b.element_size() for b in self.buffers.values() if b is not None)
 
 
 class StepContext:
@@ -96,6 +106,11 @@ class StepContext:
     def ws(self, name, shape, dtype=None):
         return self.runner.workspace.get(name, shape, dtype)
 
+    def scratch(self, name, rows, n, k):
+        if rows > 64 or self.runner.dtype != torch.bfloat16:
+            return None
+        return self.runner.workspace.scratch(name, rows, n, k)
+
     def attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window=0):
         self.runner.attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window)
 
@@ -105,7 +120,7 @@ class ModelRunner:
         self.model, self.core, self.storages, self.limits = model, core, storages, limits
         self.dtype, self.device, self.attn = dtype, device, attn
         self.ops = model.ctx.ops
-        self.workspace = Workspace(device, dtype, limits)
+        self.workspace = Workspace(device, dtype, limits, self.ops)
         G = core.num_groups
         ints = (4 * limits.max_tokens + 4 * limits.max_seqs + 1 + limits.max_logit_rows
                 + G * (limits.max_tokens + limits.max_seqs * limits.max_blocks_per_seq) + 64)

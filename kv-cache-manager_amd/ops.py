@@ -30,8 +30,11 @@ def _declare(lib):
 
     lib.kvcm_hip_last_error.restype = C.c_char_p
     fn("kvcm_embed", vp, vp, i, vp, i, i, i, vp)
-    fn("kvcm_rmsnorm", vp, vp, i, vp, vp, i, vp, i, i, i, f, i, vp)
-    fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
+    fn("kvcm_rmsnorm", vp, vp, i, vp, i, i, vp, vp, i, vp, i, i, i, f, i, vp)
+    fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp)
+    fn("kvcm_gemm_skinny_splits", i, i, i)
+    fn("kvcm_gemm_skinny", vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp)
+    fn("kvcm_reduce_store", vp, vp, i, i, i, i, i, vp)
     fn("kvcm_swiglu", vp, vp, i, i, i, vp)
     fn("kvcm_add_residual", vp, vp, i, C.c_longlong, vp)
     fn("kvcm_gemm_f32", vp, vp, vp, i, i, i, i, i, i, vp)
@@ -102,9 +105,29 @@ def embed(ids, table, out):
     _check(lib().kvcm_embed(_ptr(ids), _ptr(table), _DT[table.dtype], _ptr(out), T, H, table.shape[0], _stream()))
 
 
+class PartialSums:
+    """The output of a split-K product that has not been added up yet: ``data`` holds [splits, rows,
+    cols] 32-bit sums.  The fused consumers (rmsnorm's ``add``, rope_cache's ``source``) add them in
+    split order and round the sum to ``dtype`` as the stored product would have been."""
+
+    def __init__(self, data, splits, rows, cols, out):
+        self.data, self.splits, self.rows, self.cols, self.out = data, splits, rows, cols, out
+        self.dtype = out.dtype
+
+    def materialize(self):
+        """Adds the splits up into the product's own output buffer [rows, cols] and returns it."""
+        _check(lib().kvcm_reduce_store(_ptr(self.data), _ptr(self.out), _DT[self.out.dtype], self.rows, self.cols,
+                                       self.out.stride(0), self.splits, _stream()))
+        return self.out
+
+
 def rmsnorm(x, weight, out, eps, add=None, rows=None, write_back=True):
     """v = x[src] (+ add[src]); x[src] = v when write_back; out[r] = weight * round(v * rsqrt(mean v^2 + eps)).
-    src = rows[r] if rows is given, else r."""
+    src = rows[r] if rows is given, else r.  ``add`` is a tensor of x's shape or PartialSums."""
+    partial = add if isinstance(add, PartialSums) else None
+    if partial is not None:
+        _need(partial.cols == x.shape[1] and partial.rows == x.shape[0], "partial sums must match x")
+        add = None
     _dev(x, weight, out, add, rows)
     R, H = out.shape
     _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == H, "x must be contiguous float32 [T, H]")
@@ -116,18 +139,24 @@ def rmsnorm(x, weight, out, eps, add=None, rows=None, write_back=True):
         _i32(rows, "rows", R)
     if add is not None:
         _need(add.shape == x.shape and add.is_contiguous(), "add must match x")
-    wb = bool(write_back) and add is not None and rows is None
-    _check(lib().kvcm_rmsnorm(_ptr(x), _ptr(add), _DT[add.dtype] if add is not None else 0, _ptr(rows), _ptr(weight),
+    wb = bool(write_back) and (add is not None or partial is not None) and rows is None
+    _check(lib().kvcm_rmsnorm(_ptr(x), _ptr(add), _DT[add.dtype] if add is not None else 0,
+                              _ptr(partial.data) if partial else 0, partial.splits if partial else 0,
+                              partial.rows if partial else 0, _ptr(rows), _ptr(weight),
                               _DT[weight.dtype], _ptr(out), _DT[out.dtype], R, H, float(eps), int(wb), _stream()))
 
 
 def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcache=None, vcache=None,
-               block_size=0, rows=None):
+               block_size=0, rows=None, source=None):
     """Rotates the q and k heads of the fused rows in place (inv_freq given) and copies k (rotated)
-    and v to the paged cache (slots given).  Cache layout [pages, nkv, block_size, hd]."""
+    and v to the paged cache (slots given).  Cache layout [pages, nkv, block_size, hd].  With
+    ``source`` (PartialSums of the projection) the rows are read from there; q lands in ``qkv``."""
     _dev(qkv, positions, inv_freq, slots, kcache, vcache)
     _rows2d(qkv, "qkv")
     T = qkv.shape[0] if rows is None else rows
+    if source is not None:
+        _need(isinstance(source, PartialSums) and source.rows == T and source.cols == (nh + 2 * nkv) * hd,
+              "the partial sums do not have the shape of the fused rows")
     _need(qkv.shape[1] >= (nh + 2 * nkv) * hd, "qkv rows are too short for the head layout")
     if inv_freq is not None:
         _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == hd // 2 and inv_freq.is_contiguous(),
@@ -140,7 +169,9 @@ def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcac
             _need(c is not None and c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
                   and tuple(c.shape[1:]) == (nkv, block_size, hd), "cache must be [pages, nkv, block_size, hd]")
     _check(lib().kvcm_rope_cache(_ptr(qkv), _DT[qkv.dtype], qkv.stride(0), _ptr(positions), _ptr(inv_freq),
-                                 _ptr(slots), _ptr(kcache), _ptr(vcache), T, nh, nkv, hd, block_size, _stream()))
+                                 _ptr(slots), _ptr(kcache), _ptr(vcache), T, nh, nkv, hd, block_size,
+                                 _ptr(source.data) if source is not None else 0,
+                                 source.splits if source is not None else 0, _stream()))
 
 
 def swiglu(gate_up, out):
@@ -158,9 +189,24 @@ def add_residual(x, y):
     _check(lib().kvcm_add_residual(_ptr(x), _ptr(y), _DT[y.dtype], x.numel(), _stream()))
 
 
-def gemm(x, w, out):
-    """out[M, N] = x[M, K] @ w[N, K]^T.  float32 x float32 -> float32 (plain FMA), or
-    bfloat16 x bfloat16 -> bfloat16 | float32 (MFMA, 32-bit accumulation)."""
+# Rows from which a bfloat16 product is handed to the library (hipBLASLt through torch.matmul); the
+# reference leaves every product to its vendor library.  0 = always use the kernels of this package.
+LIBRARY_GEMM_MIN_ROWS = 128
+
+
+def skinny_splits(M, N, K):
+    """Split count the decode-shaped kernel uses for this shape, 0 when it does not take it."""
+    return lib().kvcm_gemm_skinny_splits(M, N, K)
+
+
+def gemm(x, w, out, scratch=None, keep_partial=False):
+    """out[M, N] = x[M, K] @ w[N, K]^T.  float32 x float32 -> float32 (plain FMA, fixed k order), or
+    bfloat16 x bfloat16 -> bfloat16 | float32 (MFMA, 32-bit accumulation).
+
+    For few rows (M <= 64) of a bfloat16 product the weight-streaming kernel is used; when it
+    splits K it needs ``scratch`` (float32, at least splits*M*N elements).  With ``keep_partial``
+    the un-added partial sums are returned as PartialSums (for a fused consumer) instead of ``out``.
+    """
     _dev(x, w, out)
     for t, n in ((x, "x"), (w, "w"), (out, "out")):
         _rows2d(t, n)
@@ -170,10 +216,27 @@ def gemm(x, w, out):
     if x.dtype == torch.float32:
         _need(w.dtype == torch.float32 and out.dtype == torch.float32, "a float32 gemm needs float32 operands")
         _check(lib().kvcm_gemm_f32(_ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0), _stream()))
-    else:
-        _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm operands must both be bfloat16")
-        _check(lib().kvcm_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, x.stride(0), w.stride(0),
-                                    out.stride(0), _stream()))
+        return out
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm operands must both be bfloat16")
+    S = skinny_splits(M, N, K) if (x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+                                   and w.data_ptr() % 16 == 0) else 0
+    if S > 1 and (scratch is None or scratch.numel() < S * M * N):
+        S = 1 if scratch is None else max(1, min(S, scratch.numel() // (M * N)))
+    if S >= 1:
+        if S > 1:
+            _need(scratch.dtype == torch.float32 and scratch.is_contiguous() and scratch.is_cuda, "scratch must be float32")
+        _check(lib().kvcm_gemm_skinny(_ptr(x), _ptr(w), _ptr(scratch) if S > 1 else 0, _ptr(out), _DT[out.dtype], M, N, K,
+                                      x.stride(0), w.stride(0), out.stride(0), S, _stream()))
+        if S == 1:
+            return out
+        partial = PartialSums(scratch, S, M, N, out)
+        return partial if keep_partial else partial.materialize()
+    if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 and out.is_contiguous():
+        torch.matmul(x, w.t(), out=out)
+        return out
+    _check(lib().kvcm_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, x.stride(0), w.stride(0),
+                                out.stride(0), _stream()))
+    return out
 
 
 def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, nh, nkv, hd, scale, window=0,

@@ -12,9 +12,17 @@ from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, 
 from .base import (Block, Embedding, FeedForward, Head, KVCacheNeed, Mixer, Norm, ParamSpec, PositionEncoding)
 
 
-def _linear(ctx, x, w, out):
-    ctx.ops.gemm(x, w, out)
-    return out
+def _linear(ctx, step, x, w, name, keep_partial=False, dtype=None):
+    """x @ w^T into the work buffer ``name``.  With ``keep_partial`` the result may come back as
+    un-added split-K sums (ops.PartialSums) for a consumer that adds them up itself."""
+    out = step.ws(name, (x.shape[0], w.shape[0]), dtype)
+    scratch = step.scratch(name, x.shape[0], w.shape[0], w.shape[1]) if hasattr(step, "scratch") else None
+    return ctx.ops.gemm(x, w, out, scratch=scratch, keep_partial=keep_partial and scratch is not None)
+
+
+def _tensor(value):
+    """A product's result as a plain tensor (adds partial sums up if that is what it is)."""
+    return value.materialize() if hasattr(value, "materialize") else value
 
 
 @NORMS.register("rmsnorm")
@@ -24,6 +32,8 @@ class RMSNorm(Norm):
 
     def param_specs(self):
         return [ParamSpec("weight", ((self.prefix + "weight", (self.params["size"],)),), role="vector")]
+
+    accepts_partial_sums = True
 
     def forward(self, x, out, add=None, rows=None):
         self.ctx.ops.rmsnorm(x, self.w["weight"], out, self.params["eps"], add=add, rows=rows)
@@ -45,13 +55,15 @@ class Rotary(PositionEncoding):
     def ignorable_tensors(self):
         return (self.prefix + "rotary_emb.inv_freq",)
 
-    def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None):
+    accepts_partial_sums = True
+
+    def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None, source=None):
         if head_dim != self.params["dim"]:
             raise ValueError("rotary: this kernel rotates the whole head (dim must equal head_dim)")
         k, v = cache if cache is not None else (None, None)
         self.ctx.ops.rope_cache(qkv, num_heads, num_kv_heads, head_dim, positions=step.positions,
                                 inv_freq=self.inv_freq, slots=slots, kcache=k, vcache=v,
-                                block_size=self.ctx.block_size, rows=step.rows)
+                                block_size=self.ctx.block_size, rows=step.rows, source=source)
         return cache is not None
 
 
@@ -95,17 +107,19 @@ class GQAAttention(Mixer):
         ops = self.ctx.ops
         g = self.cache.group
         kc, vc = self.cache.k(self.cache_index), self.cache.v(self.cache_index)
+        fused = getattr(self.position, "accepts_partial_sums", False)
+        res = _linear(self.ctx, step, h, self.w["wqkv"], "qkv", keep_partial=fused)
         qkv = step.ws("qkv", (step.rows, self.q_dim + 2 * self.kv_dim))
-        _linear(self.ctx, h, self.w["wqkv"], qkv)
         slots = step.slots(g) if self.cache_owner else None
+        extra = {"source": res} if hasattr(res, "materialize") else {}
         stored = self.position.apply(step, qkv, self.nh, self.nkv, self.hd,
-                                     cache=(kc, vc) if self.cache_owner else None, slots=slots)
+                                     cache=(kc, vc) if self.cache_owner else None, slots=slots, **extra)
         if self.cache_owner and not stored:
             ops.rope_cache(qkv, self.nh, self.nkv, self.hd, slots=slots, kcache=kc, vcache=vc,
                            block_size=self.ctx.block_size, rows=step.rows)
         attn = step.ws("attn", (step.rows, self.q_dim))
         step.attention(qkv, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window)
-        return _linear(self.ctx, attn, self.w["wo"], step.ws("mixer_out", (step.rows, self.ctx.hidden_size)))
+        return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
 
 
 @FEED_FORWARDS.register("swiglu")
@@ -120,10 +134,10 @@ class SwiGLU(FeedForward):
 
     def forward(self, step, h):
         I = self.params["intermediate_size"]
-        gu = _linear(self.ctx, h, self.w["w_gate_up"], step.ws("gate_up", (step.rows, 2 * I)))
+        gu = _linear(self.ctx, step, h, self.w["w_gate_up"], "gate_up")
         act = step.ws("act", (step.rows, I))
         self.ctx.ops.swiglu(gu, act)
-        return _linear(self.ctx, act, self.w["w_down"], step.ws("ffn_out", (step.rows, self.ctx.hidden_size)))
+        return _linear(self.ctx, step, act, self.w["w_down"], "ffn_out", keep_partial=True)
 
 
 @EMBEDDINGS.register("token_embedding")
@@ -156,7 +170,8 @@ class LinearHead(Head):
         return (self.prefix + "weight",) if self.params.get("tied") else ()
 
     def forward(self, step, h, out):
-        return _linear(self.ctx, h, self.w["table"], out)
+        self.ctx.ops.gemm(h, self.w["table"], out)
+        return out
 
 
 @BLOCKS.register("prenorm_residual")
@@ -166,7 +181,8 @@ class PreNormResidual(Block):
 
     def forward(self, step, x, pending):
         h = step.ws("normed", (step.rows, x.shape[1]))
-        self.parts["norm_mixer"].forward(x, h, add=pending)
+        n1, n2 = self.parts["norm_mixer"], self.parts["norm_ffn"]
+        n1.forward(x, h, add=pending if getattr(n1, "accepts_partial_sums", False) else _tensor(pending))
         a = self.parts["mixer"].forward(step, h)
-        self.parts["norm_ffn"].forward(x, h, add=a)
+        n2.forward(x, h, add=a if getattr(n2, "accepts_partial_sums", False) else _tensor(a))
         return self.parts["ffn"].forward(step, h)

@@ -115,6 +115,8 @@ class Model:
         addition) and output head on those rows only (src/model/llama.cpp:126-128)."""
         R = row_index.numel()
         h_last = step.ws("head_in", (R, self.spec.hidden_size))
+        if hasattr(pending, "materialize") and not getattr(self.final_norm, "accepts_partial_sums", False):
+            pending = pending.materialize()
         self.final_norm.forward(x, h_last, add=pending, rows=row_index)
         logits = out if out is not None else step.ws("logits", (R, self.spec.vocab_size), torch.float32)
         return self.head.forward(step, h_last, logits)

@@ -476,3 +476,75 @@ def test_temperature_sampling_follows_softmax(ops):
                torch.zeros(N, dtype=torch.int64, device=DEV), torch.zeros(N, dtype=torch.int32, device=DEV))
     freq = np.bincount(out.cpu().numpy(), minlength=4) / N
     np.testing.assert_allclose(freq, [0.1, 0.2, 0.3, 0.4], atol=0.03)
+
+
+# ----------------------------------------------------------- decode-shaped product, split K
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(2048, 2048), (2560, 2048), (11264, 2048), (2048, 5632), (48, 64), (16, 192), (320, 128)])
+def test_gemm_skinny_with_and_without_splits(ops, M, N, K):
+    rng = np.random.default_rng(M * 7 + N)
+    x = _bf16_grid(rng.normal(size=(M, K)))
+    w = _bf16_grid(rng.normal(size=(N, K)) * 0.05)
+    ref = plain.linear(x, w)
+    S = ops.skinny_splits(M, N, K)
+    assert S >= 1
+    xt, wt = _t(x, torch.bfloat16), _t(w, torch.bfloat16)
+    for dtype in (torch.bfloat16, torch.float32):
+        out = torch.zeros(M, N, dtype=dtype, device=DEV)
+        scratch = torch.zeros(max(S, 1) * M * N, dtype=torch.float32, device=DEV)
+        got = ops.gemm(xt, wt, out, scratch=scratch)
+        assert got is out
+        tol = dict(rtol=2 ** -7, atol=1e-3) if dtype == torch.bfloat16 else dict(rtol=0, atol=2e-5 * math.sqrt(K))
+        np.testing.assert_allclose(_np(out), ref, **tol)
+        again = torch.zeros_like(out)
+        ops.gemm(xt, wt, again, scratch=scratch)
+        assert torch.equal(again, out), "the same product gave another result on a second run"
+    # without scratch the kernel runs unsplit and still gives the product
+    out = torch.zeros(M, N, dtype=torch.float32, device=DEV)
+    ops.gemm(xt, wt, out)
+    np.testing.assert_allclose(_np(out), ref, rtol=0, atol=2e-5 * math.sqrt(K))
+
+
+def test_partial_sums_feed_the_fused_norm_and_rope(ops):
+    rng = np.random.default_rng(30)
+    M, H, K = 5, 2048, 2048
+    x_in = _bf16_grid(rng.normal(size=(M, K)))
+    w = _bf16_grid(rng.normal(size=(H, K)) * 0.03)
+    S = ops.skinny_splits(M, H, K)
+    assert S > 1
+    scratch = torch.zeros(S * 64 * H, dtype=torch.float32, device=DEV)
+    out = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
+    part = ops.gemm(_t(x_in, torch.bfloat16), _t(w, torch.bfloat16), out, scratch=scratch, keep_partial=True)
+    assert isinstance(part, ops.PartialSums) and part.splits == S
+    resid = rng.normal(size=(M, H)).astype(np.float32)
+    nw = _bf16_grid(1 + 0.1 * rng.normal(size=H))
+    # fused: residual += round(product); out = norm(residual)
+    xt = _t(resid, torch.float32)
+    normed = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(xt, _t(nw, torch.bfloat16), normed, 1e-5, add=part)
+    # unfused: materialise the product, then the ordinary fused add
+    prod = part.materialize()
+    xt2 = _t(resid, torch.float32)
+    normed2 = torch.zeros_like(normed)
+    ops.rmsnorm(xt2, _t(nw, torch.bfloat16), normed2, 1e-5, add=prod)
+    assert torch.equal(xt, xt2) and torch.equal(normed, normed2)
+    np.testing.assert_allclose(_np(prod), plain.linear(x_in, w, plain.round_bf16), rtol=2 ** -7, atol=1e-3)
+    # gathered rows, nothing written back
+    xt3 = _t(resid, torch.float32)
+    g = torch.zeros(2, H, dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(xt3, _t(nw, torch.bfloat16), g, 1e-5, add=part, rows=_t([4, 1], torch.int32))
+    assert torch.equal(g, normed[[4, 1]]) and torch.equal(xt3, _t(resid, torch.float32))
+
+    # rotary + cache write from partial sums equals the same from the stored rows
+    nh, nkv, hd, B = 24, 4, 64, 16                                   # (24 + 8) * 64 = 2048 columns
+    pos = _t([0, 5, 17, 100, 101], torch.int32)
+    slots = _t([3, 20, 35, 1, 16], torch.int32)
+    inv = _t(_inv_freq(hd, 1e4), torch.float32)
+    caches = [torch.zeros(3, nkv, B, hd, dtype=torch.bfloat16, device=DEV) for _ in range(4)]
+    rows_a = prod.clone()
+    ops.rope_cache(rows_a, nh, nkv, hd, positions=pos, inv_freq=inv, slots=slots, kcache=caches[0], vcache=caches[1], block_size=B)
+    rows_b = torch.zeros_like(rows_a)
+    ops.rope_cache(rows_b, nh, nkv, hd, positions=pos, inv_freq=inv, slots=slots, kcache=caches[2], vcache=caches[3],
+                   block_size=B, source=part)
+    assert torch.equal(rows_a[:, :nh * hd], rows_b[:, :nh * hd])       # q
+    assert torch.equal(caches[0], caches[2]) and torch.equal(caches[1], caches[3])
