@@ -1,0 +1,244 @@
+// Decode attention over the paged bfloat16 cache: few query rows, long contexts, the context of
+// every row cut into fixed partitions that run in parallel and are merged afterwards.
+//
+// The structure follows the reference's kernels (src/cuda/paged_attention.cu:50-203): one
+// workgroup per (kv head, row, partition) serves all GROUP query heads of that kv head, so that
+// every key and value read from the cache is used GROUP times; pass 1 writes scaled scores to LDS,
+// pass 2 turns them into exp(s - max) per head, pass 3 accumulates P*V in registers; a second
+// kernel merges the partitions by their maxima and sums.  Retuned for wave64: a token is read by
+// HD/8 lanes, 16 bytes each (8 or 4 tokens per wave and trip), partitions are 256 tokens, and
+// any group size from 1 to 8 and head sizes 64 and 128 are compiled (other shapes take the
+// generic kernel).  Partition boundaries are absolute multiples of 256: a row's result does not
+// depend on the batch around it.
+#include <cfloat>
+
+#include "common.h"
+
+namespace kvcm {
+
+constexpr int kDecWaves = 4;
+constexpr int kDecPart = 256;
+
+__device__ __forceinline__ void unpack8(const uint4 v, float* f) {
+  f[0] = bf16_bits_to_float(v.x & 0xffffu); f[1] = bf16_bits_to_float(v.x >> 16);
+  f[2] = bf16_bits_to_float(v.y & 0xffffu); f[3] = bf16_bits_to_float(v.y >> 16);
+  f[4] = bf16_bits_to_float(v.z & 0xffffu); f[5] = bf16_bits_to_float(v.z >> 16);
+  f[6] = bf16_bits_to_float(v.w & 0xffffu); f[7] = bf16_bits_to_float(v.w >> 16);
+}
+
+// partial results per (row, head, partition): HD floats of o / sum, then max, then sum
+template <int HD, int GROUP>
+__global__ void __launch_bounds__(kDecWaves* kWave)
+    attention_decode_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
+                            const uint16_t* __restrict__ vcache, const int* __restrict__ tables, int table_stride,
+                            const int* __restrict__ row_seq, const int* __restrict__ ctx_lens, int nh, int nkv, int B,
+                            float scale, int num_parts, float* __restrict__ scratch) {
+  constexpr int VEC = 8;
+  constexpr int TG = HD / VEC;         // lanes per token
+  constexpr int TPW = kWave / TG;      // tokens per wave and trip
+  constexpr int STEP = kDecWaves * TPW;
+  const int kvh = blockIdx.x, row = blockIdx.y, part = blockIdx.z;
+  const int ctx = ctx_lens[row];
+  const int start = part * kDecPart;
+  if (start >= ctx) return;
+  const int end = min(ctx, start + kDecPart);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int sub = lane / TG, lid = lane % TG;
+
+  __shared__ float scores[GROUP][kDecPart];
+  __shared__ float red[kDecWaves][GROUP][HD];
+  __shared__ float s_max[GROUP], s_sum[GROUP];
+
+  const int* table = tables + size_t(row_seq[row]) * table_stride;
+  const size_t head_stride = size_t(B) * HD, page_stride = head_stride * nkv;
+
+  float qv[GROUP][VEC];
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(q + size_t(row) * q_stride + size_t(kvh * GROUP + g) * HD + lid * VEC);
+    unpack8(raw, qv[g]);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) qv[g][e] *= scale;
+  }
+
+  // pass 1: scores
+  for (int base = start + wave * TPW; base < end; base += STEP) {
+    const int t = base + sub;
+    const bool valid = t < end;
+    float kf[VEC];
+    if (valid) {
+      const uint16_t* kp = kcache + size_t(table[t / B]) * page_stride + kvh * head_stride + size_t(t % B) * HD + lid * VEC;
+      unpack8(*reinterpret_cast<const uint4*>(kp), kf);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) kf[e] = 0.f;
+    }
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) {
+      float s = 0.f;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) s = fmaf(qv[g][e], kf[e], s);
+#pragma unroll
+      for (int o = TG / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+      if (valid && lid == 0) scores[g][t - start] = s;
+    }
+  }
+  __syncthreads();
+
+  // pass 2: exp(s - max) and its sum, one wave per head at a time
+  const int n = end - start;
+  for (int g = wave; g < GROUP; g += kDecWaves) {
+    float m = -FLT_MAX;
+    for (int i = lane; i < n; i += kWave) m = fmaxf(m, scores[g][i]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int i = lane; i < n; i += kWave) {
+      const float e = expf(scores[g][i] - m);
+      scores[g][i] = e;
+      sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) { s_max[g] = m; s_sum[g] = sum; }
+  }
+  __syncthreads();
+
+  // pass 3: P * V
+  float acc[GROUP][VEC];
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[g][e] = 0.f;
+  for (int base = start + wave * TPW; base < end; base += STEP) {
+    const int t = base + sub;
+    if (t < end) {
+      const uint16_t* vp = vcache + size_t(table[t / B]) * page_stride + kvh * head_stride + size_t(t % B) * HD + lid * VEC;
+      float vf[VEC];
+      unpack8(*reinterpret_cast<const uint4*>(vp), vf);
+#pragma unroll
+      for (int g = 0; g < GROUP; ++g) {
+        const float w = scores[g][t - start];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[g][e] = fmaf(w, vf[e], acc[g][e]);
+      }
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+#pragma unroll
+      for (int o = TG; o < kWave; o <<= 1) acc[g][e] += __shfl_xor(acc[g][e], o, kWave);
+  if (sub == 0) {
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) red[wave][g][lid * VEC + e] = acc[g][e];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < GROUP * HD; i += kDecWaves * kWave) {
+    const int g = i / HD, d = i % HD;
+    float s = red[0][g][d];
+#pragma unroll
+    for (int w = 1; w < kDecWaves; ++w) s += red[w][g][d];
+    const size_t idx = (size_t(row) * nh + kvh * GROUP + g) * num_parts + part;
+    float* dst = scratch + idx * (HD + 2);
+    dst[d] = s / s_sum[g];
+    if (d == 0) { dst[HD] = s_max[g]; dst[HD + 1] = s_sum[g]; }
+  }
+}
+
+// out = sum_p w_p o_p / sum_p w_p with w_p = sum_p * exp(max_p - max)   (paged_attention.cu:186-203)
+template <int HD>
+__global__ void attention_decode_merge_kernel(const float* __restrict__ scratch, const int* __restrict__ ctx_lens,
+                                              uint16_t* __restrict__ out, int out_stride, int nh, int num_parts) {
+  const int head = blockIdx.x, row = blockIdx.y, d = threadIdx.x;
+  const int ctx = ctx_lens[row];
+  uint16_t* o = out + size_t(row) * out_stride + size_t(head) * HD + d;
+  if (ctx <= 0) { *o = 0; return; }
+  const int np = (ctx + kDecPart - 1) / kDecPart;
+  const float* base = scratch + (size_t(row) * nh + head) * num_parts * (HD + 2);
+  float m = -FLT_MAX;
+  for (int i = 0; i < np; ++i) m = fmaxf(m, base[i * (HD + 2) + HD]);
+  float num = 0.f, den = 0.f;
+  for (int i = 0; i < np; ++i) {
+    const float w = base[i * (HD + 2) + HD + 1] * expf(base[i * (HD + 2) + HD] - m);
+    num = fmaf(w, base[i * (HD + 2) + d], num);
+    den += w;
+  }
+  *o = float_to_bf16_bits(num / den);
+}
+
+template <int HD, int GROUP>
+int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* kc, const void* vc,
+                  const int* tables, int table_stride, const int* row_seq, const int* ctx_lens, int T, int nh, int nkv,
+                  int B, float scale, int num_parts, float* scratch, hipStream_t s) {
+  attention_decode_kernel<HD, GROUP><<<dim3(nkv, T, num_parts), kDecWaves * kWave, 0, s>>>(
+      static_cast<const uint16_t*>(q), q_stride, static_cast<const uint16_t*>(kc), static_cast<const uint16_t*>(vc),
+      tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale, num_parts, scratch);
+  attention_decode_merge_kernel<HD><<<dim3(nh, T), HD, 0, s>>>(scratch, ctx_lens, static_cast<uint16_t*>(out),
+                                                               out_stride, nh, num_parts);
+  return 0;
+}
+
+template <int HD>
+int dispatch_group(int group, const void* q, int q_stride, void* out, int out_stride, const void* kc, const void* vc,
+                   const int* tables, int table_stride, const int* row_seq, const int* ctx_lens, int T, int nh,
+                   int nkv, int B, float scale, int num_parts, float* scratch, hipStream_t s) {
+#define KVCM_DEC(G) \
+  case G: return launch_decode<HD, G>(q, q_stride, out, out_stride, kc, vc, tables, table_stride, row_seq, ctx_lens, T, nh, nkv, B, scale, num_parts, scratch, s)
+  switch (group) {
+    KVCM_DEC(1); KVCM_DEC(2); KVCM_DEC(3); KVCM_DEC(4); KVCM_DEC(5); KVCM_DEC(6); KVCM_DEC(7); KVCM_DEC(8);
+    default: return -1;
+  }
+#undef KVCM_DEC
+}
+
+}  // namespace kvcm
+
+using namespace kvcm;
+
+extern "C" {
+
+// 1 when this kernel takes the shape (bfloat16 only), else 0 (use the generic kernel).
+int kvcm_attention_decode_supported(int nh, int nkv, int hd) {
+  if (nkv <= 0 || nh % nkv) return 0;
+  const int g = nh / nkv;
+  return (hd == 64 || hd == 128) && g >= 1 && g <= 8;
+}
+
+// Floats of scratch a launch needs: rows * heads * partitions * (head_dim + 2).
+long long kvcm_attention_decode_scratch(int T, int nh, int hd, int max_context) {
+  const long long parts = (max_context + kDecPart - 1) / kDecPart;
+  return static_cast<long long>(T) * nh * (parts > 0 ? parts : 1) * (hd + 2);
+}
+
+// max_context: an upper bound of every row's context length (it fixes the number of partitions
+// launched; rows with shorter contexts leave the surplus workgroups at once).
+int kvcm_attention_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                          const void* vcache, const int* tables, int table_stride, const int* row_seq,
+                          const int* ctx_lens, int T, int nh, int nkv, int hd, int B, float scale, int max_context,
+                          float* scratch, long long scratch_floats, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(kvcm_attention_decode_supported(nh, nkv, hd), "attention_decode: unsupported shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
+  KVCM_REQUIRE(T > 0 && B > 0 && max_context > 0, "attention_decode: bad sizes T=%d B=%d max_context=%d", T, B, max_context);
+  KVCM_REQUIRE(q_stride >= nh * hd && out_stride >= nh * hd && q_stride % 8 == 0, "attention_decode: bad row strides");
+  KVCM_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(vcache) % 16 == 0, "attention_decode: operands must be 16-byte aligned");
+  KVCM_REQUIRE(scratch && scratch_floats >= kvcm_attention_decode_scratch(T, nh, hd, max_context),
+               "attention_decode: scratch too small");
+  KVCM_REQUIRE(T <= 65535, "attention_decode: too many rows (%d)", T);
+  const int num_parts = (max_context + kDecPart - 1) / kDecPart;
+  KVCM_REQUIRE(num_parts <= 65535, "attention_decode: context too long");
+  const int group = nh / nkv;
+  int rc;
+  if (hd == 64)
+    rc = dispatch_group<64>(group, q, q_stride, out, out_stride, kcache, vcache, tables, table_stride, row_seq, ctx_lens,
+                            T, nh, nkv, B, scale, num_parts, scratch, s);
+  else
+    rc = dispatch_group<128>(group, q, q_stride, out, out_stride, kcache, vcache, tables, table_stride, row_seq, ctx_lens,
+                             T, nh, nkv, B, scale, num_parts, scratch, s);
+  KVCM_REQUIRE(rc == 0, "attention_decode: no kernel for group size %d", group);
+  return launch_status("attention_decode");
+}
+
+}  // extern "C"

@@ -54,6 +54,7 @@ class DecodeGraphs:
 
     def _forward_inner(self, layout, bucket):
         step = StepContext(self.runner, layout)
+        step.max_context_bound = self.runner.limits.max_context_len
         logits = self.runner.model.forward(step)
         s = self.sampler
         self.runner.ops.sample(logits, s.out[:bucket], s.temperature[:bucket], s.seeds[:bucket],

@@ -59,6 +59,15 @@ class Workspace:
                                  if splits > 1 else None)
         return self.buffers[key]
 
+    def flat(self, name, numel, dtype=torch.float32):
+        """A flat buffer of at least ``numel`` elements (grows if a larger one is asked for)."""
+        key = ("flat", name, dtype)
+        buf = self.buffers.get(key)
+        if buf is None or buf.numel() < numel:
+            buf = torch.empty(numel, dtype=dtype, device=self.device)
+            self.buffers[key] = buf
+        return buf
+
     def bytes(self):
         return sum(b.numel() * b.element_size() for b in self.buffers.values() if b is not None)
 
@@ -74,6 +83,9 @@ class StepContext:
         self.seqs, self.real_seqs = L.seqs_padded, L.seqs
         self.logit_rows_padded, self.logit_rows = L.logit_rows_padded, L.logit_rows
         self.max_context, self.max_run = L.max_context, L.max_run
+        # what kernels that size their launch by the context may assume; a captured graph sets it
+        # to the largest context the engine allows, so that the launch fits every replay
+        self.max_context_bound = max(L.max_context, 1)
         d, h = runner.meta_dev, runner.meta_host
         T, S, R = self.rows, self.seqs, self.logit_rows_padded
         self.tokens = d[L.tokens:L.tokens + T]
@@ -140,9 +152,30 @@ class ModelRunner:
         return self.meta_host
 
     # ------------------------------------------------------------------------- attention
+    # Rows up to which a step is treated as decode-shaped by the partitioned attention kernel.
+    DECODE_ATTENTION_MAX_ROWS = 512
+
     def attention(self, step, q, out, kcache, vcache, g, nh, nkv, hd, scale, window):
-        self.ops.attention(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
-                           step.ctx_lens, nh, nkv, hd, scale, window, rows=step.rows)
+        """attn = "v1": one pass over the whole context per (row, head); "v2": contexts cut into
+        partitions and merged (bfloat16, decode-shaped steps); "auto": v2 where it applies.  The
+        32-bit path always takes v1, whose result does not depend on the batch."""
+        ops = self.ops
+        partitioned = (self.attn != "v1" and window == 0 and step.max_run == 1
+                       and step.rows <= self.DECODE_ATTENTION_MAX_ROWS
+                       and ops.attention_decode_supported(nh, nkv, hd, q.dtype))
+        if self.attn == "v2" and not partitioned and q.dtype == torch.bfloat16 and step.max_run == 1:
+            raise RuntimeError(f"attn=v2: the partitioned kernel does not take heads={nh} kv_heads={nkv} "
+                               f"head_dim={hd} window={window} rows={step.rows}")
+        if partitioned:
+            bound = step.max_context_bound
+            need = ops.attention_decode_scratch(step.rows, nh, hd, bound)
+            scratch = self.workspace.flat("attention_partials", max(need, ops.attention_decode_scratch(
+                min(self.DECODE_ATTENTION_MAX_ROWS, self.limits.max_tokens), nh, hd, self.limits.max_context_len)))
+            ops.attention_decode(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
+                                 step.ctx_lens, nh, nkv, hd, scale, bound, scratch, rows=step.rows)
+            return
+        ops.attention(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
+                      step.ctx_lens, nh, nkv, hd, scale, window, rows=step.rows)
 
     # ------------------------------------------------------------------------------ steps
     def _check(self, layout: BatchLayout):

@@ -41,6 +41,10 @@ def _declare(lib):
     fn("kvcm_gemm_bf16", vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_attention_generic", vp, i, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp)
     fn("kvcm_sample", vp, i, vp, vp, vp, vp, vp, i, i, vp)
+    fn("kvcm_attention_decode_supported", i, i, i)
+    lib.kvcm_attention_decode_scratch.restype = C.c_longlong
+    lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
+    fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
 
 
 def lib():
@@ -255,6 +259,35 @@ def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, n
     _check(lib().kvcm_attention_generic(_ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache),
                                         _ptr(vcache), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh,
                                         nkv, hd, kcache.shape[2], float(scale), int(window), _stream()))
+
+
+def attention_decode_supported(nh, nkv, hd, dtype):
+    return dtype == torch.bfloat16 and bool(lib().kvcm_attention_decode_supported(nh, nkv, hd))
+
+
+def attention_decode_scratch(rows, nh, hd, max_context):
+    return int(lib().kvcm_attention_decode_scratch(rows, nh, hd, max_context))
+
+
+def attention_decode(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, nh, nkv, hd, scale, max_context,
+                     scratch, rows=None):
+    """The same result as ``attention`` for bfloat16, contexts cut into partitions of 256 tokens
+    that run in parallel and are merged; ``max_context`` bounds every row's context length."""
+    _dev(q, out, kcache, vcache, tables, row_seq, ctx_lens, scratch)
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    T = q.shape[0] if rows is None else rows
+    _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "attention_decode is bfloat16 only")
+    _need(kcache.dim() == 4 and kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape == vcache.shape
+          and kcache.shape[1] == nkv and kcache.shape[3] == hd, "cache must be [pages, nkv, block_size, hd]")
+    _need(scratch.dtype == torch.float32 and scratch.is_contiguous(), "scratch must be contiguous float32")
+    _i32(row_seq, "row_seq", T)
+    _i32(ctx_lens, "ctx_lens", T)
+    _i32(tables, "tables")
+    _check(lib().kvcm_attention_decode(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
+                                       _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh, nkv, hd,
+                                       kcache.shape[2], float(scale), int(max_context), _ptr(scratch), scratch.numel(),
+                                       _stream()))
 
 
 def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_index=None):

@@ -548,3 +548,53 @@ def test_partial_sums_feed_the_fused_norm_and_rope(ops):
                    block_size=B, source=part)
     assert torch.equal(rows_a[:, :nh * hd], rows_b[:, :nh * hd])       # q
     assert torch.equal(caches[0], caches[2]) and torch.equal(caches[1], caches[3])
+
+
+# ------------------------------------------------------------ partitioned decode attention
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 4, 64), (8, 8, 64), (16, 4, 128), (32, 4, 128), (6, 2, 64), (5, 1, 128), (7, 7, 64)])
+@pytest.mark.parametrize("B", [8, 16, 64])
+def test_partitioned_decode_attention(ops, nh, nkv, hd, B):
+    rng = np.random.default_rng(nh * 31 + hd + B)
+    lens = [700, 256, 257, 1, 255, 33]
+    P = _paged_problem(rng, lens, nh, nkv, hd, B, all_rows=False)
+    ref = _ref_attention(P, nh, nkv, hd)
+    R = P["R"]
+    for bound in (max(lens), 2048):                     # the launch may be sized for a longer context
+        out = torch.zeros(R, nh * hd, dtype=torch.bfloat16, device=DEV)
+        scratch = torch.zeros(ops.attention_decode_scratch(R, nh, hd, bound), dtype=torch.float32, device=DEV)
+        ops.attention_decode(_t(P["Q"].reshape(R, nh * hd), torch.bfloat16), out, _t(P["Kc"], torch.bfloat16),
+                             _t(P["Vc"], torch.bfloat16), _t(P["tables"], torch.int32), P["max_blocks"],
+                             _t(P["row_seq"], torch.int32), _t(P["ctx"], torch.int32), nh, nkv, hd, 1.0 / math.sqrt(hd),
+                             bound, scratch)
+        np.testing.assert_allclose(_np(out).reshape(R, nh, hd), ref, atol=1e-2, rtol=0)
+    generic = _run_attention(ops, P, nh, nkv, hd, torch.bfloat16)
+    np.testing.assert_allclose(_np(out).reshape(R, nh, hd), generic, atol=2 ** -6, rtol=0)   # v1 vs v2: a rounding apart
+
+
+def test_partitioned_decode_attention_padding_rows_and_far_key(ops):
+    rng = np.random.default_rng(40)
+    nh, nkv, hd, B = 8, 2, 64, 16
+    P = _paged_problem(rng, [900, 10], nh, nkv, hd, B, all_rows=False)
+    far = 3                                                   # first partition, while the row spans four
+    P["Q"][0, 5] = 0.0
+    P["Q"][0, 5, 7] = 40.0
+    kvec = np.zeros(hd)
+    kvec[7] = 40.0
+    P["Kl"][0][far, 1] = kvec
+    P["Kc"][P["tables"][0, far // B], 1, far % B] = kvec
+    ctx = np.array([900, 10, 0], dtype=np.int32)              # a padding row with no context
+    q = np.concatenate([P["Q"].reshape(2, nh * hd), np.ones((1, nh * hd))])
+    out = torch.full((3, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    scratch = torch.zeros(ops.attention_decode_scratch(3, nh, hd, 1024), dtype=torch.float32, device=DEV)
+    ops.attention_decode(_t(q, torch.bfloat16), out, _t(P["Kc"], torch.bfloat16), _t(P["Vc"], torch.bfloat16),
+                         _t(P["tables"], torch.int32), P["max_blocks"], _t([0, 1, 0], torch.int32), _t(ctx, torch.int32),
+                         nh, nkv, hd, 1.0, 1024, scratch)
+    got = _np(out).reshape(3, nh, hd)
+    np.testing.assert_allclose(got[0, 5], P["Vl"][0][far, 1], atol=1e-2)
+    assert not got[2].any()
+    with pytest.raises(ops.KernelError, match="scratch too small"):
+        ops.attention_decode(_t(q, torch.bfloat16), out, _t(P["Kc"], torch.bfloat16), _t(P["Vc"], torch.bfloat16),
+                             _t(P["tables"], torch.int32), P["max_blocks"], _t([0, 1, 0], torch.int32), _t(ctx, torch.int32),
+                             nh, nkv, hd, 1.0, 4096, scratch)
+    assert not ops.attention_decode_supported(12, 1, 64, torch.bfloat16) and not ops.attention_decode_supported(4, 2, 48, torch.bfloat16)
+    assert not ops.attention_decode_supported(32, 4, 64, torch.float32)
