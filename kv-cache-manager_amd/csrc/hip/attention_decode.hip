@@ -5,11 +5,11 @@
 // workgroup per (kv head, row, partition) serves all GROUP query heads of that kv head, so that
 // every key and value read from the cache is used GROUP times; pass 1 writes scaled scores to LDS,
 // pass 2 turns them into exp(s - max) per head, pass 3 accumulates P*V in registers; a second
-// kernel merges the partitions by their maxima and sums.  Retuned for wave64: a token is read by
-// HD/8 lanes, 16 bytes each (8 or 4 tokens per wave and trip), partitions are 256 tokens, and
-// any group size from 1 to 8 and head sizes 64 and 128 are compiled (other shapes take the
-// generic kernel).  Partition boundaries are absolute multiples of 256: a row's result does not
-// depend on the batch around it.
+// kernel merges the partitions by their maxima and sums.  Rebuilt for CDNA4: scores come from the
+// matrix cores with the cache's own layout as operand, all of a partition's keys and values are
+// requested before the first use, partitions are 256 tokens, and any group size from 1 to 8 and
+// head sizes 64 and 128 are compiled (other shapes take the generic kernel).  Partition
+// boundaries are absolute multiples of 256: a row's result does not depend on the batch around it.
 #include <cfloat>
 
 #include "common.h"
@@ -19,81 +19,116 @@ namespace kvcm {
 constexpr int kDecWaves = 4;
 constexpr int kDecPart = 256;
 
-__device__ __forceinline__ void unpack8(const uint4 v, float* f) {
-  f[0] = bf16_bits_to_float(v.x & 0xffffu); f[1] = bf16_bits_to_float(v.x >> 16);
-  f[2] = bf16_bits_to_float(v.y & 0xffffu); f[3] = bf16_bits_to_float(v.y >> 16);
-  f[4] = bf16_bits_to_float(v.z & 0xffffu); f[5] = bf16_bits_to_float(v.z >> 16);
-  f[6] = bf16_bits_to_float(v.w & 0xffffu); f[7] = bf16_bits_to_float(v.w >> 16);
-}
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+union Frag8 {
+  uint4 u;
+  bf16x8 v;
+};
 
 // partial results per (row, head, partition): HD floats of o / sum, then max, then sum
+//
+// Scores: each wave takes 16-token tiles; the tile's keys are the B operand of
+// v_mfma_f32_16x16x32_bf16 exactly as they lie in the cache (a lane reads 16 bytes of one token),
+// the group's query heads are the A operand (rows beyond GROUP are zero), so a tile's scores for
+// all heads cost HD/32 matrix instructions and no cross-lane traffic.  P*V: each wave takes a
+// quarter of the partition's tokens, a lane owns HD/64 output dims of every head, values are read
+// one token row per instruction and the probabilities come from LDS as broadcasts; the only
+// reduction left is over the four waves.
 template <int HD, int GROUP>
 __global__ void __launch_bounds__(kDecWaves* kWave)
     attention_decode_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                             const uint16_t* __restrict__ vcache, const int* __restrict__ tables, int table_stride,
                             const int* __restrict__ row_seq, const int* __restrict__ ctx_lens, int nh, int nkv, int B,
                             float scale, int num_parts, float* __restrict__ scratch) {
-  constexpr int VEC = 8;
-  constexpr int TG = HD / VEC;         // lanes per token
-  constexpr int TPW = kWave / TG;      // tokens per wave and trip
-  constexpr int STEP = kDecWaves * TPW;
+  constexpr int KSTEPS = HD / 32;                    // matrix instructions per 16-token tile
+  constexpr int TILES = kDecPart / 16 / kDecWaves;   // tiles per wave
+  constexpr int DPL = HD / kWave;                    // output dims per lane in P*V
+  constexpr int TOKW = kDecPart / kDecWaves;         // tokens per wave in P*V
   const int kvh = blockIdx.x, row = blockIdx.y, part = blockIdx.z;
   const int ctx = ctx_lens[row];
   const int start = part * kDecPart;
   if (start >= ctx) return;
   const int end = min(ctx, start + kDecPart);
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int sub = lane / TG, lid = lane % TG;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
 
-  __shared__ float scores[GROUP][kDecPart];
+  __shared__ __attribute__((aligned(16))) float scores[GROUP][kDecPart];
   __shared__ float red[kDecWaves][GROUP][HD];
   __shared__ float s_max[GROUP], s_sum[GROUP];
 
   const int* table = tables + size_t(row_seq[row]) * table_stride;
   const size_t head_stride = size_t(B) * HD, page_stride = head_stride * nkv;
 
-  float qv[GROUP][VEC];
-#pragma unroll
-  for (int g = 0; g < GROUP; ++g) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(q + size_t(row) * q_stride + size_t(kvh * GROUP + g) * HD + lid * VEC);
-    unpack8(raw, qv[g]);
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) qv[g][e] *= scale;
+  // where each token of the partition lives: one table lookup per thread, shared through LDS
+  // (page id and slot in the page), instead of a chain of dependent lookups per load below
+  // Tokens beyond the context point at the last valid token: every load below is then
+  // unconditional (a branch around a load makes the compiler wait for it at once), and what
+  // is loaded for them is never used (no score is stored, their probability is zero).
+  // The offset of a token's row inside this kv head's part of the cache, in units of 8 elements.
+  __shared__ uint32_t where[kDecPart];
+  {
+    const int t = min(start + int(threadIdx.x), end - 1);
+    where[threadIdx.x] = uint32_t((size_t(table[t / B]) * page_stride + kvh * head_stride + size_t(t % B) * HD) / 8);
   }
+  __syncthreads();
 
-  // pass 1: scores
-  for (int base = start + wave * TPW; base < end; base += STEP) {
-    const int t = base + sub;
-    const bool valid = t < end;
-    float kf[VEC];
-    if (valid) {
-      const uint16_t* kp = kcache + size_t(table[t / B]) * page_stride + kvh * head_stride + size_t(t % B) * HD + lid * VEC;
-      unpack8(*reinterpret_cast<const uint4*>(kp), kf);
-    } else {
+  // ---- requests first: this wave's keys (tile layout) and values (one token row per load)
+  const int n16 = lane % 16, kq = lane / 16;
+  Frag8 kf[TILES][KSTEPS];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) kf[e] = 0.f;
-    }
+  for (int i = 0; i < TILES; ++i) {
+    const int tok = (wave + i * kDecWaves) * 16 + n16;
+    const uint16_t* kp = kcache + (size_t(where[tok]) << 3) + kq * 8;
 #pragma unroll
-    for (int g = 0; g < GROUP; ++g) {
-      float s = 0.f;
+    for (int c = 0; c < KSTEPS; ++c) kf[i][c].u = *reinterpret_cast<const uint4*>(kp + c * 32);
+  }
+  static_assert(TOKW == kWave, "one lane per token of the wave's quarter");
+  const uint32_t my_where = where[wave * TOKW + lane];
+  uint32_t vraw[TOKW];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) s = fmaf(qv[g][e], kf[e], s);
+  for (int i = 0; i < TOKW; ++i) {
+    const uint32_t w = __builtin_amdgcn_readlane(my_where, i);   // token i of the quarter, the same for every lane
+    const uint16_t* vp = vcache + (size_t(w) << 3) + lane * DPL;
+    if constexpr (DPL == 1) vraw[i] = *vp;
+    else vraw[i] = *reinterpret_cast<const uint32_t*>(vp);
+  }
+  Frag8 qf[KSTEPS];
+  const int qhead = kvh * GROUP + (n16 < GROUP ? n16 : 0);
 #pragma unroll
-      for (int o = TG / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
-      if (valid && lid == 0) scores[g][t - start] = s;
+  for (int c = 0; c < KSTEPS; ++c) {
+    qf[c].u = *reinterpret_cast<const uint4*>(q + size_t(row) * q_stride + size_t(qhead) * HD + c * 32 + kq * 8);
+    if (n16 >= GROUP) qf[c].u = uint4{0u, 0u, 0u, 0u};
+  }
+  // keep every request above ahead of the first use below: the point of this kernel is that a
+  // partition costs one trip to memory, not one per token
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- pass 1: scores[head][token] = scale * q . k
+#pragma unroll
+  for (int i = 0; i < TILES; ++i) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < KSTEPS; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c].v, kf[i][c].v, acc, 0, 0, 0);
+    const int tok = (wave + i * kDecWaves) * 16 + n16;       // accumulator: column = token, rows = heads 4*kq..+3
+    if (start + tok < end) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int g = kq * 4 + r;
+        if (g < GROUP) scores[g][tok] = acc[r] * scale;
+      }
     }
   }
   __syncthreads();
 
-  // pass 2: exp(s - max) and its sum, one wave per head at a time
+  // ---- pass 2: exp(s - max) and its sum, one wave per head at a time
   const int n = end - start;
   for (int g = wave; g < GROUP; g += kDecWaves) {
     float m = -FLT_MAX;
     for (int i = lane; i < n; i += kWave) m = fmaxf(m, scores[g][i]);
     m = wave_max(m);
     float sum = 0.f;
-    for (int i = lane; i < n; i += kWave) {
-      const float e = expf(scores[g][i] - m);
+    for (int i = lane; i < kDecPart; i += kWave) {
+      const float e = i < n ? expf(scores[g][i] - m) : 0.f;   // zero beyond the context: pass 3 reads whole quarters
       scores[g][i] = e;
       sum += e;
     }
@@ -102,38 +137,34 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
   }
   __syncthreads();
 
-  // pass 3: P * V
-  float acc[GROUP][VEC];
+  // ---- pass 3: P * V, lane owns dims lane*DPL .. +DPL-1 of every head
+  float acc[GROUP][DPL];
 #pragma unroll
   for (int g = 0; g < GROUP; ++g)
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[g][e] = 0.f;
-  for (int base = start + wave * TPW; base < end; base += STEP) {
-    const int t = base + sub;
-    if (t < end) {
-      const uint16_t* vp = vcache + size_t(table[t / B]) * page_stride + kvh * head_stride + size_t(t % B) * HD + lid * VEC;
-      float vf[VEC];
-      unpack8(*reinterpret_cast<const uint4*>(vp), vf);
+    for (int e = 0; e < DPL; ++e) acc[g][e] = 0.f;
+#pragma unroll
+  for (int i = 0; i < TOKW; i += 4) {
+    float4 p[GROUP];
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) p[g] = *reinterpret_cast<const float4*>(&scores[g][wave * TOKW + i]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float vf[DPL];
+      vf[0] = bf16_bits_to_float(vraw[i + j] & 0xffffu);
+      if constexpr (DPL == 2) vf[1] = bf16_bits_to_float(vraw[i + j] >> 16);
 #pragma unroll
       for (int g = 0; g < GROUP; ++g) {
-        const float w = scores[g][t - start];
+        const float w = j == 0 ? p[g].x : j == 1 ? p[g].y : j == 2 ? p[g].z : p[g].w;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[g][e] = fmaf(w, vf[e], acc[g][e]);
+        for (int e = 0; e < DPL; ++e) acc[g][e] = fmaf(w, vf[e], acc[g][e]);
       }
     }
   }
 #pragma unroll
   for (int g = 0; g < GROUP; ++g)
 #pragma unroll
-    for (int e = 0; e < VEC; ++e)
-#pragma unroll
-      for (int o = TG; o < kWave; o <<= 1) acc[g][e] += __shfl_xor(acc[g][e], o, kWave);
-  if (sub == 0) {
-#pragma unroll
-    for (int g = 0; g < GROUP; ++g)
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) red[wave][g][lid * VEC + e] = acc[g][e];
-  }
+    for (int e = 0; e < DPL; ++e) red[wave][g][lane * DPL + e] = acc[g][e];
   __syncthreads();
   for (int i = threadIdx.x; i < GROUP * HD; i += kDecWaves * kWave) {
     const int g = i / HD, d = i % HD;

@@ -88,6 +88,110 @@ __global__ void __launch_bounds__(kNormThreads)
   }
 }
 
+// The same computation for rows whose length is a multiple of 4 and at most 1024 * VPT: every
+// thread keeps its VPT groups of four values in registers and asks for all of its inputs at once,
+// so the row costs one round trip to memory instead of one per element.  Its sum of squares adds
+// in another order than the kernel above, so the two may differ in the last bit; which of them
+// runs depends on the row length and on alignment only, never on the batch.
+template <class T> __device__ __forceinline__ void load4(const T* p, float* f);
+template <> __device__ __forceinline__ void load4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <> __device__ __forceinline__ void load4<bf16_t>(const bf16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = bf16_bits_to_float(v.x & 0xffffu); f[1] = bf16_bits_to_float(v.x >> 16);
+  f[2] = bf16_bits_to_float(v.y & 0xffffu); f[3] = bf16_bits_to_float(v.y >> 16);
+}
+template <class T> __device__ __forceinline__ void store4(T* p, const float* f);
+template <> __device__ __forceinline__ void store4<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float* f) {
+  uint2 v;
+  v.x = float_to_bf16_bits(f[0]) | (uint32_t(float_to_bf16_bits(f[1])) << 16);
+  v.y = float_to_bf16_bits(f[2]) | (uint32_t(float_to_bf16_bits(f[3])) << 16);
+  *reinterpret_cast<uint2*>(p) = v;
+}
+
+template <class TA, class TW, class TO, int VPT>
+__global__ void __launch_bounds__(kNormThreads)
+    rmsnorm_rows4_kernel(float* __restrict__ x, const TA* __restrict__ add, const float* __restrict__ partials, int S,
+                         int T, const int* __restrict__ rows, const TW* __restrict__ w, TO* __restrict__ out, int H,
+                         float eps, int write_back) {
+  __shared__ float scratch[kNormThreads / kWave + 1];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* xr = x + size_t(src) * H;
+  const size_t pstride = size_t(T) * H;
+  float v[VPT][4], wv[VPT][4];
+  bool on[VPT];
+  // thread t owns elements 4 * (t + 256 k) .. + 3
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = 4 * (threadIdx.x + k * kNormThreads);
+    on[k] = i < H;
+    if (on[k]) {
+      load4<float>(xr + i, v[k]);
+      load4<TW>(w + i, wv[k]);
+    } else {
+      v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.f;
+    }
+  }
+  if (add) {
+    const TA* ar = add + size_t(src) * H;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (!on[k]) continue;
+      float a[4];
+      load4<TA>(ar + 4 * (threadIdx.x + k * kNormThreads), a);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[k][e] += a[e];
+    }
+  } else if (partials) {
+    const float* pr = partials + size_t(src) * H;
+    float a[VPT][4];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) a[k][0] = a[k][1] = a[k][2] = a[k][3] = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < S; ++s) {
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (!on[k]) continue;
+        float p[4];
+        load4<float>(pr + s * pstride + 4 * (threadIdx.x + k * kNormThreads), p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[k][e] += p[e];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[k][e] += round_to<TO>(a[k][e]);
+  }
+  if ((add || partials) && write_back) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k)
+      if (on[k]) store4<float>(xr + 4 * (threadIdx.x + k * kNormThreads), v[k]);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += v[k][e] * v[k][e];
+  ss = block_sum<kNormThreads>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / float(H) + eps);
+  TO* o = out + size_t(r) * H;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    if (!on[k]) continue;
+    float y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = wv[k][e] * round_to<TO>(v[k][e] * inv);
+    store4<TO>(o + 4 * (threadIdx.x + k * kNormThreads), y);
+  }
+}
+
 // --------------------------------------------------------- rotary positions + cache write
 // One block per token row of the fused [q | k | v] buffer.  q and k heads are rotated in place
 // (pairs (j, j + hd/2), angle = float(pos) * inv_freq[j] in 32-bit); rotated k and plain v are
@@ -101,7 +205,8 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
                                   const float* __restrict__ inv_freq, const int* __restrict__ slots,
                                   T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int hd, int B,
                                   const float* __restrict__ partials, int S) {
-  const int t = blockIdx.x;
+  // one workgroup per (row, head): q heads, then k heads, then v heads
+  const int t = blockIdx.x, h = blockIdx.y;
   T* row = qkv + size_t(t) * row_stride;
   const int half = hd / 2;
   const int width = (nh + 2 * nkv) * hd;
@@ -116,37 +221,38 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
   const int slot = slots ? slots[t] : -1;
   const size_t page = slot >= 0 ? slot / B : 0;
   const int off = slot >= 0 ? slot % B : 0;
-  if (inv_freq) {
-    const float pos = float(positions[t]);
-    const int pairs = (nh + nkv) * half;
-    for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
-      const int h = i / half, j = i % half;
-      float sn, cs;
-      sincosf(pos * inv_freq[j], &sn, &cs);
-      const int c = h * hd + j;
-      const float a = value(c), b = value(c + half);
-      const float ra = a * cs - b * sn, rb = b * cs + a * sn;
-      if (!prow || h < nh) {
-        store_f(row + c, ra);
-        store_f(row + c + half, rb);
+  const bool is_q = h < nh, is_k = !is_q && h < nh + nkv;
+  if (is_q || is_k) {
+    T* cache_row = (is_k && slot >= 0) ? kcache + ((page * nkv + (h - nh)) * B + off) * hd : nullptr;
+    if (inv_freq) {
+      const float pos = float(positions[t]);
+      for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        float sn, cs;
+        sincosf(pos * inv_freq[j], &sn, &cs);
+        const int c = h * hd + j;
+        const float a = value(c), b = value(c + half);
+        const float ra = a * cs - b * sn, rb = b * cs + a * sn;
+        if (!prow || is_q) {
+          store_f(row + c, ra);
+          store_f(row + c + half, rb);
+        }
+        if (cache_row) {
+          store_f(cache_row + j, ra);
+          store_f(cache_row + j + half, rb);
+        }
       }
-      if (slot >= 0 && h >= nh) {
-        T* dst = kcache + ((page * nkv + (h - nh)) * B + off) * hd;
-        store_f(dst + j, ra);
-        store_f(dst + j + half, rb);
+    } else {
+      for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        const float a = value(h * hd + d);
+        if (prow && is_q) store_f(row + h * hd + d, a);
+        if (cache_row) store_f(cache_row + d, a);
       }
     }
-  } else if (prow) {
-    for (int i = threadIdx.x; i < nh * hd; i += blockDim.x) store_f(row + i, value(i));
+    return;
   }
   if (slot < 0) return;
-  const int koff = nh * hd, voff = (nh + nkv) * hd;
-  for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
-    const int h = i / hd, d = i % hd;
-    const size_t dst = ((page * nkv + h) * B + off) * hd + d;
-    if (!inv_freq) store_f(kcache + dst, value(koff + i));
-    store_f(vcache + dst, value(voff + i));
-  }
+  T* cache_row = vcache + ((page * nkv + (h - nh - nkv)) * B + off) * hd;
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) store_f(cache_row + d, value(h * hd + d));
 }
 
 // ---------------------------------------------------------------------------------- SwiGLU
@@ -198,9 +304,23 @@ int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const float* partials
   KVCM_REQUIRE(!(rows && (add || partials) && write_back), "rmsnorm: a gathered add cannot write back");
   KVCM_REQUIRE(!(add && partials), "rmsnorm: the added term is a tensor or partial sums, not both");
   KVCM_REQUIRE(!partials || (S >= 1 && T >= 1), "rmsnorm: partial sums need their split count and row count");
-#define KVCM_NORM(TA, TW, TO)                                                                              \
-  rmsnorm_kernel<TA, TW, TO><<<R, kNormThreads, 0, s>>>(x, static_cast<const TA*>(add), partials, S, T, rows, \
-                                                        static_cast<const TW*>(w), static_cast<TO*>(out), H, eps, write_back)
+  const bool rows4 = H % 4 == 0 && H <= 8 * 1024 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(add) % 16 == 0 && reinterpret_cast<uintptr_t>(partials) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int vpt = (H + 1023) / 1024;
+#define KVCM_NORM4(TA, TW, TO, VPT)                                                                                  \
+  rmsnorm_rows4_kernel<TA, TW, TO, VPT><<<R, kNormThreads, 0, s>>>(x, static_cast<const TA*>(add), partials, S, T, rows, \
+                                                                   static_cast<const TW*>(w), static_cast<TO*>(out), H, eps, write_back)
+#define KVCM_NORM(TA, TW, TO)                                                                                 \
+  do {                                                                                                        \
+    if (!rows4)                                                                                               \
+      rmsnorm_kernel<TA, TW, TO><<<R, kNormThreads, 0, s>>>(x, static_cast<const TA*>(add), partials, S, T, rows, \
+                                                            static_cast<const TW*>(w), static_cast<TO*>(out), H, eps, write_back); \
+    else if (vpt <= 1) KVCM_NORM4(TA, TW, TO, 1);                                                             \
+    else if (vpt <= 2) KVCM_NORM4(TA, TW, TO, 2);                                                             \
+    else if (vpt <= 4) KVCM_NORM4(TA, TW, TO, 4);                                                             \
+    else KVCM_NORM4(TA, TW, TO, 8);                                                                           \
+  } while (0)
   const int key = ((add ? add_dtype : out_dtype) << 2) | (w_dtype << 1) | out_dtype;
   switch (key) {
     case 0b000: KVCM_NORM(float, float, float); break;
@@ -211,6 +331,7 @@ int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const float* partials
     default: KVCM_REQUIRE(false, "rmsnorm: unsupported dtypes add=%d w=%d out=%d", add_dtype, w_dtype, out_dtype);
   }
 #undef KVCM_NORM
+#undef KVCM_NORM4
   return launch_status("rmsnorm");
 }
 
@@ -223,14 +344,15 @@ int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, 
   KVCM_REQUIRE(!slots || (kcache && vcache && B > 0), "rope: cache write without a cache");
   KVCM_REQUIRE(!inv_freq || positions, "rope: rotation without positions");
   KVCM_REQUIRE(!partials || S >= 1, "rope: partial sums need their split count");
-  const int work = (nh + nkv) * hd / 2;
-  const int threads = work >= 256 ? 256 : work >= 128 ? 128 : 64;
+  KVCM_REQUIRE(nh + 2 * nkv <= 65535 && nh + 2 * nkv > 0, "rope: too many heads");
+  const dim3 grid(T, nh + 2 * nkv);
+  const int threads = 64;
   if (dtype == kF32)
-    rope_cache_kernel<float><<<T, threads, 0, s>>>(static_cast<float*>(qkv), row_stride, positions, inv_freq, slots,
+    rope_cache_kernel<float><<<grid, threads, 0, s>>>(static_cast<float*>(qkv), row_stride, positions, inv_freq, slots,
                                                   static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, hd, B,
                                                   partials, S);
   else if (dtype == kBF16)
-    rope_cache_kernel<bf16_t><<<T, threads, 0, s>>>(static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots,
+    rope_cache_kernel<bf16_t><<<grid, threads, 0, s>>>(static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots,
                                                    static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, hd, B,
                                                    partials, S);
   else KVCM_REQUIRE(false, "rope: unknown dtype %d", dtype);

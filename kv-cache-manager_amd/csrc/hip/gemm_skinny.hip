@@ -40,12 +40,10 @@ __global__ void __launch_bounds__(256)
 
   const uint16_t* wrow = W + size_t(n0 + r) * ldw + kq * 16;
   const uint16_t* xrow[MT];
-  bool live[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + r;
-    live[t] = m < M;
-    xrow[t] = X + size_t(live[t] ? m : 0) * ldx + kq * 16;
+    xrow[t] = X + size_t(m < M ? m : 0) * ldx + kq * 16;
   }
   f32x4 acc[MT];
 #pragma unroll
@@ -61,13 +59,14 @@ __global__ void __launch_bounds__(256)
     b[3].u = *reinterpret_cast<const uint4*>(p + kUnit + 8);
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
+      // rows beyond M read row 0 (always there) and are dropped at the store: no branch
+      // around a load, which would make the compiler wait for it on the spot
       Frag a[4];
       const uint16_t* q = xrow[t] + size_t(u) * kUnit;
-      const uint4 zero = {0u, 0u, 0u, 0u};
-      a[0].u = live[t] ? *reinterpret_cast<const uint4*>(q) : zero;
-      a[1].u = live[t] ? *reinterpret_cast<const uint4*>(q + 8) : zero;
-      a[2].u = live[t] ? *reinterpret_cast<const uint4*>(q + kUnit) : zero;
-      a[3].u = live[t] ? *reinterpret_cast<const uint4*>(q + kUnit + 8) : zero;
+      a[0].u = *reinterpret_cast<const uint4*>(q);
+      a[1].u = *reinterpret_cast<const uint4*>(q + 8);
+      a[2].u = *reinterpret_cast<const uint4*>(q + kUnit);
+      a[3].u = *reinterpret_cast<const uint4*>(q + kUnit + 8);
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[i].v, acc[t], 0, 0, 0);
     }
@@ -81,9 +80,8 @@ __global__ void __launch_bounds__(256)
     for (int t = 0; t < MT; ++t) {
       Frag a[2];
       const uint16_t* q = xrow[t] + size_t(u) * kUnit;
-      const uint4 zero = {0u, 0u, 0u, 0u};
-      a[0].u = live[t] ? *reinterpret_cast<const uint4*>(q) : zero;
-      a[1].u = live[t] ? *reinterpret_cast<const uint4*>(q + 8) : zero;
+      a[0].u = *reinterpret_cast<const uint4*>(q);
+      a[1].u = *reinterpret_cast<const uint4*>(q + 8);
 #pragma unroll
       for (int i = 0; i < 2; ++i) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[i].v, acc[t], 0, 0, 0);
     }
