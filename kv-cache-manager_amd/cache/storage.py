@@ -1,7 +1,10 @@
 """Device memory of the cache groups.
 
-A paged group keeps, for each of its layers, keys and values as [pages, kv_heads, block_size,
-head_dim] (the reference's layout, src/cuda/kv_cache.h:1-2), all layers of the group in one
+A paged group keeps, for each of its layers, keys as [pages, kv_heads, block_size, head_dim] (the
+reference's layout, src/cuda/kv_cache.h:1-2) and values transposed inside the page, [pages,
+kv_heads, head_dim, block_size]: eight consecutive tokens of one value dim are then 16 contiguous
+bytes, which is exactly the operand a matrix instruction wants for P*V (the reduction runs over
+tokens), just as eight dims of one token are for Q*K^T.  All layers of the group share one
 allocation; a page id means the same page in every layer of the group.  A state group keeps one
 slot per admitted request and layer.  Memory is zeroed once at construction and never on reuse:
 a reused page holds its previous owner's data beyond the new owner's length, and only the
@@ -21,10 +24,13 @@ class KVStorage:
                                 dtype=dtype, device=device)
 
     def k(self, layer: int) -> torch.Tensor:
+        """[pages, kv_heads, block_size, head_dim]"""
         return self.data[layer, 0]
 
     def v(self, layer: int) -> torch.Tensor:
-        return self.data[layer, 1]
+        """[pages, kv_heads, head_dim, block_size]: the same memory shape, read transposed"""
+        n = self.need
+        return self.data[layer, 1].view(self.num_blocks, n.num_kv_heads, n.head_dim, self.block_size)
 
     @property
     def bytes_per_block(self) -> int:

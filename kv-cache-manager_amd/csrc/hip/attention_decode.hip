@@ -28,12 +28,11 @@ union Frag8 {
 
 // partial results per (row, head, partition): HD floats of o / sum, then max, then sum
 //
-// Scores: each wave takes 16-token tiles; the tile's keys are the B operand of
-// v_mfma_f32_16x16x32_bf16 exactly as they lie in the cache (a lane reads 16 bytes of one token),
-// the group's query heads are the A operand (rows beyond GROUP are zero), so a tile's scores for
-// all heads cost HD/32 matrix instructions and no cross-lane traffic.  P*V: each wave takes a
-// quarter of the partition's tokens, a lane owns HD/64 output dims of every head, values are read
-// one token row per instruction and the probabilities come from LDS as broadcasts; the only
+// Both products run on the matrix cores with the cache's own layouts as the B operand, 16 bytes
+// per lane straight from global memory: for the scores a lane reads 8 dims of one token (keys are
+// [slot][dim]), for P*V it reads 8 tokens of one dim (values are [dim][slot]).  The group's query
+// heads are the rows of the A operand (rows beyond GROUP are zero).  Each wave takes every fourth
+// 16-token tile for the scores and a quarter of the partition's tokens for P*V; the only
 // reduction left is over the four waves.
 template <int HD, int GROUP>
 __global__ void __launch_bounds__(kDecWaves* kWave)
@@ -41,10 +40,10 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
                             const uint16_t* __restrict__ vcache, const int* __restrict__ tables, int table_stride,
                             const int* __restrict__ row_seq, const int* __restrict__ ctx_lens, int nh, int nkv, int B,
                             float scale, int num_parts, float* __restrict__ scratch) {
-  constexpr int KSTEPS = HD / 32;                    // matrix instructions per 16-token tile
-  constexpr int TILES = kDecPart / 16 / kDecWaves;   // tiles per wave
-  constexpr int DPL = HD / kWave;                    // output dims per lane in P*V
-  constexpr int TOKW = kDecPart / kDecWaves;         // tokens per wave in P*V
+  constexpr int KSTEPS = HD / 32;                    // matrix instructions per 16-token tile of scores
+  constexpr int TILES = kDecPart / 16 / kDecWaves;   // score tiles per wave
+  constexpr int DT = HD / 16;                        // 16-dim tiles of the output
+  constexpr int VSTEPS = kDecPart / 32 / kDecWaves;  // 32-token steps of P*V per wave
   const int kvh = blockIdx.x, row = blockIdx.y, part = blockIdx.z;
   const int ctx = ctx_lens[row];
   const int start = part * kDecPart;
@@ -53,44 +52,48 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
 
   __shared__ __attribute__((aligned(16))) float scores[GROUP][kDecPart];
-  __shared__ float red[kDecWaves][GROUP][HD];
+  __shared__ __attribute__((aligned(16))) float red[kDecWaves][16][HD + 4];
   __shared__ float s_max[GROUP], s_sum[GROUP];
 
   const int* table = tables + size_t(row_seq[row]) * table_stride;
-  const size_t head_stride = size_t(B) * HD, page_stride = head_stride * nkv;
+  const size_t head_elems = size_t(B) * HD, page_elems = head_elems * nkv;
 
-  // where each token of the partition lives: one table lookup per thread, shared through LDS
-  // (page id and slot in the page), instead of a chain of dependent lookups per load below
-  // Tokens beyond the context point at the last valid token: every load below is then
-  // unconditional (a branch around a load makes the compiler wait for it at once), and what
-  // is loaded for them is never used (no score is stored, their probability is zero).
-  // The offset of a token's row inside this kv head's part of the cache, in units of 8 elements.
-  __shared__ uint32_t where[kDecPart];
+  // Where each token of the partition lives, one table lookup per thread, shared through LDS:
+  // for keys the offset of the token's row, for values the offset of the token's slot in dim 0,
+  // both inside this kv head's part of the cache and in units of 8 elements.  Tokens beyond the
+  // context point at the last valid token (keys) or the last valid group of 8 (values), so that
+  // every load below is unconditional (a branch around a load makes the compiler wait for it at
+  // once); what is loaded for them is never used: no score is stored, their probability is zero.
+  __shared__ uint32_t where_k[kDecPart];
+  __shared__ uint32_t where_v[kDecPart / 8];
   {
     const int t = min(start + int(threadIdx.x), end - 1);
-    where[threadIdx.x] = uint32_t((size_t(table[t / B]) * page_stride + kvh * head_stride + size_t(t % B) * HD) / 8);
+    const size_t head0 = size_t(table[t / B]) * page_elems + kvh * head_elems;
+    where_k[threadIdx.x] = uint32_t((head0 + size_t(t % B) * HD) / 8);
+    if (threadIdx.x % 8 == 0) {
+      const int tv = min(start + int(threadIdx.x), (end - 1) & ~7);
+      where_v[threadIdx.x / 8] = uint32_t((size_t(table[tv / B]) * page_elems + kvh * head_elems + tv % B) / 8);
+    }
   }
   __syncthreads();
 
-  // ---- requests first: this wave's keys (tile layout) and values (one token row per load)
+  // ---- requests first: this wave's keys and values
   const int n16 = lane % 16, kq = lane / 16;
   Frag8 kf[TILES][KSTEPS];
 #pragma unroll
   for (int i = 0; i < TILES; ++i) {
     const int tok = (wave + i * kDecWaves) * 16 + n16;
-    const uint16_t* kp = kcache + (size_t(where[tok]) << 3) + kq * 8;
+    const uint16_t* kp = kcache + (size_t(where_k[tok]) << 3) + kq * 8;
 #pragma unroll
     for (int c = 0; c < KSTEPS; ++c) kf[i][c].u = *reinterpret_cast<const uint4*>(kp + c * 32);
   }
-  static_assert(TOKW == kWave, "one lane per token of the wave's quarter");
-  const uint32_t my_where = where[wave * TOKW + lane];
-  uint32_t vraw[TOKW];
+  Frag8 vf[VSTEPS][DT];
 #pragma unroll
-  for (int i = 0; i < TOKW; ++i) {
-    const uint32_t w = __builtin_amdgcn_readlane(my_where, i);   // token i of the quarter, the same for every lane
-    const uint16_t* vp = vcache + (size_t(w) << 3) + lane * DPL;
-    if constexpr (DPL == 1) vraw[i] = *vp;
-    else vraw[i] = *reinterpret_cast<const uint32_t*>(vp);
+  for (int j = 0; j < VSTEPS; ++j) {
+    const int tok8 = (wave * VSTEPS + j) * 4 + kq;      // which group of 8 tokens this lane reads
+    const uint16_t* vp = vcache + (size_t(where_v[tok8]) << 3) + size_t(n16) * B;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) vf[j][d].u = *reinterpret_cast<const uint4*>(vp + size_t(d) * 16 * B);
   }
   Frag8 qf[KSTEPS];
   const int qhead = kvh * GROUP + (n16 < GROUP ? n16 : 0);
@@ -137,34 +140,30 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
   }
   __syncthreads();
 
-  // ---- pass 3: P * V, lane owns dims lane*DPL .. +DPL-1 of every head
-  float acc[GROUP][DPL];
+  // ---- pass 3: out[head][dim] += P[head][token] * V[token][dim]; P rounded to bfloat16 as the A operand
+  f32x4 o[DT];
 #pragma unroll
-  for (int g = 0; g < GROUP; ++g)
+  for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int e = 0; e < DPL; ++e) acc[g][e] = 0.f;
-#pragma unroll
-  for (int i = 0; i < TOKW; i += 4) {
-    float4 p[GROUP];
-#pragma unroll
-    for (int g = 0; g < GROUP; ++g) p[g] = *reinterpret_cast<const float4*>(&scores[g][wave * TOKW + i]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float vf[DPL];
-      vf[0] = bf16_bits_to_float(vraw[i + j] & 0xffffu);
-      if constexpr (DPL == 2) vf[1] = bf16_bits_to_float(vraw[i + j] >> 16);
-#pragma unroll
-      for (int g = 0; g < GROUP; ++g) {
-        const float w = j == 0 ? p[g].x : j == 1 ? p[g].y : j == 2 ? p[g].z : p[g].w;
-#pragma unroll
-        for (int e = 0; e < DPL; ++e) acc[g][e] = fmaf(w, vf[e], acc[g][e]);
-      }
+  for (int j = 0; j < VSTEPS; ++j) {
+    Frag8 pf;
+    pf.u = uint4{0u, 0u, 0u, 0u};
+    if (n16 < GROUP) {
+      const float* pr = &scores[n16][(wave * VSTEPS + j) * 32 + kq * 8];
+      const float4 a = *reinterpret_cast<const float4*>(pr), b = *reinterpret_cast<const float4*>(pr + 4);
+      pf.u.x = float_to_bf16_bits(a.x) | (uint32_t(float_to_bf16_bits(a.y)) << 16);
+      pf.u.y = float_to_bf16_bits(a.z) | (uint32_t(float_to_bf16_bits(a.w)) << 16);
+      pf.u.z = float_to_bf16_bits(b.x) | (uint32_t(float_to_bf16_bits(b.y)) << 16);
+      pf.u.w = float_to_bf16_bits(b.z) | (uint32_t(float_to_bf16_bits(b.w)) << 16);
     }
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf[j][d].v, o[d], 0, 0, 0);
   }
+  // accumulator: column = dim n16 of tile d, rows = heads 4*kq..+3
 #pragma unroll
-  for (int g = 0; g < GROUP; ++g)
+  for (int d = 0; d < DT; ++d)
 #pragma unroll
-    for (int e = 0; e < DPL; ++e) red[wave][g][lane * DPL + e] = acc[g][e];
+    for (int r = 0; r < 4; ++r) red[wave][kq * 4 + r][d * 16 + n16] = o[d][r];
   __syncthreads();
   for (int i = threadIdx.x; i < GROUP * HD; i += kDecWaves * kWave) {
     const int g = i / HD, d = i % HD;
@@ -231,8 +230,8 @@ using namespace kvcm;
 extern "C" {
 
 // 1 when this kernel takes the shape (bfloat16 only), else 0 (use the generic kernel).
-int kvcm_attention_decode_supported(int nh, int nkv, int hd) {
-  if (nkv <= 0 || nh % nkv) return 0;
+int kvcm_attention_decode_supported(int nh, int nkv, int hd, int B) {
+  if (nkv <= 0 || nh % nkv || B <= 0 || B % 8) return 0;
   const int g = nh / nkv;
   return (hd == 64 || hd == 128) && g >= 1 && g <= 8;
 }
@@ -250,8 +249,9 @@ int kvcm_attention_decode(const void* q, int q_stride, void* out, int out_stride
                           const int* ctx_lens, int T, int nh, int nkv, int hd, int B, float scale, int max_context,
                           float* scratch, long long scratch_floats, hipStream_t s) {
   if (T == 0) return 0;
-  KVCM_REQUIRE(kvcm_attention_decode_supported(nh, nkv, hd), "attention_decode: unsupported shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
+  KVCM_REQUIRE(kvcm_attention_decode_supported(nh, nkv, hd, B), "attention_decode: unsupported shape heads=%d kv_heads=%d head_dim=%d page=%d", nh, nkv, hd, B);
   KVCM_REQUIRE(T > 0 && B > 0 && max_context > 0, "attention_decode: bad sizes T=%d B=%d max_context=%d", T, B, max_context);
+  KVCM_REQUIRE(B % 8 == 0, "attention_decode: the page size %d is not a multiple of 8", B);
   KVCM_REQUIRE(q_stride >= nh * hd && out_stride >= nh * hd && q_stride % 8 == 0, "attention_decode: bad row strides");
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(vcache) % 16 == 0, "attention_decode: operands must be 16-byte aligned");

@@ -100,11 +100,11 @@ __global__ void __launch_bounds__(kAttnWaves* kWave)
     for (int j = j_lo; j < j_hi; ++j) {
       const float pj = __shfl(p, j, kWave);
       const int tj = c0 + j;
-      const T* vp = vcache + size_t(table[tj / B]) * page_stride + kvh * head_stride + size_t(tj % B) * hd;
+      const T* vp = vcache + size_t(table[tj / B]) * page_stride + kvh * head_stride + tj % B;  // [dim][slot]
 #pragma unroll
       for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
         const int d = lane + i * kWave;
-        if (d < hd) o[i] = fmaf(pj, load_f(vp + d), o[i]);
+        if (d < hd) o[i] = fmaf(pj, load_f(vp + size_t(d) * B), o[i]);
       }
     }
     m = m_new;

@@ -195,7 +195,8 @@ __global__ void __launch_bounds__(kNormThreads)
 // --------------------------------------------------------- rotary positions + cache write
 // One block per token row of the fused [q | k | v] buffer.  q and k heads are rotated in place
 // (pairs (j, j + hd/2), angle = float(pos) * inv_freq[j] in 32-bit); rotated k and plain v are
-// copied to the paged cache at slot = page * B + offset, layout [page][kv_head][B][hd].
+// copied to the paged cache at slot = page * B + offset; keys [page][kv_head][B][hd], values
+// transposed inside the page [page][kv_head][hd][B].
 // inv_freq == null: no rotation.  slots == null or slot < 0: no cache write.
 // partials != null: the fused rows do not exist yet; they are the split-K sums [S][rows][width]
 // of the projection that makes them (added in split order, rounded to the storage type), and only
@@ -251,8 +252,9 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
     return;
   }
   if (slot < 0) return;
-  T* cache_row = vcache + ((page * nkv + (h - nh - nkv)) * B + off) * hd;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) store_f(cache_row + d, value(h * hd + d));
+  // values are stored transposed inside the page: [page][kv_head][dim][slot]
+  T* cache_head = vcache + (page * nkv + (h - nh - nkv)) * size_t(hd) * B + off;
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) store_f(cache_head + size_t(d) * B, value(h * hd + d));
 }
 
 // ---------------------------------------------------------------------------------- SwiGLU

@@ -162,7 +162,7 @@ class ModelRunner:
         ops = self.ops
         partitioned = (self.attn != "v1" and window == 0 and step.max_run == 1
                        and step.rows <= self.DECODE_ATTENTION_MAX_ROWS
-                       and ops.attention_decode_supported(nh, nkv, hd, q.dtype))
+                       and ops.attention_decode_supported(nh, nkv, hd, q.dtype, kcache.shape[2]))
         if self.attn == "v2" and not partitioned and q.dtype == torch.bfloat16 and step.max_run == 1:
             raise RuntimeError(f"attn=v2: the partitioned kernel does not take heads={nh} kv_heads={nkv} "
                                f"head_dim={hd} window={window} rows={step.rows}")

@@ -41,7 +41,7 @@ def _declare(lib):
     fn("kvcm_gemm_bf16", vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_attention_generic", vp, i, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp)
     fn("kvcm_sample", vp, i, vp, vp, vp, vp, vp, i, i, vp)
-    fn("kvcm_attention_decode_supported", i, i, i)
+    fn("kvcm_attention_decode_supported", i, i, i, i)
     lib.kvcm_attention_decode_scratch.restype = C.c_longlong
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
@@ -169,9 +169,10 @@ def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcac
         _need(positions is not None, "rotation needs positions")
     if slots is not None:
         _i32(slots, "slots", T)
-        for c in (kcache, vcache):
-            _need(c is not None and c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
-                  and tuple(c.shape[1:]) == (nkv, block_size, hd), "cache must be [pages, nkv, block_size, hd]")
+        _need(kcache is not None and kcache.dtype == qkv.dtype and kcache.is_contiguous() and kcache.dim() == 4
+              and tuple(kcache.shape[1:]) == (nkv, block_size, hd), "key cache must be [pages, nkv, block_size, hd]")
+        _need(vcache is not None and vcache.dtype == qkv.dtype and vcache.is_contiguous() and vcache.dim() == 4
+              and tuple(vcache.shape[1:]) == (nkv, hd, block_size), "value cache must be [pages, nkv, hd, block_size]")
     _check(lib().kvcm_rope_cache(_ptr(qkv), _DT[qkv.dtype], qkv.stride(0), _ptr(positions), _ptr(inv_freq),
                                  _ptr(slots), _ptr(kcache), _ptr(vcache), T, nh, nkv, hd, block_size,
                                  _ptr(source.data) if source is not None else 0,
@@ -243,6 +244,13 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
     return out
 
 
+def _check_caches(kcache, vcache, nkv, hd):
+    _need(kcache.dim() == 4 and kcache.is_contiguous() and kcache.shape[1] == nkv and kcache.shape[3] == hd,
+          "key cache must be [pages, nkv, block_size, hd]")
+    _need(vcache.dim() == 4 and vcache.is_contiguous() and tuple(vcache.shape) == (kcache.shape[0], nkv, hd, kcache.shape[2]),
+          "value cache must be [pages, nkv, hd, block_size]")
+
+
 def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, nh, nkv, hd, scale, window=0,
               rows=None):
     """out[r, h, :] = softmax(scale * q[r, h] . K[0:ctx_r]) V[0:ctx_r] over the paged cache."""
@@ -251,8 +259,7 @@ def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, n
     _rows2d(out, "out")
     T = q.shape[0] if rows is None else rows
     _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype, "attention operands must share one dtype")
-    _need(kcache.dim() == 4 and kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape == vcache.shape
-          and kcache.shape[1] == nkv and kcache.shape[3] == hd, "cache must be [pages, nkv, block_size, hd]")
+    _check_caches(kcache, vcache, nkv, hd)
     _i32(row_seq, "row_seq", T)
     _i32(ctx_lens, "ctx_lens", T)
     _i32(tables, "tables")
@@ -261,8 +268,8 @@ def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, n
                                         nkv, hd, kcache.shape[2], float(scale), int(window), _stream()))
 
 
-def attention_decode_supported(nh, nkv, hd, dtype):
-    return dtype == torch.bfloat16 and bool(lib().kvcm_attention_decode_supported(nh, nkv, hd))
+def attention_decode_supported(nh, nkv, hd, dtype, block_size=16):
+    return dtype == torch.bfloat16 and bool(lib().kvcm_attention_decode_supported(nh, nkv, hd, block_size))
 
 
 def attention_decode_scratch(rows, nh, hd, max_context):
@@ -278,8 +285,7 @@ def attention_decode(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_
     _rows2d(out, "out")
     T = q.shape[0] if rows is None else rows
     _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "attention_decode is bfloat16 only")
-    _need(kcache.dim() == 4 and kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape == vcache.shape
-          and kcache.shape[1] == nkv and kcache.shape[3] == hd, "cache must be [pages, nkv, block_size, hd]")
+    _check_caches(kcache, vcache, nkv, hd)
     _need(scratch.dtype == torch.float32 and scratch.is_contiguous(), "scratch must be contiguous float32")
     _i32(row_seq, "row_seq", T)
     _i32(ctx_lens, "ctx_lens", T)

@@ -29,6 +29,12 @@ def _np(t):
     return t.detach().float().cpu().numpy().astype(np.float64)
 
 
+def _vt(vc, dtype):
+    """A value cache built as [pages, kv_heads, slot, dim] in the layout the kernels read:
+    [pages, kv_heads, dim, slot]."""
+    return torch.tensor(np.ascontiguousarray(np.asarray(vc).transpose(0, 1, 3, 2)), dtype=dtype, device=DEV)
+
+
 def _bf16_grid(a):
     return plain.round_bf16(a)
 
@@ -156,10 +162,10 @@ def test_reshape_and_cache_scatters_to_slots(ops, dtype):
     natural = slots[skipped]
     slots[skipped] = -1
     kc = torch.zeros(NB, KVH, B, HD, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(NB, KVH, HD, B, dtype=dtype, device=DEV)        # values lie transposed inside a page
     buf = _t(rows, dtype)
     ops.rope_cache(buf[:, :stride], NH, KVH, HD, slots=_t(slots, torch.int32), kcache=kc, vcache=vc, block_size=B)
-    K, V = _np(kc), _np(vc)
+    K, V = _np(kc), _np(vc).transpose(0, 1, 3, 2)
     for t in range(T):
         k_src = rows[t, NH * HD:(NH + KVH) * HD].reshape(KVH, HD)
         v_src = rows[t, (NH + KVH) * HD:(NH + 2 * KVH) * HD].reshape(KVH, HD)
@@ -178,12 +184,12 @@ def test_fused_rope_and_cache_write_stores_rotated_keys(ops):
     pos = np.array([3, 4, 5, 40, 41], dtype=np.int32)
     slots = np.array([8, 9, 10, 0, 1], dtype=np.int32)
     kc = torch.zeros(3, KVH, B, HD, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(3, KVH, HD, B, device=DEV)
     buf = _t(rows, torch.float32)
     ops.rope_cache(buf, NH, KVH, HD, positions=_t(pos, torch.int32), inv_freq=_t(_inv_freq(HD, 1e4), torch.float32),
                    slots=_t(slots, torch.int32), kcache=kc, vcache=vc, block_size=B)
     k_ref = plain.rotary(rows[:, NH * HD:(NH + KVH) * HD].reshape(T, KVH, HD), pos, 1e4)
-    K, V = _np(kc), _np(vc)
+    K, V = _np(kc), _np(vc).transpose(0, 1, 3, 2)
     for t in range(T):
         np.testing.assert_allclose(K[slots[t] // B, :, slots[t] % B], k_ref[t], atol=1e-5)
         np.testing.assert_array_equal(V[slots[t] // B, :, slots[t] % B],
@@ -314,7 +320,7 @@ def _paged_problem(rng, ctx_lens, nh, nkv, hd, B, all_rows, shuffle=True, spare=
 
 def _run_attention(ops, P, nh, nkv, hd, dtype, window=0, scale=None):
     out = torch.zeros(P["R"], nh * hd, dtype=dtype, device=DEV)
-    ops.attention(_t(P["Q"].reshape(P["R"], nh * hd), dtype), out, _t(P["Kc"], dtype), _t(P["Vc"], dtype),
+    ops.attention(_t(P["Q"].reshape(P["R"], nh * hd), dtype), out, _t(P["Kc"], dtype), _vt(P["Vc"], dtype),
                   _t(P["tables"], torch.int32), P["max_blocks"], _t(P["row_seq"], torch.int32), _t(P["ctx"], torch.int32),
                   nh, nkv, hd, scale if scale is not None else 1.0 / math.sqrt(hd), window)
     return _np(out).reshape(P["R"], nh, hd)
@@ -540,7 +546,8 @@ def test_partial_sums_feed_the_fused_norm_and_rope(ops):
     pos = _t([0, 5, 17, 100, 101], torch.int32)
     slots = _t([3, 20, 35, 1, 16], torch.int32)
     inv = _t(_inv_freq(hd, 1e4), torch.float32)
-    caches = [torch.zeros(3, nkv, B, hd, dtype=torch.bfloat16, device=DEV) for _ in range(4)]
+    caches = [torch.zeros(3, nkv, B, hd, dtype=torch.bfloat16, device=DEV) if i % 2 == 0 else
+              torch.zeros(3, nkv, hd, B, dtype=torch.bfloat16, device=DEV) for i in range(4)]
     rows_a = prod.clone()
     ops.rope_cache(rows_a, nh, nkv, hd, positions=pos, inv_freq=inv, slots=slots, kcache=caches[0], vcache=caches[1], block_size=B)
     rows_b = torch.zeros_like(rows_a)
@@ -563,7 +570,7 @@ def test_partitioned_decode_attention(ops, nh, nkv, hd, B):
         out = torch.zeros(R, nh * hd, dtype=torch.bfloat16, device=DEV)
         scratch = torch.zeros(ops.attention_decode_scratch(R, nh, hd, bound), dtype=torch.float32, device=DEV)
         ops.attention_decode(_t(P["Q"].reshape(R, nh * hd), torch.bfloat16), out, _t(P["Kc"], torch.bfloat16),
-                             _t(P["Vc"], torch.bfloat16), _t(P["tables"], torch.int32), P["max_blocks"],
+                             _vt(P["Vc"], torch.bfloat16), _t(P["tables"], torch.int32), P["max_blocks"],
                              _t(P["row_seq"], torch.int32), _t(P["ctx"], torch.int32), nh, nkv, hd, 1.0 / math.sqrt(hd),
                              bound, scratch)
         np.testing.assert_allclose(_np(out).reshape(R, nh, hd), ref, atol=1e-2, rtol=0)
@@ -586,15 +593,16 @@ def test_partitioned_decode_attention_padding_rows_and_far_key(ops):
     q = np.concatenate([P["Q"].reshape(2, nh * hd), np.ones((1, nh * hd))])
     out = torch.full((3, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
     scratch = torch.zeros(ops.attention_decode_scratch(3, nh, hd, 1024), dtype=torch.float32, device=DEV)
-    ops.attention_decode(_t(q, torch.bfloat16), out, _t(P["Kc"], torch.bfloat16), _t(P["Vc"], torch.bfloat16),
+    ops.attention_decode(_t(q, torch.bfloat16), out, _t(P["Kc"], torch.bfloat16), _vt(P["Vc"], torch.bfloat16),
                          _t(P["tables"], torch.int32), P["max_blocks"], _t([0, 1, 0], torch.int32), _t(ctx, torch.int32),
                          nh, nkv, hd, 1.0, 1024, scratch)
     got = _np(out).reshape(3, nh, hd)
     np.testing.assert_allclose(got[0, 5], P["Vl"][0][far, 1], atol=1e-2)
     assert not got[2].any()
     with pytest.raises(ops.KernelError, match="scratch too small"):
-        ops.attention_decode(_t(q, torch.bfloat16), out, _t(P["Kc"], torch.bfloat16), _t(P["Vc"], torch.bfloat16),
+        ops.attention_decode(_t(q, torch.bfloat16), out, _t(P["Kc"], torch.bfloat16), _vt(P["Vc"], torch.bfloat16),
                              _t(P["tables"], torch.int32), P["max_blocks"], _t([0, 1, 0], torch.int32), _t(ctx, torch.int32),
                              nh, nkv, hd, 1.0, 4096, scratch)
     assert not ops.attention_decode_supported(12, 1, 64, torch.bfloat16) and not ops.attention_decode_supported(4, 2, 48, torch.bfloat16)
+    assert not ops.attention_decode_supported(32, 4, 64, torch.bfloat16, block_size=4)
     assert not ops.attention_decode_supported(32, 4, 64, torch.float32)
