@@ -156,9 +156,11 @@ class ModelRunner:
     DECODE_ATTENTION_MAX_ROWS = 512
 
     def attention(self, step, q, out, kcache, vcache, g, nh, nkv, hd, scale, window):
-        """attn = "v1": one pass over the whole context per (row, head); "v2": contexts cut into
-        partitions and merged (bfloat16, decode-shaped steps); "auto": v2 where it applies.  The
-        32-bit path always takes v1, whose result does not depend on the batch."""
+        """attn = "v1": the generic kernel, one pass over the whole context per (row, head); "v2" and
+        "auto": for bfloat16, decode-shaped steps take the kernel that cuts contexts into partitions
+        and merges them, steps with runs of positions take the tiled kernel; "v2" insists on the
+        partitioned kernel for decode steps.  The 32-bit path always takes v1, whose result does
+        not depend on the batch."""
         ops = self.ops
         partitioned = (self.attn != "v1" and window == 0 and step.max_run == 1
                        and step.rows <= self.DECODE_ATTENTION_MAX_ROWS
@@ -173,6 +175,12 @@ class ModelRunner:
                 min(self.DECODE_ATTENTION_MAX_ROWS, self.limits.max_tokens), nh, hd, self.limits.max_context_len)))
             ops.attention_decode(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
                                  step.ctx_lens, nh, nkv, hd, scale, bound, scratch, rows=step.rows)
+            return
+        if (self.attn != "v1" and window == 0 and step.max_run > 1
+                and ops.attention_prefill_supported(nh, nkv, hd, q.dtype, kcache.shape[2])):
+            # runs of consecutive positions: keys are read once per 64 query rows, on the matrix cores
+            ops.attention_prefill(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.run_start,
+                                  step.seq_start, step.real_seqs, step.max_run, nh, nkv, hd, scale)
             return
         ops.attention(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
                       step.ctx_lens, nh, nkv, hd, scale, window, rows=step.rows)

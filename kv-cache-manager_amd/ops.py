@@ -42,6 +42,8 @@ def _declare(lib):
     fn("kvcm_attention_generic", vp, i, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp)
     fn("kvcm_sample", vp, i, vp, vp, vp, vp, vp, i, i, vp)
     fn("kvcm_attention_decode_supported", i, i, i, i)
+    fn("kvcm_attention_prefill_supported", i, i, i, i)
+    fn("kvcm_attention_prefill", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, i, f, vp)
     lib.kvcm_attention_decode_scratch.restype = C.c_longlong
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
@@ -294,6 +296,28 @@ def attention_decode(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_
                                        _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh, nkv, hd,
                                        kcache.shape[2], float(scale), int(max_context), _ptr(scratch), scratch.numel(),
                                        _stream()))
+
+
+def attention_prefill_supported(nh, nkv, hd, dtype, block_size=16):
+    return dtype == torch.bfloat16 and bool(lib().kvcm_attention_prefill_supported(nh, nkv, hd, block_size))
+
+
+def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, seq_start, num_seqs, max_run, nh, nkv, hd,
+                      scale):
+    """Causal attention for runs of consecutive positions (bfloat16): sequence s owns rows
+    run_start[s] .. run_start[s+1]-1, the first of them at position seq_start[s]; every row sees the
+    sequence's cached tokens up to its own position.  The same result as ``attention``."""
+    _dev(q, out, kcache, vcache, tables, run_start, seq_start)
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "attention_prefill is bfloat16 only")
+    _check_caches(kcache, vcache, nkv, hd)
+    _i32(run_start, "run_start", num_seqs + 1)
+    _i32(seq_start, "seq_start", num_seqs)
+    _i32(tables, "tables", num_seqs * table_stride)
+    _check(lib().kvcm_attention_prefill(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
+                                        _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), num_seqs, max_run,
+                                        nh, nkv, hd, kcache.shape[2], float(scale), _stream()))
 
 
 def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_index=None):

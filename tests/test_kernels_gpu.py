@@ -606,3 +606,75 @@ def test_partitioned_decode_attention_padding_rows_and_far_key(ops):
     assert not ops.attention_decode_supported(12, 1, 64, torch.bfloat16) and not ops.attention_decode_supported(4, 2, 48, torch.bfloat16)
     assert not ops.attention_decode_supported(32, 4, 64, torch.bfloat16, block_size=4)
     assert not ops.attention_decode_supported(32, 4, 64, torch.float32)
+
+
+# ------------------------------------------------------------------- tiled prefill attention
+def _run_prefill(ops, P, runs, nh, nkv, hd, scale=None):
+    """runs: per sequence (first position, number of rows); rows of P are those positions in order."""
+    R = P["R"]
+    out = torch.full((R, nh * hd), 3.0, dtype=torch.bfloat16, device=DEV)
+    run_start = np.concatenate([[0], np.cumsum([n for _, n in runs])]).astype(np.int32)
+    ops.attention_prefill(_t(P["Q"].reshape(R, nh * hd), torch.bfloat16), out, _t(P["Kc"], torch.bfloat16),
+                          _vt(P["Vc"], torch.bfloat16), _t(P["tables"], torch.int32), P["max_blocks"], _t(run_start, torch.int32),
+                          _t([s for s, _ in runs], torch.int32), len(runs), max(n for _, n in runs), nh, nkv, hd,
+                          scale if scale is not None else 1.0 / math.sqrt(hd))
+    return _np(out).reshape(R, nh, hd)
+
+
+def _runs_problem(rng, runs, nh, nkv, hd, B):
+    """Sequences whose cache holds start+n tokens; query rows are positions start .. start+n-1."""
+    P = _paged_problem(rng, [s + n for s, n in runs], nh, nkv, hd, B, all_rows=True)
+    keep, row = [], 0
+    for s, n in runs:
+        keep += list(range(row + s, row + s + n))
+        row += s + n
+    P["Q"], P["row_seq"], P["ctx"], P["R"] = P["Q"][keep], P["row_seq"][keep], P["ctx"][keep], len(keep)
+    return P
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (4, 4, 128), (6, 1, 64), (32, 4, 64)])
+@pytest.mark.parametrize("B", [8, 16, 64])
+def test_prefill_attention_runs_anywhere(ops, nh, nkv, hd, B):
+    rng = np.random.default_rng(nh + hd + B)
+    runs = [(0, 130), (0, 1), (77, 2), (200, 1), (15, 64), (63, 65), (0, 16), (31, 17)]
+    P = _runs_problem(rng, runs, nh, nkv, hd, B)
+    got = _run_prefill(ops, P, runs, nh, nkv, hd)
+    ref = _ref_attention(P, nh, nkv, hd)
+    np.testing.assert_allclose(got, ref, atol=1.5e-2, rtol=0)
+    generic = _run_attention(ops, P, nh, nkv, hd, torch.bfloat16)
+    np.testing.assert_allclose(got, generic, atol=2e-2, rtol=0)
+
+
+def test_prefill_attention_is_causal_at_tile_and_page_edges(ops):
+    """A huge key at position t must be seen by rows t, t+1, .. and by no row before it."""
+    rng = np.random.default_rng(50)
+    nh, nkv, hd, B = 4, 2, 64, 16
+    runs = [(0, 200)]
+    for t in (0, 15, 16, 63, 64, 65, 127, 128, 199):
+        P = _runs_problem(rng, runs, nh, nkv, hd, B)
+        P["Q"][:, 1] = 0.0
+        P["Q"][:, 1, 9] = 30.0
+        kvec = np.zeros(hd)
+        kvec[9] = 30.0
+        P["Kl"][0][t, 0] = kvec
+        P["Kc"][P["tables"][0, t // B], 0, t % B] = kvec
+        got = _run_prefill(ops, P, runs, nh, nkv, hd, scale=1.0)
+        np.testing.assert_allclose(got[t:, 1], np.broadcast_to(P["Vl"][0][t, 0], got[t:, 1].shape), atol=2e-2)
+        if t > 0:
+            ref = _ref_attention(P, nh, nkv, hd, scale=1.0)
+            np.testing.assert_allclose(got[:t, 1], ref[:t, 1], atol=2e-2)
+            assert np.abs(got[t - 1, 1] - P["Vl"][0][t, 0]).max() > 0.1
+
+
+def test_prefill_attention_long_prompt(ops):
+    rng = np.random.default_rng(51)
+    nh, nkv, hd, B = 8, 2, 64, 16
+    runs = [(0, 1500), (1000, 300)]
+    P = _runs_problem(rng, runs, nh, nkv, hd, B)
+    got = _run_prefill(ops, P, runs, nh, nkv, hd)
+    rows = [0, 1, 63, 64, 700, 1499, 1500, 1799]
+    ref = np.zeros((len(rows), nh, hd))
+    for k, r in enumerate(rows):
+        s, c = P["row_seq"][r], P["ctx"][r]
+        ref[k] = plain.attention(P["Q"][r:r + 1], P["Kl"][s][:c], P["Vl"][s][:c], [c - 1], np.arange(c), 1.0 / math.sqrt(hd))[0]
+    np.testing.assert_allclose(got[rows], ref, atol=1e-2, rtol=0)
