@@ -2,15 +2,24 @@
 // sequence (a whole prompt, or a portion that starts anywhere) against every key the sequence has
 // in the cache, its own included.  The reference runs its decode kernel row by row for this
 // (src/cuda/paged_attention.cu:50-183, docs/design.md:113-114): every row re-reads all its keys.
-// Here a workgroup takes 64 query rows of one head, each of its four waves 16 of them, and walks
-// the keys 64 at a time with a running maximum (no score buffer), so keys are read once per 64
-// rows; Q*K^T and P*V run on the matrix cores (v_mfma_f32_16x16x32_bf16) with the cache's own
-// layouts as B operands, 16 bytes per lane straight from global memory: keys [slot][dim] give 8
-// dims of one token, values [dim][slot] give 8 tokens of one dim.  Probabilities pass through LDS
-// once, as bfloat16, to change from the accumulator layout to the A-operand layout.
+//
+// Here a workgroup takes 128 query rows of one head, each of its four waves 32 of them (two
+// 16-row tiles), and walks the keys 64 at a time with a running maximum (no score buffer).  A
+// chunk of keys and values is staged in LDS once per workgroup, double-buffered: the next chunk's
+// global loads are in flight while the current one is multiplied.
+//
+// Both products run on the matrix cores (v_mfma_f32_16x16x32_bf16), transposed:
+//   S^T[token][row] = K[token][dim] * Q^T[dim][row]      A = keys as they lie ([slot][dim]),  B = Q
+//   O^T[dim][row]  += V^T[dim][token] * P^T[token][row]  A = values as they lie ([dim][slot]), B = P
+// In the accumulator of S^T a lane holds, for ONE query row (lane % 16), four tokens of each
+// 16-token tile; after exp those registers, rounded to bfloat16 and packed, ARE the B operand of
+// the second product (the order of the reduction index inside a matrix instruction is free as long
+// as both operands agree, so the values are read from LDS in that same token order).  The
+// probabilities never touch LDS, a row's maximum and sum live in one lane each, and the output is
+// stored four dims at a time.
 //
 // The only mask is causal: a row at position p sees tokens t <= p.  Rows of different sequences
-// never share a workgroup.  Head sizes 64 and 128, pages that hold a multiple of 8 tokens.
+// never share a workgroup.  Head sizes 64 and 128; pages of 8, 16, 32, ... tokens (a power of two).
 #include <cfloat>
 
 #include "common.h"
@@ -19,40 +28,52 @@ namespace kvcm {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 union PFrag {
   uint4 u;
+  uint2 h[2];
   bf16x8 v;
 };
 
 constexpr int kPfWaves = 4;
-constexpr int kPfRows = 16 * kPfWaves;  // query rows per workgroup
-constexpr int kPfChunk = 64;            // keys per trip
-constexpr int kPfPitch = kPfChunk + 8;  // LDS row pitch of the probability tile, in bfloat16
+constexpr int kPfThreads = kPfWaves * kWave;
+constexpr int kPfRT = 2;                         // 16-row tiles per wave
+constexpr int kPfWaveRows = 16 * kPfRT;
+constexpr int kPfRows = kPfWaveRows * kPfWaves;  // query rows per workgroup
+constexpr int kPfChunk = 64;                     // keys per trip
+constexpr int kPfPad = 8;                        // bfloat16 of padding per LDS row (keeps 16-byte alignment)
 
-__device__ __forceinline__ float row16_max(float v) {
-#pragma unroll
-  for (int o = 1; o < 16; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-  return v;
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  union { bf16x2_t v; uint32_t u; } r;
+  r.v = __builtin_convertvector(float2_t{a, b}, bf16x2_t);   // one v_cvt_pk_bf16_f32
+  return r.u;
 }
-__device__ __forceinline__ float row16_sum(float v) {
-#pragma unroll
-  for (int o = 1; o < 16; o <<= 1) v += __shfl_xor(v, o, kWave);
-  return v;
+// all-reduce over the four lanes that share lane % 16 (lanes l, l^16, l^32, l^48)
+__device__ __forceinline__ float quad_rows_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  return fmaxf(v, __shfl_xor(v, 32, kWave));
+}
+__device__ __forceinline__ float quad_rows_sum(float v) {
+  v += __shfl_xor(v, 16, kWave);
+  return v + __shfl_xor(v, 32, kWave);
 }
 
 template <int HD>
-__global__ void __launch_bounds__(kPfWaves* kWave)
+__global__ void __launch_bounds__(kPfThreads)
     attention_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                              const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                              const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
-                             const int* __restrict__ seq_start, int nh, int nkv, int B, float scale) {
-  constexpr int KSTEPS = HD / 32;  // matrix instructions per 16-token tile of scores
-  constexpr int DT = HD / 16;      // 16-dim tiles of the output
-  const int tile = blockIdx.x, seq = blockIdx.y, head = blockIdx.z;
+                             const int* __restrict__ seq_start, int nh, int nkv, int B, int b_shift, float scale) {
+  constexpr int KSTEPS = HD / 32;                          // matrix instructions per 16-token tile of scores
+  constexpr int DT = HD / 16;                              // 16-dim tiles of the output
+  constexpr int PIECES = kPfChunk * HD / 8 / kPfThreads;   // 16-byte pieces of a chunk per thread (keys; as many of values)
+  constexpr int KPITCH = HD + kPfPad, VPITCH = kPfChunk + kPfPad;
+  const int tile = gridDim.x - 1 - blockIdx.x, seq = blockIdx.y, head = blockIdx.z;   // long rows first
   const int row0 = run_start[seq], n_rows = run_start[seq + 1] - row0;
+  const int block_first = tile * kPfRows;
+  if (block_first >= n_rows) return;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
-  const int first = tile * kPfRows + wave * 16;  // first row of this wave inside the run
-  if (first >= n_rows) return;                   // whole waves leave; nothing below synchronises across waves
   const int n16 = lane % 16, kq = lane / 16;
   const int pos0 = seq_start[seq];
   const int kvh = head / (nh / nkv);
@@ -60,108 +81,166 @@ __global__ void __launch_bounds__(kPfWaves* kWave)
   const size_t head_elems = size_t(B) * HD, page_elems = head_elems * nkv;
   const uint16_t* kbase = kcache + kvh * head_elems;
   const uint16_t* vbase = vcache + kvh * head_elems;
+  const int block_last_pos = pos0 + min(block_first + kPfRows, n_rows) - 1;
+  const int first = block_first + wave * kPfWaveRows;   // first row of this wave inside the run
+  const bool wave_on = first < n_rows;
+  const int wave_last_pos = pos0 + min(first + kPfWaveRows, n_rows) - 1;
+  const int wave_first_pos = pos0 + min(first, n_rows - 1);
+  const float scale_log2 = scale * 1.4426950408889634f;   // scores are kept in units of log2: exp(x) = exp2(x log2 e)
+  const int b_mask = B - 1;
 
-  __shared__ __attribute__((aligned(16))) uint16_t p_lds[kPfWaves][16][kPfPitch];
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][kPfChunk][KPITCH];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][HD][VPITCH];
+  // the sequence's page ids up to the workgroup's last position: the address of a piece is one
+  // LDS read away instead of one more trip to global memory
+  extern __shared__ int page_lds[];
+  for (int i = threadIdx.x; i <= (block_last_pos >> b_shift); i += kPfThreads) page_lds[i] = table[i];
 
-  // A operand of the scores: lane holds 8 dims of query row n16 (rows past the run repeat its last row)
-  PFrag qf[KSTEPS];
-  {
-    const int r = row0 + min(first + n16, n_rows - 1);
+  // B operand of the scores: lane holds 8 dims of query row n16 of each tile (rows past the run
+  // repeat its last row; they are never stored).  That row's position is what the lane may see.
+  PFrag qf[kPfRT][KSTEPS];
+  int pos[kPfRT];
+#pragma unroll
+  for (int rt = 0; rt < kPfRT; ++rt) {
+    const int r = min(first + rt * 16 + n16, n_rows - 1);
+    pos[rt] = pos0 + r;
 #pragma unroll
     for (int c = 0; c < KSTEPS; ++c)
-      qf[c].u = *reinterpret_cast<const uint4*>(q + size_t(r) * q_stride + size_t(head) * HD + c * 32 + kq * 8);
+      qf[rt][c].u = *reinterpret_cast<const uint4*>(q + size_t(row0 + r) * q_stride + size_t(head) * HD + c * 32 + kq * 8);
   }
-  // accumulator rows of this lane: 4*kq + i; their positions decide what they may see
-  int pos[4];
+  float m[kPfRT], l[kPfRT];
+  f32x4 o[kPfRT][DT];   // O^T: column = query row n16, rows = dims 16 d + 4 kq + i
 #pragma unroll
-  for (int i = 0; i < 4; ++i) pos[i] = pos0 + min(first + 4 * kq + i, n_rows - 1);
-  const int last_pos = pos0 + min(first + 15, n_rows - 1);  // the wave's last row
+  for (int rt = 0; rt < kPfRT; ++rt) {
+    m[rt] = -FLT_MAX;
+    l[rt] = 0.f;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[rt][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  __syncthreads();   // page_lds is filled
 
-  float m[4], l[4];
-  f32x4 o[DT];
+  // What this thread moves from the cache to LDS for a chunk that starts at token c0: PIECES
+  // pieces of keys (8 dims of one token) and as many of values (8 tokens of one dim).  Tokens past
+  // the workgroup's last position are read from that position's place instead (always valid
+  // memory); the mask keeps them out.
+  uint4 kreg[PIECES], vreg[PIECES];
+  auto request = [&](int c0) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { m[i] = -FLT_MAX; l[i] = 0.f; }
+    for (int i = 0; i < PIECES; ++i) {
+      const int e = threadIdx.x + i * kPfThreads;
+      const int t = min(c0 + e / (HD / 8), block_last_pos);
+      kreg[i] = *reinterpret_cast<const uint4*>(kbase + size_t(page_lds[t >> b_shift]) * page_elems +
+                                                size_t(t & b_mask) * HD + (e % (HD / 8)) * 8);
+      const int tv = min(c0 + (e % 8) * 8, block_last_pos & ~7);
+      vreg[i] = *reinterpret_cast<const uint4*>(vbase + size_t(page_lds[tv >> b_shift]) * page_elems +
+                                                size_t(e / 8) * B + (tv & b_mask));
+    }
+  };
+  auto stage = [&](int buf) {
 #pragma unroll
-  for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < PIECES; ++i) {
+      const int e = threadIdx.x + i * kPfThreads;
+      *reinterpret_cast<uint4*>(&k_lds[buf][e / (HD / 8)][(e % (HD / 8)) * 8]) = kreg[i];
+      *reinterpret_cast<uint4*>(&v_lds[buf][e / 8][(e % 8) * 8]) = vreg[i];
+    }
+  };
 
-  for (int c0 = 0; c0 <= last_pos; c0 += kPfChunk) {
-    // ---- requests: keys of four 16-token tiles, values of two 32-token steps.  Tokens past the
-    // wave's last position point at that position: loads stay unconditional, the mask removes them.
-    PFrag kf[4][KSTEPS], vf[2][DT];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int t = min(c0 + j * 16 + n16, last_pos);
-      const uint16_t* kp = kbase + size_t(table[t / B]) * page_elems + size_t(t % B) * HD + kq * 8;
-#pragma unroll
-      for (int c = 0; c < KSTEPS; ++c) kf[j][c].u = *reinterpret_cast<const uint4*>(kp + c * 32);
-    }
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const int t = min(c0 + c * 32 + kq * 8, last_pos & ~7);
-      const uint16_t* vp = vbase + size_t(table[t / B]) * page_elems + t % B + size_t(n16) * B;
-#pragma unroll
-      for (int d = 0; d < DT; ++d) vf[c][d].u = *reinterpret_cast<const uint4*>(vp + size_t(d) * 16 * B);
-    }
+  request(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int c0 = 0; c0 <= block_last_pos; c0 += kPfChunk, buf ^= 1) {
+    // The next chunk's loads are in flight while this one is multiplied.  After the last chunk
+    // the same chunk is asked for again: no branch around the loads (the compiler would wait for
+    // them at once), and nobody reads what is staged then.
+    request(c0 + kPfChunk <= block_last_pos ? c0 + kPfChunk : c0);
 
-    // ---- scores: s[j][i] = scale * q[row 4kq+i] . k[token c0 + 16j + n16]
-    f32x4 s[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < KSTEPS; ++c) s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c].v, kf[j][c].v, s[j], 0, 0, 0);
-    }
-    float mx[4], alpha[4], sum[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      mx[i] = -FLT_MAX;
+    if (wave_on && c0 <= wave_last_pos) {
+      // ---- S^T: s[rt][j][i] = k[token c0 + 16 j + 4 kq + i] . q[row n16 of tile rt]
+      f32x4 s[kPfRT][4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int t = c0 + j * 16 + n16;
-        s[j][i] = t <= pos[i] ? s[j][i] * scale : -FLT_MAX;
-        mx[i] = fmaxf(mx[i], s[j][i]);
+        PFrag kf[KSTEPS];
+#pragma unroll
+        for (int c = 0; c < KSTEPS; ++c) kf[c].u = *reinterpret_cast<const uint4*>(&k_lds[buf][j * 16 + n16][c * 32 + kq * 8]);
+#pragma unroll
+        for (int rt = 0; rt < kPfRT; ++rt) {
+          s[rt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < KSTEPS; ++c)
+            s[rt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c].v, qf[rt][c].v, s[rt][j], 0, 0, 0);
+        }
       }
-      mx[i] = row16_max(mx[i]);
-      const float m_new = fmaxf(m[i], mx[i]);   // finite from the first trip on: token 0 is visible to every row
-      alpha[i] = expf(m[i] - m_new);
-      m[i] = m_new;
-      sum[i] = 0.f;
-    }
-    // ---- probabilities, to LDS in the accumulator layout (row 4kq+i, column 16j+n16)
+      // ---- running maximum and sum of the lane's query row; probabilities stay in registers
+      const bool diagonal = c0 + kPfChunk - 1 > wave_first_pos;   // some row of the wave cannot see the whole chunk
+      PFrag pf[kPfRT][2];   // B operands of the two 32-token steps
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+      for (int rt = 0; rt < kPfRT; ++rt) {
+        float mx = -FLT_MAX;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = s[j][i] > -FLT_MAX ? expf(s[j][i] - m[i]) : 0.f;
-        sum[i] += p;
-        p_lds[wave][4 * kq + i][j * 16 + n16] = float_to_bf16_bits(p);
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int t = c0 + j * 16 + 4 * kq + i;
+            s[rt][j][i] = (!diagonal || t <= pos[rt]) ? s[rt][j][i] * scale_log2 : -FLT_MAX;
+            mx = fmaxf(mx, s[rt][j][i]);
+          }
+        mx = quad_rows_max(mx);
+        const float m_new = fmaxf(m[rt], mx);   // finite from the first trip on: token 0 is visible to every row
+        const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_new);
+        m[rt] = m_new;
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            s[rt][j][i] = __builtin_amdgcn_exp2f(s[rt][j][i] - m_new);   // masked: exp2(-huge) = 0
+            sum += s[rt][j][i];
+          }
+        l[rt] = l[rt] * alpha + quad_rows_sum(sum);
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[rt][d][i] *= alpha;
+        // step c covers tiles 2c and 2c+1: reduction index e < 4 -> token 16(2c) + 4kq + e, e >= 4 -> 16(2c+1) + 4kq + e-4
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          pf[rt][c].u.x = pack_bf16(s[rt][2 * c][0], s[rt][2 * c][1]);
+          pf[rt][c].u.y = pack_bf16(s[rt][2 * c][2], s[rt][2 * c][3]);
+          pf[rt][c].u.z = pack_bf16(s[rt][2 * c + 1][0], s[rt][2 * c + 1][1]);
+          pf[rt][c].u.w = pack_bf16(s[rt][2 * c + 1][2], s[rt][2 * c + 1][3]);
+        }
       }
+      // ---- O^T += V^T * P^T, values read in the same token order
 #pragma unroll
-    for (int i = 0; i < 4; ++i) l[i] = l[i] * alpha[i] + row16_sum(sum[i]);
+      for (int c = 0; c < 2; ++c)
 #pragma unroll
-    for (int d = 0; d < DT; ++d)
+        for (int d = 0; d < DT; ++d) {
+          PFrag vf;
+          vf.h[0] = *reinterpret_cast<const uint2*>(&v_lds[buf][d * 16 + n16][(2 * c) * 16 + 4 * kq]);
+          vf.h[1] = *reinterpret_cast<const uint2*>(&v_lds[buf][d * 16 + n16][(2 * c + 1) * 16 + 4 * kq]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[d][i] *= alpha[i];
-    __builtin_amdgcn_wave_barrier();  // the wave's own LDS traffic stays in program order
-    // ---- out += P * V, P read back in the A-operand layout (row n16, 8 tokens kq*8..)
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      PFrag pf;
-      pf.u = *reinterpret_cast<const uint4*>(&p_lds[wave][n16][c * 32 + kq * 8]);
-#pragma unroll
-      for (int d = 0; d < DT; ++d) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf[c][d].v, o[d], 0, 0, 0);
+          for (int rt = 0; rt < kPfRT; ++rt) o[rt][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][c].v, o[rt][d], 0, 0, 0);
+        }
     }
-    __builtin_amdgcn_wave_barrier();
+    stage(buf ^ 1);
+    __syncthreads();
   }
 
+  if (!wave_on) return;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = first + 4 * kq + i;
+  for (int rt = 0; rt < kPfRT; ++rt) {
+    const int r = first + rt * 16 + n16;
     if (r >= n_rows) continue;
-    uint16_t* orow = out + size_t(row0 + r) * out_stride + size_t(head) * HD + n16;
-    const float inv = 1.0f / l[i];
+    uint16_t* orow = out + size_t(row0 + r) * out_stride + size_t(head) * HD + 4 * kq;
+    const float inv = 1.0f / l[rt];
 #pragma unroll
-    for (int d = 0; d < DT; ++d) orow[d * 16] = float_to_bf16_bits(o[d][i] * inv);
+    for (int d = 0; d < DT; ++d) {
+      uint2 v;
+      v.x = pack_bf16(o[rt][d][0] * inv, o[rt][d][1] * inv);
+      v.y = pack_bf16(o[rt][d][2] * inv, o[rt][d][3] * inv);
+      *reinterpret_cast<uint2*>(orow + d * 16) = v;
+    }
   }
 }
 
@@ -172,7 +251,7 @@ using namespace kvcm;
 extern "C" {
 
 int kvcm_attention_prefill_supported(int nh, int nkv, int hd, int B) {
-  return nkv > 0 && nh % nkv == 0 && (hd == 64 || hd == 128) && B > 0 && B % 8 == 0;
+  return nkv > 0 && nh % nkv == 0 && (hd == 64 || hd == 128) && B >= 8 && (B & (B - 1)) == 0;
 }
 
 // run_start [S+1]: first row of each sequence's run of consecutive positions (rows of a run are
@@ -189,15 +268,20 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
   KVCM_REQUIRE(q_stride >= nh * hd && out_stride >= nh * hd && q_stride % 8 == 0, "attention_prefill: bad row strides");
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(vcache) % 16 == 0, "attention_prefill: operands must be 16-byte aligned");
+  KVCM_REQUIRE(out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0, "attention_prefill: output must be 8-byte aligned");
+  int b_shift = 0;
+  while ((1 << b_shift) < B) ++b_shift;
   const dim3 grid((max_run + kPfRows - 1) / kPfRows, S, nh);
+  const size_t page_bytes = sizeof(int) * size_t(table_stride);
+  KVCM_REQUIRE(page_bytes <= 48 * 1024, "attention_prefill: page tables of %d entries do not fit LDS", table_stride);
   const uint16_t *qq = static_cast<const uint16_t*>(q), *kc = static_cast<const uint16_t*>(kcache),
                  *vc = static_cast<const uint16_t*>(vcache);
   if (hd == 64)
-    attention_prefill_kernel<64><<<grid, kPfWaves * kWave, 0, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
-                                                                  tables, table_stride, run_start, seq_start, nh, nkv, B, scale);
+    attention_prefill_kernel<64><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
+                                                             tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale);
   else
-    attention_prefill_kernel<128><<<grid, kPfWaves * kWave, 0, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
-                                                                   tables, table_stride, run_start, seq_start, nh, nkv, B, scale);
+    attention_prefill_kernel<128><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
+                                                              tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale);
   return launch_status("attention_prefill");
 }
 

@@ -205,7 +205,7 @@ template <class T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, const int* __restrict__ slots,
                                   T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int hd, int B,
-                                  const float* __restrict__ partials, int S) {
+                                  const float* __restrict__ partials, int S, const float2* __restrict__ cos_sin) {
   // one workgroup per (row, head): q heads, then k heads, then v heads
   const int t = blockIdx.x, h = blockIdx.y;
   T* row = qkv + size_t(t) * row_stride;
@@ -229,7 +229,13 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
       const float pos = float(positions[t]);
       for (int j = threadIdx.x; j < half; j += blockDim.x) {
         float sn, cs;
-        sincosf(pos * inv_freq[j], &sn, &cs);
+        if (cos_sin) {   // computed once per step by rope_table_kernel, the same values
+          const float2 t2 = cos_sin[size_t(t) * half + j];
+          cs = t2.x;
+          sn = t2.y;
+        } else {
+          sincosf(pos * inv_freq[j], &sn, &cs);
+        }
         const int c = h * hd + j;
         const float a = value(c), b = value(c + half);
         const float ra = a * cs - b * sn, rb = b * cs + a * sn;
@@ -255,6 +261,19 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
   // values are stored transposed inside the page: [page][kv_head][dim][slot]
   T* cache_head = vcache + (page * nkv + (h - nh - nkv)) * size_t(hd) * B + off;
   for (int d = threadIdx.x; d < hd; d += blockDim.x) store_f(cache_head + size_t(d) * B, value(h * hd + d));
+}
+
+// cos and sin of float(pos) * inv_freq[j] for every row of a step: the angles depend on the row
+// only, so a step computes them once and every layer's rotation reads them.
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float2* __restrict__ cos_sin, int half) {
+  const int t = blockIdx.x;
+  const float pos = float(positions[t]);
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    float sn, cs;
+    sincosf(pos * inv_freq[j], &sn, &cs);
+    cos_sin[size_t(t) * half + j] = float2{cs, sn};
+  }
 }
 
 // ---------------------------------------------------------------------------------- SwiGLU
@@ -339,12 +358,13 @@ int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const float* partials
 
 int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, const float* inv_freq,
                     const int* slots, void* kcache, void* vcache, int T, int nh, int nkv, int hd, int B,
-                    const float* partials, int S, hipStream_t s) {
+                    const float* partials, int S, const float* cos_sin, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(hd > 0 && hd % 2 == 0, "rope: head_dim %d must be even", hd);
   KVCM_REQUIRE(nh >= 0 && nkv >= 0 && row_stride >= (nh + 2 * nkv) * hd, "rope: row stride %d too small", row_stride);
   KVCM_REQUIRE(!slots || (kcache && vcache && B > 0), "rope: cache write without a cache");
   KVCM_REQUIRE(!inv_freq || positions, "rope: rotation without positions");
+  KVCM_REQUIRE(!cos_sin || inv_freq, "rope: a cos/sin table without rotation");
   KVCM_REQUIRE(!partials || S >= 1, "rope: partial sums need their split count");
   KVCM_REQUIRE(nh + 2 * nkv <= 65535 && nh + 2 * nkv > 0, "rope: too many heads");
   const dim3 grid(T, nh + 2 * nkv);
@@ -352,13 +372,21 @@ int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, 
   if (dtype == kF32)
     rope_cache_kernel<float><<<grid, threads, 0, s>>>(static_cast<float*>(qkv), row_stride, positions, inv_freq, slots,
                                                   static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, hd, B,
-                                                  partials, S);
+                                                  partials, S, reinterpret_cast<const float2*>(cos_sin));
   else if (dtype == kBF16)
     rope_cache_kernel<bf16_t><<<grid, threads, 0, s>>>(static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots,
                                                    static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, hd, B,
-                                                   partials, S);
+                                                   partials, S, reinterpret_cast<const float2*>(cos_sin));
   else KVCM_REQUIRE(false, "rope: unknown dtype %d", dtype);
   return launch_status("rope_cache");
+}
+
+// cos_sin [T][half][2] floats
+int kvcm_rope_table(const int* positions, const float* inv_freq, float* cos_sin, int T, int half, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && half > 0, "rope_table: bad sizes T=%d half=%d", T, half);
+  rope_table_kernel<<<T, 64, 0, s>>>(positions, inv_freq, reinterpret_cast<float2*>(cos_sin), half);
+  return launch_status("rope_table");
 }
 
 int kvcm_swiglu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t s) {

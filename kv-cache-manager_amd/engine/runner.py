@@ -86,6 +86,7 @@ class StepContext:
         # what kernels that size their launch by the context may assume; a captured graph sets it
         # to the largest context the engine allows, so that the launch fits every replay
         self.max_context_bound = max(L.max_context, 1)
+        self.shared = {}    # what parts of one step compute once and share (keyed by the part kind)
         d, h = runner.meta_dev, runner.meta_host
         T, S, R = self.rows, self.seqs, self.logit_rows_padded
         self.tokens = d[L.tokens:L.tokens + T]

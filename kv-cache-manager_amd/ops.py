@@ -31,7 +31,8 @@ def _declare(lib):
     lib.kvcm_hip_last_error.restype = C.c_char_p
     fn("kvcm_embed", vp, vp, i, vp, i, i, i, vp)
     fn("kvcm_rmsnorm", vp, vp, i, vp, i, i, vp, vp, i, vp, i, i, i, f, i, vp)
-    fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp)
+    fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp, vp)
+    fn("kvcm_rope_table", vp, vp, vp, i, i, vp)
     fn("kvcm_gemm_skinny_splits", i, i, i)
     fn("kvcm_gemm_skinny", vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp)
     fn("kvcm_reduce_store", vp, vp, i, i, i, i, i, vp)
@@ -152,8 +153,21 @@ def rmsnorm(x, weight, out, eps, add=None, rows=None, write_back=True):
                               _DT[weight.dtype], _ptr(out), _DT[out.dtype], R, H, float(eps), int(wb), _stream()))
 
 
+def rope_table(positions, inv_freq, out, rows=None):
+    """out[t, j] = (cos, sin) of float(positions[t]) * inv_freq[j]: the angles of a step, computed
+    once and read by every layer's rotation."""
+    _dev(positions, inv_freq, out)
+    T = out.shape[0] if rows is None else rows
+    _i32(positions, "positions", T)
+    _need(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous(), "inv_freq must be float32")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.dim() == 3 and out.shape[1] == inv_freq.numel()
+          and out.shape[2] == 2 and out.shape[0] >= T, "the table must be float32 [rows, head_dim/2, 2]")
+    _check(lib().kvcm_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(out), T, inv_freq.numel(), _stream()))
+    return out
+
+
 def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcache=None, vcache=None,
-               block_size=0, rows=None, source=None):
+               block_size=0, rows=None, source=None, cos_sin=None):
     """Rotates the q and k heads of the fused rows in place (inv_freq given) and copies k (rotated)
     and v to the paged cache (slots given).  Cache layout [pages, nkv, block_size, hd].  With
     ``source`` (PartialSums of the projection) the rows are read from there; q lands in ``qkv``."""
@@ -169,6 +183,9 @@ def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcac
               "inv_freq must hold head_dim/2 float32 values")
         _i32(positions, "positions", T)
         _need(positions is not None, "rotation needs positions")
+    if cos_sin is not None:
+        _need(inv_freq is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
+              and cos_sin.numel() >= T * hd, "cos_sin must be float32 [rows, head_dim/2, 2]")
     if slots is not None:
         _i32(slots, "slots", T)
         _need(kcache is not None and kcache.dtype == qkv.dtype and kcache.is_contiguous() and kcache.dim() == 4
@@ -178,7 +195,7 @@ def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcac
     _check(lib().kvcm_rope_cache(_ptr(qkv), _DT[qkv.dtype], qkv.stride(0), _ptr(positions), _ptr(inv_freq),
                                  _ptr(slots), _ptr(kcache), _ptr(vcache), T, nh, nkv, hd, block_size,
                                  _ptr(source.data) if source is not None else 0,
-                                 source.splits if source is not None else 0, _stream()))
+                                 source.splits if source is not None else 0, _ptr(cos_sin), _stream()))
 
 
 def swiglu(gate_up, out):

@@ -61,9 +61,20 @@ class Rotary(PositionEncoding):
         if head_dim != self.params["dim"]:
             raise ValueError("rotary: this kernel rotates the whole head (dim must equal head_dim)")
         k, v = cache if cache is not None else (None, None)
+        # the angles depend on the row only: the first layer of a step computes cos and sin, the
+        # others (same theta and dim) read them
+        table = None
+        shared = getattr(step, "shared", None)
+        if shared is not None:
+            key = ("rotary", float(self.params["theta"]), head_dim)
+            table = shared.get(key)
+            if table is None:
+                table = step.ws("rotary_cos_sin_%d" % head_dim, (step.rows, head_dim), torch.float32).view(step.rows, head_dim // 2, 2)
+                self.ctx.ops.rope_table(step.positions, self.inv_freq, table, rows=step.rows)
+                shared[key] = table
         self.ctx.ops.rope_cache(qkv, num_heads, num_kv_heads, head_dim, positions=step.positions,
                                 inv_freq=self.inv_freq, slots=slots, kcache=k, vcache=v,
-                                block_size=self.ctx.block_size, rows=step.rows, source=source)
+                                block_size=self.ctx.block_size, rows=step.rows, source=source, cos_sin=table)
         return cache is not None
 
 

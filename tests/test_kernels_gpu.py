@@ -148,6 +148,24 @@ def test_rope_dot_products_depend_on_distance_only(ops):
     assert abs(dot(5, 3) - base) > 1e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_from_a_step_table_equals_rope_with_inline_angles(ops, dtype):
+    rng = np.random.default_rng(41)
+    T, NH, NKV, HD = 7, 3, 1, 80
+    qkv = _bf16_grid(rng.normal(size=(T, (NH + 2 * NKV) * HD)))
+    pos = _t(np.array([0, 1, 63, 64, 1000, 4095, 100000], dtype=np.int32), torch.int32)
+    inv = _t(_inv_freq(HD, 5e5), torch.float32)
+    a, b = _t(qkv, dtype), _t(qkv, dtype)
+    table = torch.empty(T, HD // 2, 2, device=DEV)
+    ops.rope_table(pos, inv, table)
+    ops.rope_cache(a, NH, NKV, HD, positions=pos, inv_freq=inv)
+    ops.rope_cache(b, NH, NKV, HD, positions=pos, inv_freq=inv, cos_sin=table)
+    assert torch.equal(a, b)
+    ang = _np(pos)[:, None].astype(np.float32) * _np(inv)[None, :].astype(np.float32)
+    np.testing.assert_allclose(_np(table)[..., 0], np.cos(ang.astype(np.float64)), atol=2e-6)
+    np.testing.assert_allclose(_np(table)[..., 1], np.sin(ang.astype(np.float64)), atol=2e-6)
+
+
 # ------------------------------------------------------------------------------- KV write
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_reshape_and_cache_scatters_to_slots(ops, dtype):
