@@ -85,13 +85,15 @@ def prefill_run(eng, tokens, vocab, reps=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=240)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--only-prefill", action="store_true",
+                    help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N with N > 1 is not supported")
@@ -125,6 +127,18 @@ def main():
     del tensors
     torch.cuda.empty_cache()
 
+    def prefill_record():
+        T = 2048
+        sec = prefill_run(eng, T, V)
+        flops = (2.0 * T * (L * (layer_params - 2 * H)) + 2.0 * V * H
+                 + L * 4.0 * (T * (T + 1) / 2) * cfg.head_dim * cfg.num_attention_heads)
+        return {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
+                "frac": round(flops / sec / PEAK_FLOPS[key], 4)}
+
+    if args.only_prefill:
+        print(json.dumps({"prefill": prefill_record()}), flush=True)
+        return
+
     seconds, ctx = decode_run(eng, args.batch, args.prompt_len, args.steps, args.warmup, V)
     value = args.batch * args.steps / seconds
     out = {
@@ -147,11 +161,7 @@ def main():
             points[f"decode_b{b}_ms"] = round(1e3 * s / k, 4)
             points[f"decode_b{b}_hbm_frac"] = roofline(b, s / k, c)["frac"]
         out["points"] = points
-        T = 2048
-        sec = prefill_run(eng, T, V)
-        flops = 2.0 * T * (L * (layer_params - 2 * H)) + 2.0 * V * H + L * 4.0 * (T * (T + 1) / 2) * cfg.head_dim * cfg.num_attention_heads
-        out["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
-                          "frac": round(flops / sec / PEAK_FLOPS[key], 4)}
+        out["prefill"] = prefill_record()
     print(json.dumps(out), flush=True)
 
 

@@ -122,7 +122,7 @@ class BatchLayout:
     """Offsets (in int32 elements) of every array inside one packed metadata buffer."""
     FIELDS = ("rows", "seqs", "logit_rows", "max_context", "max_run", "total",
               "tokens", "positions", "context_lens", "row_seq", "run_start", "seq_start", "seq_end",
-              "logit_row_index", "state_slots", "rows_padded", "seqs_padded", "logit_rows_padded")
+              "logit_row_index", "state_slots", "rows_padded", "seqs_padded", "logit_rows_padded", "sampling")
     GROUP_BASE, GROUP_STRIDE = 20, 4
 
     def __init__(self, desc, num_groups):

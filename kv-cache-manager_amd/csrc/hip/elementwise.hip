@@ -126,42 +126,49 @@ __global__ void __launch_bounds__(kNormThreads)
   const size_t pstride = size_t(T) * H;
   float v[VPT][4], wv[VPT][4];
   bool on[VPT];
-  // thread t owns elements 4 * (t + 256 k) .. + 3
+  int at[VPT];
+  // thread t owns elements 4 * (t + 256 k) .. + 3.  Every load is unconditional (a thread beyond
+  // the row reads the row's last four elements and its values are zeroed afterwards): a branch
+  // around a load makes the compiler wait for that load on the spot, one memory latency each.
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int i = 4 * (threadIdx.x + k * kNormThreads);
     on[k] = i < H;
-    if (on[k]) {
-      load4<float>(xr + i, v[k]);
-      load4<TW>(w + i, wv[k]);
-    } else {
-      v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.f;
-    }
+    at[k] = on[k] ? i : H - 4;
+    load4<float>(xr + at[k], v[k]);
+    load4<TW>(w + at[k], wv[k]);
   }
   if (add) {
     const TA* ar = add + size_t(src) * H;
+    float a[VPT][4];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      if (!on[k]) continue;
-      float a[4];
-      load4<TA>(ar + 4 * (threadIdx.x + k * kNormThreads), a);
+    for (int k = 0; k < VPT; ++k) load4<TA>(ar + at[k], a[k]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[k][e] += a[e];
-    }
+    for (int k = 0; k < VPT; ++k)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[k][e] += a[k][e];
   } else if (partials) {
     const float* pr = partials + size_t(src) * H;
     float a[VPT][4];
 #pragma unroll
     for (int k = 0; k < VPT; ++k) a[k][0] = a[k][1] = a[k][2] = a[k][3] = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < S; ++s) {
+    // four splits per trip, all their loads requested before the first sum; a split beyond S
+    // reads split S - 1 again and adds nothing, so the order of the sums is that of the splits
+    for (int s0 = 0; s0 < S; s0 += 4) {
+      float p[4][VPT][4];
 #pragma unroll
-      for (int k = 0; k < VPT; ++k) {
-        if (!on[k]) continue;
-        float p[4];
-        load4<float>(pr + s * pstride + 4 * (threadIdx.x + k * kNormThreads), p);
+      for (int j = 0; j < 4; ++j) {
+        const int sj = s0 + j < S ? s0 + j : S - 1;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) a[k][e] += p[e];
+        for (int k = 0; k < VPT; ++k) load4<float>(pr + sj * pstride + at[k], p[j][k]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool keep = s0 + j < S;
+#pragma unroll
+        for (int k = 0; k < VPT; ++k)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[k][e] += keep ? p[j][k][e] : 0.f;
       }
     }
 #pragma unroll
@@ -169,6 +176,9 @@ __global__ void __launch_bounds__(kNormThreads)
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[k][e] += round_to<TO>(a[k][e]);
   }
+#pragma unroll
+  for (int k = 0; k < VPT; ++k)
+    if (!on[k]) v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.f;
   if ((add || partials) && write_back) {
 #pragma unroll
     for (int k = 0; k < VPT; ++k)
@@ -216,7 +226,13 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
   auto value = [&](int c) {
     if (!prow) return load_f(row + c);
     float a = 0.f;
-    for (int s = 0; s < S; ++s) a += prow[s * pstride + c];
+    for (int s0 = 0; s0 < S; s0 += 4) {   // four loads requested together; a split beyond S adds nothing
+      float p[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) p[j] = prow[(s0 + j < S ? s0 + j : S - 1) * pstride + c];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a += s0 + j < S ? p[j] : 0.f;
+    }
     return round_to<T>(a);
   };
   const int slot = slots ? slots[t] : -1;
@@ -263,6 +279,67 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
   for (int d = threadIdx.x; d < hd; d += blockDim.x) store_f(cache_head + size_t(d) * B, value(h * hd + d));
 }
 
+// The same for whole fused rows (no partial sums) whose head size is a multiple of 16: a thread
+// takes 8 pairs of a q or k head (or 16 values of a v head) with vector loads and stores, so a
+// prompt's rows move at memory speed.  Same formulas, same values as the kernel above.
+template <class T>
+__global__ void __launch_bounds__(256)
+    rope_cache_vec_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
+                          const float* __restrict__ inv_freq, const int* __restrict__ slots, T* __restrict__ kcache,
+                          T* __restrict__ vcache, int nh, int nkv, int hd, int B, const float2* __restrict__ cos_sin,
+                          long long items) {
+  const long long item = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x;
+  if (item >= items) return;
+  const int cph = hd / 16, heads = nh + 2 * nkv, half = hd / 2;
+  const int c = int(item % cph), h = int((item / cph) % heads), t = int(item / (static_cast<long long>(cph) * heads));
+  T* row = qkv + size_t(t) * row_stride + size_t(h) * hd;
+  const int slot = slots ? slots[t] : -1;
+  const size_t page = slot >= 0 ? slot / B : 0;
+  const int off = slot >= 0 ? slot % B : 0;
+  if (h >= nh + nkv) {   // a v head: 16 values to the transposed page
+    if (slot < 0) return;
+    float v[16];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) load4<T>(row + c * 16 + 4 * k, v + 4 * k);
+    T* cache_head = vcache + (page * nkv + (h - nh - nkv)) * size_t(hd) * B + off;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) store_f(cache_head + size_t(c * 16 + e) * B, v[e]);
+    return;
+  }
+  const bool is_k = h >= nh;
+  T* cache_row = (is_k && slot >= 0) ? kcache + ((page * nkv + (h - nh)) * B + off) * hd : nullptr;
+  const int j0 = c * 8;
+  float a[8], b[8];
+  load4<T>(row + j0, a); load4<T>(row + j0 + 4, a + 4);
+  load4<T>(row + half + j0, b); load4<T>(row + half + j0 + 4, b + 4);
+  if (inv_freq) {
+    float cs[8], sn[8];
+    if (cos_sin) {
+      const float4* tab = reinterpret_cast<const float4*>(cos_sin + size_t(t) * half + j0);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float4 v = tab[k];
+        cs[2 * k] = v.x; sn[2 * k] = v.y; cs[2 * k + 1] = v.z; sn[2 * k + 1] = v.w;
+      }
+    } else {
+      const float pos = float(positions[t]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sincosf(pos * inv_freq[j0 + e], &sn[e], &cs[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float ra = a[e] * cs[e] - b[e] * sn[e], rb = b[e] * cs[e] + a[e] * sn[e];
+      a[e] = ra; b[e] = rb;
+    }
+    store4<T>(row + j0, a); store4<T>(row + j0 + 4, a + 4);
+    store4<T>(row + half + j0, b); store4<T>(row + half + j0 + 4, b + 4);
+  }
+  if (cache_row) {
+    store4<T>(cache_row + j0, a); store4<T>(cache_row + j0 + 4, a + 4);
+    store4<T>(cache_row + half + j0, b); store4<T>(cache_row + half + j0 + 4, b + 4);
+  }
+}
+
 // cos and sin of float(pos) * inv_freq[j] for every row of a step: the angles depend on the row
 // only, so a step computes them once and every layer's rotation reads them.
 __global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
@@ -290,6 +367,21 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     const float s = x / (1.0f + expf(-x));
     store_f(o + i, round_to<T>(s) * load_f(u + i));
   }
+}
+
+template <class T>
+__global__ void __launch_bounds__(256) swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int I) {
+  const int t = blockIdx.y;
+  const int i = 8 * (blockIdx.x * blockDim.x + threadIdx.x);
+  if (i >= I) return;
+  const T* g = gu + size_t(t) * 2 * I + i;
+  float x[8], u[8], y[8];
+  load4<T>(g, x); load4<T>(g + 4, x + 4);
+  load4<T>(g + I, u); load4<T>(g + I + 4, u + 4);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) y[e] = round_to<T>(x[e] / (1.0f + expf(-x[e]))) * u[e];
+  T* o = out + size_t(t) * I + i;
+  store4<T>(o, y); store4<T>(o + 4, y + 4);
 }
 
 // ------------------------------------------------------------------------------- residual
@@ -367,6 +459,23 @@ int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, 
   KVCM_REQUIRE(!cos_sin || inv_freq, "rope: a cos/sin table without rotation");
   KVCM_REQUIRE(!partials || S >= 1, "rope: partial sums need their split count");
   KVCM_REQUIRE(nh + 2 * nkv <= 65535 && nh + 2 * nkv > 0, "rope: too many heads");
+  const bool aligned = reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0 && row_stride % 4 == 0;
+  if (!partials && hd % 16 == 0 && aligned) {
+    const long long items = static_cast<long long>(T) * (nh + 2 * nkv) * (hd / 16);
+    const long long blocks = (items + 255) / 256;
+    KVCM_REQUIRE(blocks < (1ll << 31), "rope: too many rows");
+    if (dtype == kF32)
+      rope_cache_vec_kernel<float><<<static_cast<unsigned>(blocks), 256, 0, s>>>(
+          static_cast<float*>(qkv), row_stride, positions, inv_freq, slots, static_cast<float*>(kcache),
+          static_cast<float*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), items);
+    else if (dtype == kBF16)
+      rope_cache_vec_kernel<bf16_t><<<static_cast<unsigned>(blocks), 256, 0, s>>>(
+          static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots, static_cast<bf16_t*>(kcache),
+          static_cast<bf16_t*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), items);
+    else KVCM_REQUIRE(false, "rope: unknown dtype %d", dtype);
+    return launch_status("rope_cache");
+  }
   const dim3 grid(T, nh + 2 * nkv);
   const int threads = 64;
   if (dtype == kF32)
@@ -392,6 +501,13 @@ int kvcm_rope_table(const int* positions, const float* inv_freq, float* cos_sin,
 int kvcm_swiglu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  if (I % 8 == 0 && reinterpret_cast<uintptr_t>(gate_up) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const dim3 vgrid((I / 8 + 255) / 256, T);
+    if (dtype == kF32) swiglu_vec_kernel<float><<<vgrid, 256, 0, s>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), I);
+    else if (dtype == kBF16) swiglu_vec_kernel<bf16_t><<<vgrid, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out), I);
+    else KVCM_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+    return launch_status("swiglu");
+  }
   const dim3 grid((I + 255) / 256, T);
   if (dtype == kF32) swiglu_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), I);
   else if (dtype == kBF16) swiglu_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out), I);

@@ -10,6 +10,11 @@
 // 32-bit partial sums go to scratch [S][M][N] and the consumer adds them in split order:
 // reduce_store below, or the fused consumers (residual add + RMS norm, SwiGLU, rotary + cache
 // write) in elementwise.hip.  No atomics: the result is the same on every run.
+//
+// SWIGLU variant: W is a fused [gate (I rows) | up (I rows)] matrix; a workgroup takes 8 gate rows
+// and the 8 up rows of the same columns, and stores act = round(round(silu(g)) * u) [M, I]
+// directly (g, u rounded to the storage type first, exactly what the separate SwiGLU kernel
+// computes from the stored product).  Unsplit only.
 #include "common.h"
 
 namespace kvcm {
@@ -24,21 +29,21 @@ union Frag {
   bf16x8 v;
 };
 
-template <int MT, class TO>
+template <int MT, class TO, bool SWIGLU>
 __global__ void __launch_bounds__(256)
     gemm_skinny_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ partials,
                        TO* __restrict__ out, int M, int N, int K, int ldx, int ldw, int ldo, int S) {
   __shared__ f32x4 red[4][MT][kWave];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int r = lane % 16, kq = lane / 16;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * (SWIGLU ? 8 : 16);   // SWIGLU: N is I, the width of the result
   const int s = blockIdx.y;
   const int units = K / kUnit;
   const int u_lo = int((long long)units * s / S), u_hi = int((long long)units * (s + 1) / S);
   const int span = u_hi - u_lo;
   const int w_lo = u_lo + span * wave / 4, w_hi = u_lo + span * (wave + 1) / 4;
 
-  const uint16_t* wrow = W + size_t(n0 + r) * ldw + kq * 16;
+  const uint16_t* wrow = W + size_t(SWIGLU ? (r < 8 ? n0 + r : N + n0 + r - 8) : n0 + r) * ldw + kq * 16;
   const uint16_t* xrow[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -90,6 +95,28 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
   for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
   __syncthreads();
+  if constexpr (SWIGLU) {
+    for (int item = threadIdx.x; item < MT * kWave; item += 256) {
+      const int t = item / kWave, l = item % kWave;
+      if (l % 16 >= 8) continue;
+      f32x4 g = red[0][t][l], up = red[0][t][l + 8];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) {
+        const f32x4 a = red[w][t][l], b = red[w][t][l + 8];
+        g[0] += a[0]; g[1] += a[1]; g[2] += a[2]; g[3] += a[3];
+        up[0] += b[0]; up[1] += b[1]; up[2] += b[2]; up[3] += b[3];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = t * 16 + (l / 16) * 4 + i;
+        if (m >= M) continue;
+        const float x = round_to<TO>(g[i]);
+        const float act = x / (1.0f + expf(-x));
+        store_f(out + size_t(m) * ldo + n0 + l % 16, round_to<TO>(act) * round_to<TO>(up[i]));
+      }
+    }
+    return;
+  }
   for (int item = threadIdx.x; item < MT * kWave; item += 256) {
     const int t = item / kWave, l = item % kWave;
     f32x4 v = red[0][t][l];
@@ -152,7 +179,7 @@ int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, i
   const uint16_t* w = static_cast<const uint16_t*>(W);
   const int mt = (M + 15) / 16;
 #define KVCM_SKINNY(MT, TO) \
-  gemm_skinny_kernel<MT, TO><<<grid, 256, 0, st>>>(x, w, partials, static_cast<TO*>(out), M, N, K, ldx, ldw, ldo, S)
+  gemm_skinny_kernel<MT, TO, false><<<grid, 256, 0, st>>>(x, w, partials, static_cast<TO*>(out), M, N, K, ldx, ldw, ldo, S)
   if (out_dtype == kBF16) {
     if (mt == 1) KVCM_SKINNY(1, bf16_t); else if (mt == 2) KVCM_SKINNY(2, bf16_t); else if (mt == 3) KVCM_SKINNY(3, bf16_t); else KVCM_SKINNY(4, bf16_t);
   } else if (out_dtype == kF32) {
@@ -162,6 +189,37 @@ int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, i
   }
 #undef KVCM_SKINNY
   return launch_status("gemm_skinny");
+}
+
+// May act = swiglu(X * [gate | up]^T) be computed in one launch?  I is the width of the result.
+int kvcm_gemm_skinny_swiglu_supported(int M, int I, int K) {
+  // below 320 column tiles a split product fills the chip better than this unsplit one
+  return M > 0 && M <= 64 && I > 0 && I % 8 == 0 && K > 0 && K % kUnit == 0 && I / 8 >= 320;
+}
+
+// W [2 I, K] (gate rows, then up rows); out [M, I].
+int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dtype, int M, int I, int K, int ldx,
+                            int ldw, int ldo, hipStream_t st) {
+  KVCM_REQUIRE(kvcm_gemm_skinny_swiglu_supported(M, I, K), "gemm_skinny_swiglu: unsupported shape M=%d I=%d K=%d", M, I, K);
+  KVCM_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0 && reinterpret_cast<uintptr_t>(X) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(W) % 16 == 0,
+               "gemm_skinny_swiglu: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
+  KVCM_REQUIRE(ldx >= K && ldw >= K && out != nullptr && ldo >= I, "gemm_skinny_swiglu: leading dimensions too small");
+  const dim3 grid(I / 8, 1);
+  const uint16_t* x = static_cast<const uint16_t*>(X);
+  const uint16_t* w = static_cast<const uint16_t*>(W);
+  const int mt = (M + 15) / 16;
+#define KVCM_SKINNY(MT, TO) \
+  gemm_skinny_kernel<MT, TO, true><<<grid, 256, 0, st>>>(x, w, nullptr, static_cast<TO*>(out), M, I, K, ldx, ldw, ldo, 1)
+  if (out_dtype == kBF16) {
+    if (mt == 1) KVCM_SKINNY(1, bf16_t); else if (mt == 2) KVCM_SKINNY(2, bf16_t); else if (mt == 3) KVCM_SKINNY(3, bf16_t); else KVCM_SKINNY(4, bf16_t);
+  } else if (out_dtype == kF32) {
+    if (mt == 1) KVCM_SKINNY(1, float); else if (mt == 2) KVCM_SKINNY(2, float); else if (mt == 3) KVCM_SKINNY(3, float); else KVCM_SKINNY(4, float);
+  } else {
+    KVCM_REQUIRE(false, "gemm_skinny_swiglu: unknown output dtype %d", out_dtype);
+  }
+#undef KVCM_SKINNY
+  return launch_status("gemm_skinny_swiglu");
 }
 
 int kvcm_reduce_store(const float* partials, void* out, int out_dtype, int M, int N, int ldo, int S, hipStream_t st) {

@@ -10,7 +10,7 @@
 
 namespace kvcm {
 
-constexpr int kSampleThreads = 256;
+constexpr int kSampleThreads = 1024;  // one workgroup per row: its latency is the kernel's time
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   z += 0x9E3779B97F4A7C15ull;
@@ -33,6 +33,7 @@ __global__ void __launch_bounds__(kSampleThreads)
   }
   float best = -INFINITY;
   int idx = 0x7fffffff;
+#pragma unroll 4
   for (int j = threadIdx.x; j < V; j += kSampleThreads) {
     float v = row[j];
     if (temp > 0.f) {

@@ -5,6 +5,7 @@
 // and padding to a fixed shape are additions.
 #pragma once
 #include <cstdint>
+#include <cstring>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -18,6 +19,11 @@ struct BatchEntry {
   int start;
   int count;
   std::vector<int32_t> want;  // offsets inside [0, count) whose logits are asked for
+  // how a token is drawn from each wanted row (the sampling kernel reads them from the same buffer)
+  float temperature = 0.f;
+  uint64_t sampler_seed = 0;
+  int64_t request_id = 0;
+  int32_t token_index = 0;
 };
 
 // Index of each field in the descriptor array.
@@ -25,6 +31,9 @@ enum BatchDesc : int {
   kRows = 0, kSeqs, kLogitRows, kMaxContext, kMaxRun, kTotalInts,
   kOffTokens, kOffPositions, kOffContextLens, kOffRowSeq, kOffRunStart, kOffSeqStart, kOffSeqEnd,
   kOffLogitRows, kOffStateSlots, kRowsPadded, kSeqsPadded, kLogitRowsPadded,
+  // sampling parameters per (padded) logit row, starting at an even offset so that the 64-bit
+  // arrays are aligned: float temperature[Rp], int32 token_index[Rp], uint64 seed[Rp], int64 request_id[Rp]
+  kOffSampling,
   kGroupBase = 20,  // per group: slots offset, tables offset, table stride, (spare)
   kGroupStride = 4,
 };
@@ -86,6 +95,9 @@ inline void build_batch(const KVManager& kv, const std::vector<BatchEntry>& entr
     desc[kGroupBase + kGroupStride * g + 1] = static_cast<int32_t>(o_tables[g]);
     desc[kGroupBase + kGroupStride * g + 2] = paged ? widest[g] : 0;
   }
+  cursor += cursor & 1;
+  const int64_t o_samp = take(6 * int64_t(Rp));
+  desc[kOffSampling] = static_cast<int32_t>(o_samp);
   if (cursor > cap) throw std::length_error("build_batch: the metadata buffer is too small");
   if (cursor > INT32_MAX) throw std::length_error("build_batch: metadata exceeds 2^31 ints");
   desc[kTotalInts] = static_cast<int32_t>(cursor);
@@ -130,6 +142,11 @@ inline void build_batch(const KVManager& kv, const std::vector<BatchEntry>& entr
     }
     for (int w : e.want) {
       if (w < 0 || w >= e.count) throw std::invalid_argument("build_batch: wanted place outside the run");
+      static_assert(sizeof(float) == 4, "the buffer holds 32-bit floats");
+      std::memcpy(out + o_samp + lrow, &e.temperature, 4);
+      out[o_samp + Rp + lrow] = e.token_index;
+      std::memcpy(out + o_samp + 2 * int64_t(Rp) + 2 * int64_t(lrow), &e.sampler_seed, 8);
+      std::memcpy(out + o_samp + 4 * int64_t(Rp) + 2 * int64_t(lrow), &e.request_id, 8);
       out[o_lrow + lrow++] = out[o_run + s] + w;
     }
   }

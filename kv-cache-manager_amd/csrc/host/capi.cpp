@@ -423,6 +423,10 @@ int kvcm_build_batch_from_plan(void* c, int pad_rows, int pad_seqs, int pad_logi
       e.start = p.start;
       e.count = p.num_tokens;
       if (p.samples) e.want = {p.num_tokens - 1};
+      e.temperature = p.seq->temperature;
+      e.sampler_seed = p.seq->sampler_seed;
+      e.request_id = p.seq->id;
+      e.token_index = p.seq->num_generated();
       entries.push_back(std::move(e));
     }
     build_batch(*core->kv, entries, pad_rows, pad_seqs, pad_logit_rows, table_stride, out, cap, desc);

@@ -94,8 +94,7 @@ class Engine:
             info.rows, info.seqs = layout.rows, layout.seqs
             ids = np.zeros(0, dtype=np.int32)
             if sampling:
-                ids = self.sampler.sample(logits, [p.temperature for p in sampling], [p.seed for p in sampling],
-                                          [p.id for p in sampling], [p.gen_index for p in sampling])
+                ids = self.sampler.sample_on_device(logits, self.runner.last_step.sampling_params())
             else:
                 torch.cuda.current_stream().synchronize()
         nxt, k = [], 0

@@ -56,9 +56,9 @@ class DecodeGraphs:
         step = StepContext(self.runner, layout)
         step.max_context_bound = self.runner.limits.max_context_len
         logits = self.runner.model.forward(step)
-        s = self.sampler
-        self.runner.ops.sample(logits, s.out[:bucket], s.temperature[:bucket], s.seeds[:bucket],
-                               s.request_ids[:bucket], s.token_index[:bucket])
+        # the sampling parameters lie in the metadata buffer (padding rows: temperature 0, dropped)
+        t, seeds, ids, idx = step.sampling_params()
+        self.runner.ops.sample(logits, self.sampler.out[:bucket], t, seeds, ids, idx)
 
     def run(self, plan) -> np.ndarray:
         n = len(plan)
@@ -71,18 +71,6 @@ class DecodeGraphs:
         runner.meta_dev[:total].copy_(runner._pinned[:total], non_blocking=True)
         runner._upload_done.record()
         runner._upload_pending = True
-        # sampling parameters for the real rows; padding rows keep temperature 0 (argmax, dropped)
-        temps = np.zeros(bucket, dtype=np.float32)
-        seeds = np.zeros(bucket, dtype=np.uint64)
-        reqs = np.zeros(bucket, dtype=np.int64)
-        idx = np.zeros(bucket, dtype=np.int32)
-        for k, p in enumerate(plan):
-            temps[k], seeds[k], reqs[k], idx[k] = p.temperature, p.seed & ((1 << 64) - 1), p.id, p.gen_index
-        s.temperature[:bucket].copy_(torch.from_numpy(temps))
-        s.seeds[:bucket].copy_(torch.from_numpy(seeds.view(np.int64)))
-        s.request_ids[:bucket].copy_(torch.from_numpy(reqs))
-        s.token_index[:bucket].copy_(torch.from_numpy(idx))
-
         graph = self.graphs.get(bucket)
         if graph is None:
             self._forward(layout, bucket)                 # eager once: creates every work buffer
@@ -92,5 +80,4 @@ class DecodeGraphs:
                 self._forward(layout, bucket)
             self.graphs[bucket] = graph
         graph.replay()
-        s._host[:bucket].copy_(s.out[:bucket])            # synchronous download
-        return s._host[:n].numpy().copy()
+        return s.download(n)

@@ -105,6 +105,13 @@ class StepContext:
         self.host_seq_end = h[L.seq_end:L.seq_end + S]
         self.host_state_slots = h[L.state_slots:L.state_slots + S]
 
+    def sampling_params(self):
+        """(temperature f32, seeds i64 bit patterns, request ids i64, token index i32), one entry per
+        padded logit row, on the device: they travel in the step's metadata buffer."""
+        d, o, R = self.runner.meta_dev, self.layout.sampling, self.logit_rows_padded
+        return (d[o:o + R].view(torch.float32), d[o + 2 * R:o + 4 * R].view(torch.int64),
+                d[o + 4 * R:o + 6 * R].view(torch.int64), d[o + R:o + 2 * R])
+
     def slots(self, g):
         L = self.layout
         return self.runner.meta_dev[L.slots[g]:L.slots[g] + self.rows]
@@ -135,7 +142,7 @@ class ModelRunner:
         self.ops = model.ctx.ops
         self.workspace = Workspace(device, dtype, limits, self.ops)
         G = core.num_groups
-        ints = (4 * limits.max_tokens + 4 * limits.max_seqs + 1 + limits.max_logit_rows
+        ints = (4 * limits.max_tokens + 4 * limits.max_seqs + 1 + 7 * limits.max_logit_rows
                 + G * (limits.max_tokens + limits.max_seqs * limits.max_blocks_per_seq) + 64)
         self._pinned = torch.empty(ints, dtype=torch.int32, pin_memory=True)
         self.meta_host = self._pinned.numpy()
@@ -221,6 +228,7 @@ class ModelRunner:
         x, pending = self.model.run_layers(step)
         if layout.logit_rows_padded == 0:
             return None
+        self.last_step = step
         return self.model.head_logits(step, x, pending, step.logit_row_index)[:layout.logit_rows]
 
     def execute_to_host(self, layout: BatchLayout) -> Optional[np.ndarray]:

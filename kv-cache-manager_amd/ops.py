@@ -33,6 +33,8 @@ def _declare(lib):
     fn("kvcm_rmsnorm", vp, vp, i, vp, i, i, vp, vp, i, vp, i, i, i, f, i, vp)
     fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp, vp)
     fn("kvcm_rope_table", vp, vp, vp, i, i, vp)
+    fn("kvcm_gemm_skinny_swiglu_supported", i, i, i)
+    fn("kvcm_gemm_skinny_swiglu", vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_gemm_skinny_splits", i, i, i)
     fn("kvcm_gemm_skinny", vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp)
     fn("kvcm_reduce_store", vp, vp, i, i, i, i, i, vp)
@@ -261,6 +263,25 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
     _check(lib().kvcm_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, x.stride(0), w.stride(0),
                                 out.stride(0), _stream()))
     return out
+
+
+def gemm_swiglu(x, w_gate_up, out):
+    """out[M, I] = swiglu(x[M, K] @ w_gate_up[2 I, K]^T) in one launch, or False when this shape
+    has no fused kernel (then the caller runs the product and ``swiglu`` one after the other:
+    the same values)."""
+    _dev(x, w_gate_up, out)
+    for t, n in ((x, "x"), (w_gate_up, "w_gate_up"), (out, "out")):
+        _rows2d(t, n)
+    M, K = x.shape
+    I = out.shape[1]
+    _need(w_gate_up.shape == (2 * I, K) and out.shape[0] == M, "gemm_swiglu shapes do not agree")
+    if not (x.dtype == w_gate_up.dtype == out.dtype == torch.bfloat16 and x.stride(0) % 8 == 0
+            and w_gate_up.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
+            and lib().kvcm_gemm_skinny_swiglu_supported(M, I, K)):
+        return False
+    _check(lib().kvcm_gemm_skinny_swiglu(_ptr(x), _ptr(w_gate_up), _ptr(out), _DT[out.dtype], M, I, K, x.stride(0),
+                                         w_gate_up.stride(0), out.stride(0), _stream()))
+    return True
 
 
 def _check_caches(kcache, vcache, nkv, hd):

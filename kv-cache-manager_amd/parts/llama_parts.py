@@ -145,9 +145,10 @@ class SwiGLU(FeedForward):
 
     def forward(self, step, h):
         I = self.params["intermediate_size"]
-        gu = _linear(self.ctx, step, h, self.w["w_gate_up"], "gate_up")
         act = step.ws("act", (step.rows, I))
-        self.ctx.ops.swiglu(gu, act)
+        if not self.ctx.ops.gemm_swiglu(h, self.w["w_gate_up"], act):      # few rows: one launch
+            gu = _linear(self.ctx, step, h, self.w["w_gate_up"], "gate_up")
+            self.ctx.ops.swiglu(gu, act)
         return _linear(self.ctx, step, act, self.w["w_down"], "ffn_out", keep_partial=True)
 
 

@@ -36,5 +36,18 @@ class Sampler:
             self.token_index[:R].copy_(torch.tensor(list(token_index), dtype=torch.int32))
             self.ops.sample(logits, out, self.temperature[:R], self.seeds[:R], self.request_ids[:R],
                             self.token_index[:R])
-        self._host[:R].copy_(out)          # synchronous: the ids are needed on the host now
+        return self.download(R)
+
+    def sample_on_device(self, logits: torch.Tensor, params) -> np.ndarray:
+        """As ``sample`` with the parameters already on the device: (temperature, seeds, request
+        ids, token index) as the step's metadata buffer carries them."""
+        R = logits.shape[0]
+        if R > self.max_rows:
+            raise RuntimeError(f"sampler: {R} rows exceed the limit of {self.max_rows}")
+        t, seeds, ids, idx = params
+        self.ops.sample(logits, self.out[:R], t[:R], seeds[:R], ids[:R], idx[:R])
+        return self.download(R)
+
+    def download(self, R: int) -> np.ndarray:
+        self._host[:R].copy_(self.out[:R])          # synchronous: the ids are needed on the host now
         return self._host[:R].numpy().copy()

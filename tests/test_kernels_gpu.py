@@ -575,6 +575,24 @@ def test_partial_sums_feed_the_fused_norm_and_rope(ops):
     assert torch.equal(caches[0], caches[2]) and torch.equal(caches[1], caches[3])
 
 
+def test_skinny_gemm_with_swiglu_epilogue_equals_product_then_swiglu(ops):
+    rng = np.random.default_rng(77)
+    for M, I, K in ((8, 2560, 256), (1, 5632, 2048), (37, 2568, 192), (64, 2560, 128)):
+        x = _t(rng.normal(size=(M, K)), torch.bfloat16)
+        w = _t(rng.normal(size=(2 * I, K)) * 0.1, torch.bfloat16)
+        act = torch.zeros(M, I, dtype=torch.bfloat16, device=DEV)
+        assert ops.gemm_swiglu(x, w, act)
+        gu = torch.zeros(M, 2 * I, dtype=torch.bfloat16, device=DEV)
+        ops.gemm(x, w, gu)                                   # unsplit: no scratch given
+        ref = torch.zeros_like(act)
+        ops.swiglu(gu, ref)
+        assert torch.equal(act, ref)
+    small = torch.zeros(8, 256, dtype=torch.bfloat16, device=DEV)      # too few columns to fill the chip unsplit
+    assert not ops.gemm_swiglu(_t(rng.normal(size=(8, 64)), torch.bfloat16), _t(rng.normal(size=(512, 64)), torch.bfloat16), small)
+    big = torch.zeros(65, 2560, dtype=torch.bfloat16, device=DEV)      # too many rows for the streaming kernel
+    assert not ops.gemm_swiglu(_t(rng.normal(size=(65, 64)), torch.bfloat16), _t(rng.normal(size=(5120, 64)), torch.bfloat16), big)
+
+
 # ------------------------------------------------------------ partitioned decode attention
 @pytest.mark.parametrize("nh,nkv,hd", [(32, 4, 64), (8, 8, 64), (16, 4, 128), (32, 4, 128), (6, 2, 64), (5, 1, 128), (7, 7, 64)])
 @pytest.mark.parametrize("B", [8, 16, 64])
@@ -584,9 +602,9 @@ def test_partitioned_decode_attention(ops, nh, nkv, hd, B):
     P = _paged_problem(rng, lens, nh, nkv, hd, B, all_rows=False)
     ref = _ref_attention(P, nh, nkv, hd)
     R = P["R"]
-    for bound in (max(lens), 2048):                     # the launch may be sized for a longer context
-        out = torch.zeros(R, nh * hd, dtype=torch.bfloat16, device=DEV)
-        scratch = torch.zeros(ops.attention_decode_scratch(R, nh, hd, bound), dtype=torch.float32, device=DEV)
+    for bound in (max(lens), 2048, 2048):               # the launch may be sized for a longer context
+        out = torch.full((R, nh * hd), 9.0, dtype=torch.bfloat16, device=DEV)
+        scratch = torch.full((ops.attention_decode_scratch(R, nh, hd, bound),), float("nan"), dtype=torch.float32, device=DEV)
         ops.attention_decode(_t(P["Q"].reshape(R, nh * hd), torch.bfloat16), out, _t(P["Kc"], torch.bfloat16),
                              _vt(P["Vc"], torch.bfloat16), _t(P["tables"], torch.int32), P["max_blocks"],
                              _t(P["row_seq"], torch.int32), _t(P["ctx"], torch.int32), nh, nkv, hd, 1.0 / math.sqrt(hd),

@@ -1,5 +1,6 @@
 """The scheduler's decisions with a fake model (every sampled token is 42), as the reference
 tests them (tests/test_scheduler.cpp), plus portions of prompts under a token budget."""
+import numpy as np
 from kvcm_amd.cache.manager import HostCore
 
 
@@ -191,3 +192,26 @@ def test_chunked_preemption_recomputes_and_finishes():
     done, steps = run_to_completion(m, check_whole=False)
     assert len(done) == 5 and all(len(f.generated) == 30 for f in done)
     assert m.counters()["preemptions"] > 0 and m.blocks_in_use() == 0
+
+
+def test_plan_batch_carries_sampling_parameters_for_every_logit_row():
+    core = HostCore(num_blocks=32, block_size=4, max_seq_len=64, max_num_seqs=8, max_batched_tokens=64)
+    big = (1 << 63) + 12345                                  # a seed beyond the signed range keeps its bits
+    core.sched_add(7, [1, 2, 3], 4, temperature=0.5, sampler_seed=big)
+    core.sched_add(9, [4, 5, 6, 7, 8], 4, temperature=0.0, sampler_seed=3)
+    plan = core.schedule()
+    assert [p.id for p in plan] == [7, 9]
+    out = np.full(4096, 77, dtype=np.int32)
+    L = core.build_batch_from_plan(out, pad_logit_rows=4)
+    R = L.logit_rows_padded
+    assert L.logit_rows == 2 and R == 4 and L.sampling % 2 == 0 and L.sampling + 6 * R <= L.total
+    o = L.sampling
+    np.testing.assert_array_equal(out[o:o + R].view(np.float32), [0.5, 0.0, 0.0, 0.0])
+    np.testing.assert_array_equal(out[o + R:o + 2 * R], [0, 0, 0, 0])                    # index of the token to draw
+    np.testing.assert_array_equal(out[o + 2 * R:o + 4 * R].view(np.uint64), [big, 3, 0, 0])
+    np.testing.assert_array_equal(out[o + 4 * R:o + 6 * R].view(np.int64), [7, 9, 0, 0])
+    core.update([11, 12])
+    core.schedule()
+    L = core.build_batch_from_plan(out)
+    o, R = L.sampling, L.logit_rows_padded
+    np.testing.assert_array_equal(out[o + R:o + 2 * R], [1, 1])                          # second generated token
