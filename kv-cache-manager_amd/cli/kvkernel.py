@@ -1,0 +1,126 @@
+"""kvkernel: the decode attention kernels alone, over a grid of context lengths, batch sizes and
+page sizes, with the reference tool's flags and columns (src/main_kernel_bench.cpp:34-126):
+
+  --ctx 128,256,512,1024,2048  --batch 1,8,32,128  --block-size 16  --heads 32  --kv-heads 4
+  --head-dim 64  --iters 100  --out FILE.csv  [--graph]
+
+Four variants per point: v1 (one pass over the context per row and head) and v2 (contexts cut
+into partitions that run in parallel and are merged), each through a shuffled block table
+("paged") and through a table of consecutive pages ("contiguous").  5 warm-up calls, then
+``--iters`` timed calls between two events; GB/s = 2 * batch * ctx * kv_heads * head_dim * 2 bytes
+/ time, the keys and values a call has to read once.  Zero-filled bfloat16 cache, scale 0.125.
+With --graph (not in the reference) the timed calls are replays of one captured HIP graph that
+holds ``--iters`` calls, which takes the host's launch cost out of the figure.
+Columns: registers per lane, LDS per workgroup, workgroups per CU, occupancy (resident waves as a
+percentage of a CU's 32 wave slots), workgroups launched and how many rounds of the chip they make.
+"""
+import sys
+
+import numpy as np
+
+from .args import Args
+
+PEAK_GBS = 8000.0      # MI355X HBM3E
+WAVE_SLOTS_PER_CU = 32
+
+
+def _ints(s):
+    return [int(x) for x in s.split(",") if x]
+
+
+def main(argv=None):
+    a = Args(sys.argv[1:] if argv is None else argv)
+    ctxs, batches, blocks = _ints(a.str("ctx", "128,256,512,1024,2048")), _ints(a.str("batch", "1,8,32,128")), _ints(a.str("block-size", "16"))
+    heads, kvh, hd = a.i32("heads", 32), a.i32("kv-heads", 4), a.i32("head-dim", 64)
+    iters, out_csv = a.i32("iters", 100), a.str("out", "")
+    use_graph = a.flag("graph")
+    a.warn_unused()
+
+    import torch
+    from .. import ops
+    ops.lib()
+    dev = torch.device("cuda:0")
+    props = torch.cuda.get_device_properties(dev)
+    cus = props.multi_processor_count
+    print(f"device {props.name}, {cus} CUs, peak HBM bandwidth {PEAK_GBS:.1f} GB/s")
+    f = open(out_csv, "w") if out_csv else None
+    if f:
+        f.write("block_size,batch,ctx,variant,us,gbps,pct_peak,regs,lds_bytes,wgs_per_cu,occupancy_pct,wgs,rounds\n")
+    print("%5s %6s %6s %-16s %10s %9s %7s %5s %7s %6s %6s %7s" % ("B", "batch", "ctx", "variant", "us/call", "GB/s",
+                                                                   "%peak", "regs", "lds", "wg/CU", "occ%", "rounds"))
+    rng = np.random.default_rng(0)
+    bf16 = torch.bfloat16
+    for B in blocks:
+        for batch in batches:
+            for ctx in ctxs:
+                mb = (ctx + B - 1) // B
+                nb = batch * mb
+                K = torch.zeros(nb, kvh, B, hd, dtype=bf16, device=dev)
+                V = torch.zeros(nb, kvh, hd, B, dtype=bf16, device=dev)
+                Q = torch.zeros(batch, heads * hd, dtype=bf16, device=dev)
+                O = torch.zeros(batch, heads * hd, dtype=bf16, device=dev)
+                seq_tab = np.arange(nb, dtype=np.int32)
+                tables = {"paged": torch.tensor(rng.permutation(seq_tab), device=dev),
+                          "contiguous": torch.tensor(seq_tab, device=dev)}
+                rows = torch.arange(batch, dtype=torch.int32, device=dev)
+                lens = torch.full((batch,), ctx, dtype=torch.int32, device=dev)
+                v2_ok = ops.attention_decode_supported(heads, kvh, hd, bf16, B)
+                scratch = (torch.zeros(ops.attention_decode_scratch(batch, heads, hd, ctx), dtype=torch.float32, device=dev)
+                           if v2_ok else None)
+                nbytes = 2.0 * batch * ctx * kvh * hd * 2
+
+                def v1(tab):
+                    ops.attention(Q, O, K, V, tab, mb, rows, lens, heads, kvh, hd, 0.125)
+
+                def v2(tab):
+                    ops.attention_decode(Q, O, K, V, tab, mb, rows, lens, heads, kvh, hd, 0.125, ctx, scratch)
+
+                for version, call in (("v1", v1), ("v2", v2)):
+                    for layout in ("paged", "contiguous"):
+                        name = f"{layout}-{version}"
+                        if version == "v2" and not v2_ok:
+                            print("%5d %6d %6d %-16s %10s" % (B, batch, ctx, name, "unsupported"))
+                            continue
+                        tab = tables[layout]
+                        for _ in range(5):
+                            call(tab)
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        if use_graph:
+                            torch.cuda.synchronize()
+                            graph = torch.cuda.CUDAGraph()
+                            with torch.cuda.graph(graph):
+                                for _ in range(iters):
+                                    call(tab)
+                            graph.replay()
+                            torch.cuda.synchronize()
+                            e0.record()
+                            graph.replay()
+                            e1.record()
+                        else:
+                            e0.record()
+                            for _ in range(iters):
+                                call(tab)
+                            e1.record()
+                        e1.synchronize()
+                        us = 1e3 * e0.elapsed_time(e1) / iters
+                        gbs = nbytes / (us * 1e-6) / 1e9
+                        info = ops.attention_kernel_info(version, heads, kvh, hd)
+                        waves = info["threads"] // 64
+                        occ = 100.0 * info["workgroups_per_cu"] * waves / WAVE_SLOTS_PER_CU
+                        wgs = ((batch * heads + 3) // 4 if version == "v1"
+                               else kvh * batch * ((ctx + 255) // 256))
+                        rounds = wgs / float(max(info["workgroups_per_cu"], 1) * cus)
+                        print("%5d %6d %6d %-16s %10.2f %9.1f %6.1f%% %5d %6dB %6d %5.0f%% %7.2f" % (
+                            B, batch, ctx, name, us, gbs, 100 * gbs / PEAK_GBS, info["regs"], info["lds_bytes"],
+                            info["workgroups_per_cu"], occ, rounds))
+                        if f:
+                            f.write("%d,%d,%d,%s,%.3f,%.2f,%.2f,%d,%d,%d,%.1f,%d,%.3f\n" % (
+                                B, batch, ctx, name, us, gbs, 100 * gbs / PEAK_GBS, info["regs"], info["lds_bytes"],
+                                info["workgroups_per_cu"], occ, wgs, rounds))
+    if f:
+        f.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -210,6 +210,27 @@ int launch_decode(const void* q, int q_stride, void* out, int out_stride, const 
   return 0;
 }
 
+template <int HD, int GROUP>
+int decode_kernel_info(int* out) {
+  hipFuncAttributes a;
+  if (hipFuncGetAttributes(&a, reinterpret_cast<const void*>(&attention_decode_kernel<HD, GROUP>)) != hipSuccess) return -1;
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attention_decode_kernel<HD, GROUP>, kDecWaves * kWave, 0) != hipSuccess) return -1;
+  out[0] = a.numRegs; out[1] = static_cast<int>(a.sharedSizeBytes); out[2] = per_cu; out[3] = kDecWaves * kWave;
+  return 0;
+}
+
+template <int HD>
+int dispatch_info(int group, int* out) {
+  switch (group) {
+    case 1: return decode_kernel_info<HD, 1>(out); case 2: return decode_kernel_info<HD, 2>(out);
+    case 3: return decode_kernel_info<HD, 3>(out); case 4: return decode_kernel_info<HD, 4>(out);
+    case 5: return decode_kernel_info<HD, 5>(out); case 6: return decode_kernel_info<HD, 6>(out);
+    case 7: return decode_kernel_info<HD, 7>(out); case 8: return decode_kernel_info<HD, 8>(out);
+    default: return -1;
+  }
+}
+
 template <int HD>
 int dispatch_group(int group, const void* q, int q_stride, void* out, int out_stride, const void* kc, const void* vc,
                    const int* tables, int table_stride, const int* row_seq, const int* ctx_lens, int T, int nh,
@@ -234,6 +255,15 @@ int kvcm_attention_decode_supported(int nh, int nkv, int hd, int B) {
   if (nkv <= 0 || nh % nkv || B <= 0 || B % 8) return 0;
   const int g = nh / nkv;
   return (hd == 64 || hd == 128) && g >= 1 && g <= 8;
+}
+
+// What the compiled kernel for this shape uses: out = {vector registers per lane, bytes of LDS
+// per workgroup, workgroups that fit on one CU, threads per workgroup}.
+int kvcm_attention_decode_info(int nh, int nkv, int hd, int* out) {
+  KVCM_REQUIRE(kvcm_attention_decode_supported(nh, nkv, hd, 8), "attention_decode_info: unsupported shape");
+  const int rc = hd == 64 ? dispatch_info<64>(nh / nkv, out) : dispatch_info<128>(nh / nkv, out);
+  KVCM_REQUIRE(rc == 0, "attention_decode_info: the runtime gave no attributes");
+  return 0;
 }
 
 // Floats of scratch a launch needs: rows * heads * partitions * (head_dim + 2).

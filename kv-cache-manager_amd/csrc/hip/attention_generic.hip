@@ -120,6 +120,20 @@ __global__ void __launch_bounds__(kAttnWaves* kWave)
 
 using namespace kvcm;
 
+// out = {vector registers per lane, bytes of LDS per workgroup, workgroups that fit on one CU,
+// threads per workgroup} of the bfloat16 kernel at this head size.
+extern "C" int kvcm_attention_generic_info(int hd, int* out) {
+  hipFuncAttributes a;
+  const size_t lds = sizeof(float) * kAttnWaves * hd;
+  int per_cu = 0;
+  KVCM_REQUIRE(hipFuncGetAttributes(&a, reinterpret_cast<const void*>(&attention_generic_kernel<bf16_t>)) == hipSuccess &&
+                   hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attention_generic_kernel<bf16_t>,
+                                                                kAttnWaves * kWave, lds) == hipSuccess,
+               "attention_generic_info: the runtime gave no attributes");
+  out[0] = a.numRegs; out[1] = static_cast<int>(a.sharedSizeBytes + lds); out[2] = per_cu; out[3] = kAttnWaves * kWave;
+  return 0;
+}
+
 extern "C" int kvcm_attention_generic(const void* q, int dtype, int q_stride, void* out, int out_stride,
                                       const void* kcache, const void* vcache, const int* tables, int table_stride,
                                       const int* row_seq, const int* ctx_lens, int T, int nh, int nkv, int hd,

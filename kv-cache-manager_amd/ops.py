@@ -33,6 +33,8 @@ def _declare(lib):
     fn("kvcm_rmsnorm", vp, vp, i, vp, i, i, vp, vp, i, vp, i, i, i, f, i, vp)
     fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp, vp)
     fn("kvcm_rope_table", vp, vp, vp, i, i, vp)
+    fn("kvcm_attention_decode_info", i, i, i, vp)
+    fn("kvcm_attention_generic_info", i, vp)
     fn("kvcm_gemm_skinny_swiglu_supported", i, i, i)
     fn("kvcm_gemm_skinny_swiglu", vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_gemm_skinny_splits", i, i, i)
@@ -310,6 +312,17 @@ def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, n
 
 def attention_decode_supported(nh, nkv, hd, dtype, block_size=16):
     return dtype == torch.bfloat16 and bool(lib().kvcm_attention_decode_supported(nh, nkv, hd, block_size))
+
+
+def attention_kernel_info(variant, nh, nkv, hd):
+    """{"regs", "lds_bytes", "workgroups_per_cu", "threads"} of the compiled bfloat16 attention
+    kernel: variant "v1" (one pass per row and head) or "v2" (partitioned)."""
+    out = (C.c_int * 4)()
+    if variant == "v1":
+        _check(lib().kvcm_attention_generic_info(hd, out))
+    else:
+        _check(lib().kvcm_attention_decode_info(nh, nkv, hd, out))
+    return dict(regs=out[0], lds_bytes=out[1], workgroups_per_cu=out[2], threads=out[3])
 
 
 def attention_decode_scratch(rows, nh, hd, max_context):
