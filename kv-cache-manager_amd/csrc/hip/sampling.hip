@@ -33,14 +33,27 @@ __global__ void __launch_bounds__(kSampleThreads)
   }
   float best = -INFINITY;
   int idx = 0x7fffffff;
-#pragma unroll 4
-  for (int j = threadIdx.x; j < V; j += kSampleThreads) {
-    float v = row[j];
-    if (temp > 0.f) {
-      const float u = (float(mix64(key + uint64_t(j)) >> 41) + 0.5f) * (1.0f / 8388608.0f);  // exact in 24 bits
-      v = v / temp - logf(-logf(u));
+  // 16 values per thread and trip, all requested before the first is looked at (an index beyond
+  // the row reads its last element and is skipped afterwards): the row costs a few trips to
+  // memory, not one per element
+  constexpr int kBatch = 16;
+  for (int j0 = threadIdx.x; j0 < V; j0 += kSampleThreads * kBatch) {
+    float v[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int j = j0 + u * kSampleThreads;
+      v[u] = row[j < V ? j : V - 1];
     }
-    if (v > best || (v == best && j < idx)) { best = v; idx = j; }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int j = j0 + u * kSampleThreads;
+      float x = v[u];
+      if (temp > 0.f) {
+        const float r = (float(mix64(key + uint64_t(j)) >> 41) + 0.5f) * (1.0f / 8388608.0f);  // exact in 24 bits
+        x = x / temp - logf(-logf(r));
+      }
+      if (j < V && (x > best || (x == best && j < idx))) { best = x; idx = j; }
+    }
   }
   __shared__ float sv[kSampleThreads / kWave];
   __shared__ int si[kSampleThreads / kWave];
