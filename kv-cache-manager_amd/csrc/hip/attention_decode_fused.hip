@@ -1,0 +1,334 @@
+// One launch for what a decode row needs between the QKV projection and the output projection:
+// sum the projection's split-K partial sums, rotate q and k, store the new k and v to their page,
+// and attend over the whole context.  The reference runs these as separate kernels
+// (src/model/llama.cpp:108-116: rope, reshape_and_cache, paged_attention); on this chip a
+// decode step is bound by the number of dependent launches, not by bytes, so they are one here.
+//
+// One workgroup per (kv head, row) serves the row's whole query group.  After a common prologue
+// (q to LDS, new key and value to their page) its four waves work on their own: the context is
+// walked in chunks of 256 tokens, wave w takes tokens 64 w .. 64 w + 63 of every chunk, keeps its
+// own running maximum, sum and output, and asks for the keys and values of its next chunk before
+// it computes the current one.  No barrier inside the loop; the four partial results are merged
+// through LDS at the end, always in wave order.
+//
+// Both products run on the matrix cores, transposed: S^T = K Q^T puts one query head in each
+// accumulator column, so a lane's softmax concerns one head only and its eight probabilities of a
+// 32-token group are, packed to bfloat16, exactly the B operand of O^T += V^T P^T.  Scores never
+// touch LDS.  The row -> token assignment of the two key tiles of a group is chosen so that those
+// eight tokens are consecutive, which is what the transposed value pages ([dim][slot]) offer as
+// 16-byte fragments.
+// Only steps whose rows all belong to different sequences may use it: a row's new key is written
+// by its own workgroup and read by nobody else.
+#include <cfloat>
+
+#include "common.h"
+
+namespace kvcm {
+
+constexpr int kFusWaves = 4;
+constexpr int kFusChunk = 256;
+constexpr float kFusNone = -1.0e30f;   // "no score yet": finite, so that differences stay finite
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2v;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2v;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+union FragF {
+  uint4 u;
+  bf16x8 v;
+};
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+  union { bf16x2v v; uint32_t u; } r;
+  r.v = __builtin_convertvector(f32x2v{a, b}, bf16x2v);   // one v_cvt_pk_bf16_f32, round to nearest even
+  return r.u;
+}
+
+template <int HD, int GROUP>
+__global__ void __launch_bounds__(kFusWaves* kWave)
+    attention_decode_fused_kernel(const float* __restrict__ partials, int S, size_t pstride,
+                                  const uint16_t* __restrict__ qkv, int qkv_stride,
+                                  const float2* __restrict__ cos_sin, const int* __restrict__ slots,
+                                  uint16_t* __restrict__ kcache, uint16_t* __restrict__ vcache,
+                                  const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
+                                  const int* __restrict__ ctx_lens, int nh, int nkv, int B, float scale,
+                                  uint16_t* __restrict__ out, int out_stride) {
+  constexpr int KSTEPS = HD / 32;   // matrix instructions per 16-token tile of scores
+  constexpr int DT = HD / 16;       // 16-dim tiles of the output
+  constexpr int HALF = HD / 2;
+  const int kvh = blockIdx.x, row = blockIdx.y;
+  const int ctx = ctx_lens[row];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds[GROUP][HD];
+  __shared__ __attribute__((aligned(16))) float red[kFusWaves][16][HD + 4];
+  __shared__ float w_max[kFusWaves][16], w_sum[kFusWaves][16];
+
+  if (ctx <= 0) {   // a padding row: zeros, nothing read or stored
+    for (int i = threadIdx.x; i < GROUP * HD; i += kFusWaves * kWave)
+      out[size_t(row) * out_stride + size_t(kvh) * GROUP * HD + i] = 0;
+    return;
+  }
+  const int* table = tables + size_t(row_seq[row]) * table_stride;
+  const size_t head_elems = size_t(B) * HD, page_elems = head_elems * nkv;
+  const int nchunks = (ctx + kFusChunk - 1) / kFusChunk;
+  const int last = nchunks - 1;
+
+  // Where this wave's 64 tokens of chunk c live: lane l looks up token 64 w + l, the offset of its
+  // key row and of its group of 8 value slots, both inside this kv head's part of the cache and in
+  // units of 8 elements.  Tokens beyond the context point at the last valid token (keys) or the
+  // last valid group of 8 (values), so that every load below is unconditional; what they bring is
+  // masked out.  The lanes that need an offset get it by a shuffle.
+  struct Where { uint32_t k, v; };
+  auto lookup = [&](int c) {
+    const int t0 = c * kFusChunk + wave * 64 + lane;
+    const int t = min(t0, ctx - 1), tv = min(t0, (ctx - 1) & ~7);
+    const int pk = table[t / B], pv = table[tv / B];
+    Where w;
+    w.k = uint32_t((size_t(pk) * page_elems + kvh * head_elems + size_t(t % B) * HD) / 8);
+    w.v = uint32_t((size_t(pv) * page_elems + kvh * head_elems + tv % B) / 8);
+    return w;
+  };
+  // lookups run two chunks ahead of the computation, so that their trip to memory is never waited for
+  Where wha = lookup(0), whb = lookup(min(1, last));
+
+  // ---- prologue: this row's q (GROUP heads), k and v (one kv head) from the projection
+  const int width = (nh + 2 * nkv) * HD;
+  const float* prow = partials ? partials + size_t(row) * width : nullptr;
+  const uint16_t* rrow = qkv + size_t(row) * qkv_stride;
+  auto value = [&](int col) {
+    if (!prow) return bf16_bits_to_float(rrow[col]);
+    float a = 0.f;
+    for (int s0 = 0; s0 < S; s0 += 4) {   // four loads requested together; a split beyond S adds nothing
+      float p[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) p[j] = prow[(s0 + j < S ? s0 + j : S - 1) * pstride + col];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a += s0 + j < S ? p[j] : 0.f;
+    }
+    return bf16_bits_to_float(float_to_bf16_bits(a));   // the projection's result is a bfloat16 value
+  };
+  const int slot = slots ? slots[row] : -1;
+  const size_t page = slot >= 0 ? slot / B : 0;
+  const int off = slot >= 0 ? slot % B : 0;
+  for (int item = threadIdx.x; item < (GROUP + 2) * HALF; item += kFusWaves * kWave) {
+    const int h = item / HALF, j = item % HALF;   // 0..GROUP-1: q heads, GROUP: k, GROUP+1: v
+    const int col = (h < GROUP ? (kvh * GROUP + h) * HD : h == GROUP ? (nh + kvh) * HD : (nh + nkv + kvh) * HD) + j;
+    float a = value(col), b = value(col + HALF);
+    if (h <= GROUP && cos_sin) {
+      const float2 t2 = cos_sin[size_t(row) * HALF + j];
+      rotate_pair(a, b, t2.x, t2.y);
+    }
+    const uint16_t ab = float_to_bf16_bits(a), bb = float_to_bf16_bits(b);
+    if (h < GROUP) {
+      q_lds[h][j] = ab;
+      q_lds[h][j + HALF] = bb;
+    } else if (slot >= 0) {
+      if (h == GROUP) {
+        uint16_t* kr = kcache + ((page * nkv + kvh) * B + off) * HD;
+        kr[j] = ab;
+        kr[j + HALF] = bb;
+      } else {   // values lie transposed inside the page: [dim][slot]
+        uint16_t* vr = vcache + (page * nkv + kvh) * size_t(HD) * B + off;
+        vr[size_t(j) * B] = ab;
+        vr[size_t(j + HALF) * B] = bb;
+      }
+    }
+  }
+  __syncthreads();   // q in LDS; the new key and value are stored before any wave of this workgroup loads them
+
+  const int n16 = lane % 16, kq = lane / 16;
+  // B operand of S^T = K Q^T: lane = (query head n16, dims 8 kq .. + 7 of every 32); heads beyond the group are zero
+  FragF qf[KSTEPS];
+#pragma unroll
+  for (int c = 0; c < KSTEPS; ++c) {
+    qf[c].u = *reinterpret_cast<const uint4*>(&q_lds[n16 < GROUP ? n16 : 0][c * 32 + kq * 8]);
+    if (n16 >= GROUP) qf[c].u = uint4{0u, 0u, 0u, 0u};
+  }
+
+  // A chunk's operands for this wave: two groups of 32 tokens; a group's keys as two 16-row tiles
+  // whose row r holds token 8 (r / 4) + 4 tile + r % 4 of the group, its values as [dim][8 tokens].
+  struct Chunk {
+    FragF k[2][2][KSTEPS];
+    FragF v[2][DT];
+  };
+  auto request = [&](const Where& wh, Chunk& ch) {
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int tok = g * 32 + 8 * (n16 / 4) + 4 * t + n16 % 4;
+        const uint16_t* kp = kcache + (size_t(__shfl(wh.k, tok, kWave)) << 3) + kq * 8;
+#pragma unroll
+        for (int c = 0; c < KSTEPS; ++c) ch.k[g][t][c].u = *reinterpret_cast<const uint4*>(kp + c * 32);
+      }
+      const uint16_t* vp = vcache + (size_t(__shfl(wh.v, g * 32 + 8 * kq, kWave)) << 3) + size_t(n16) * B;
+#pragma unroll
+      for (int d = 0; d < DT; ++d) ch.v[g][d].u = *reinterpret_cast<const uint4*>(vp + size_t(d) * 16 * B);
+    }
+  };
+
+  // running state of this lane's head (n16): maximum (log2 domain), this lane's share of the sum,
+  // and O^T (column = head, rows = dims 16 d + 4 kq + i)
+  float m_run = kFusNone, l_run = 0.f;
+  f32x4 o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float scale2 = scale * 1.4426950408889634f;
+
+  auto compute = [&](int c, const Chunk& ch) {
+    const int base = c * kFusChunk + wave * 64 + 8 * kq;   // this lane's first token of group 0
+    float s[2][8];
+    float mx = kFusNone;
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < KSTEPS; ++k) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ch.k[g][t][k].v, qf[k].v, acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {   // accumulator row 4 kq + i of tile t = token 8 kq + 4 t + i of the group
+          const bool valid = base + g * 32 + 4 * t + i < ctx;
+          s[g][4 * t + i] = valid ? acc[i] * scale2 : kFusNone;
+          mx = fmaxf(mx, s[g][4 * t + i]);
+        }
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = exp2f(m_run - m_new);
+    m_run = m_new;
+    float sum = 0.f;
+    FragF pf[2];
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      float p[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        p[j] = s[g][j] > 0.5f * kFusNone ? exp2f(s[g][j] - m_new) : 0.f;
+        sum += p[j];
+      }
+      pf[g].u = uint4{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3]), pack2_bf16(p[4], p[5]), pack2_bf16(p[6], p[7])};
+    }
+    l_run = l_run * alpha + sum;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
+#pragma unroll
+      for (int g = 0; g < 2; ++g) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ch.v[g][d].v, pf[g].v, o[d], 0, 0, 0);
+    }
+  };
+
+  // The chunk after the last repeats the last one, so that no load sits behind a branch; what it
+  // brings is never used.
+  Chunk cha, chb;
+  request(wha, cha);
+  wha = lookup(min(2, last));
+  for (int c = 0; c < nchunks; c += 2) {
+    request(whb, chb);                 // chunk c + 1
+    whb = lookup(min(c + 3, last));
+    __builtin_amdgcn_sched_barrier(0);
+    compute(c, cha);
+    if (c + 1 >= nchunks) break;
+    request(wha, cha);                 // chunk c + 2
+    wha = lookup(min(c + 4, last));
+    __builtin_amdgcn_sched_barrier(0);
+    compute(c + 1, chb);
+  }
+
+  // ---- the four waves' results, merged in wave order: out = sum_w e_w o_w / sum_w e_w l_w, e_w = 2^(m_w - m)
+  l_run += __shfl_xor(l_run, 16, kWave);
+  l_run += __shfl_xor(l_run, 32, kWave);
+  if (kq == 0) { w_max[wave][n16] = m_run; w_sum[wave][n16] = l_run; }
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][n16][d * 16 + 4 * kq + i] = o[d][i];
+  __syncthreads();
+  for (int i = threadIdx.x; i < GROUP * HD; i += kFusWaves * kWave) {
+    const int g = i / HD, d = i % HD;
+    float m = w_max[0][g];
+#pragma unroll
+    for (int w = 1; w < kFusWaves; ++w) m = fmaxf(m, w_max[w][g]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < kFusWaves; ++w) {
+      const float e = exp2f(w_max[w][g] - m);
+      num = fmaf(e, red[w][g][d], num);
+      den = fmaf(e, w_sum[w][g], den);
+    }
+    out[size_t(row) * out_stride + size_t(kvh * GROUP + g) * HD + d] = float_to_bf16_bits(num / den);
+  }
+}
+
+template <int HD>
+int dispatch_fused(int group, dim3 grid, hipStream_t s, const float* partials, int S, size_t pstride, const uint16_t* qkv,
+                   int qkv_stride, const float2* cos_sin, const int* slots, uint16_t* kc, uint16_t* vc,
+                   const int* tables, int table_stride, const int* row_seq, const int* ctx_lens, int nh, int nkv, int B,
+                   float scale, uint16_t* out, int out_stride) {
+#define KVCM_FUSED(G)                                                                                                   \
+  case G:                                                                                                               \
+    attention_decode_fused_kernel<HD, G><<<grid, kFusWaves * kWave, 0, s>>>(partials, S, pstride, qkv, qkv_stride,      \
+                                                                           cos_sin, slots, kc, vc, tables, table_stride, \
+                                                                           row_seq, ctx_lens, nh, nkv, B, scale, out,   \
+                                                                           out_stride);                                 \
+    return 0
+  switch (group) {
+    KVCM_FUSED(1); KVCM_FUSED(2); KVCM_FUSED(3); KVCM_FUSED(4); KVCM_FUSED(5); KVCM_FUSED(6); KVCM_FUSED(7); KVCM_FUSED(8);
+    default: return -1;
+  }
+#undef KVCM_FUSED
+}
+
+}  // namespace kvcm
+
+using namespace kvcm;
+
+extern "C" {
+
+// 1 when this kernel takes the shape (bfloat16 only), else 0.
+int kvcm_attention_decode_fused_supported(int nh, int nkv, int hd, int B) {
+  if (nkv <= 0 || nh % nkv || B <= 0 || B % 8) return 0;
+  const int g = nh / nkv;
+  return (hd == 64 || hd == 128) && g >= 1 && g <= 8;
+}
+
+// Rows of T different sequences.  The projection's result is either `partials` (split-K sums
+// [S][T][width], width = (nh + 2 nkv) * hd, added in split order) or, when partials is null, the
+// bfloat16 rows `qkv`.  cos_sin [T][hd/2] (cos, sin) rotates q and k by pairs (j, j + hd/2); null:
+// no rotation.  slots [T]: where the row's key and value go (page * B + offset; negative or a
+// null array: nothing is stored and the context is read as it is).  ctx_lens[t] includes the
+// row's own token.
+int kvcm_attention_decode_fused(const float* partials, int S, const void* qkv, int qkv_stride, const float* cos_sin,
+                                const int* slots, void* kcache, void* vcache, const int* tables, int table_stride,
+                                const int* row_seq, const int* ctx_lens, int T, int nh, int nkv, int hd, int B,
+                                float scale, void* out, int out_stride, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(kvcm_attention_decode_fused_supported(nh, nkv, hd, B),
+               "attention_decode_fused: unsupported shape heads=%d kv_heads=%d head_dim=%d page=%d", nh, nkv, hd, B);
+  KVCM_REQUIRE(T > 0 && T <= 65535 && nkv <= 65535, "attention_decode_fused: bad row count %d", T);
+  KVCM_REQUIRE(partials ? (S >= 1 && S <= 64) : (qkv != nullptr && qkv_stride >= (nh + 2 * nkv) * hd),
+               "attention_decode_fused: no projection result (splits %d, row stride %d)", S, qkv_stride);
+  KVCM_REQUIRE(out_stride >= nh * hd, "attention_decode_fused: output rows too short");
+  KVCM_REQUIRE(reinterpret_cast<uintptr_t>(kcache) % 16 == 0 && reinterpret_cast<uintptr_t>(vcache) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(cos_sin) % 8 == 0,
+               "attention_decode_fused: operands must be 16-byte aligned");
+  const size_t pstride = size_t(T) * (nh + 2 * nkv) * hd;
+  const dim3 grid(nkv, T);
+  int rc;
+  if (hd == 64)
+    rc = dispatch_fused<64>(nh / nkv, grid, s, partials, S, pstride, static_cast<const uint16_t*>(qkv), qkv_stride,
+                            reinterpret_cast<const float2*>(cos_sin), slots, static_cast<uint16_t*>(kcache),
+                            static_cast<uint16_t*>(vcache), tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale,
+                            static_cast<uint16_t*>(out), out_stride);
+  else
+    rc = dispatch_fused<128>(nh / nkv, grid, s, partials, S, pstride, static_cast<const uint16_t*>(qkv), qkv_stride,
+                             reinterpret_cast<const float2*>(cos_sin), slots, static_cast<uint16_t*>(kcache),
+                             static_cast<uint16_t*>(vcache), tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale,
+                             static_cast<uint16_t*>(out), out_stride);
+  KVCM_REQUIRE(rc == 0, "attention_decode_fused: no kernel for group size %d", nh / nkv);
+  return launch_status("attention_decode_fused");
+}
+
+}  // extern "C"

@@ -34,6 +34,15 @@ template <class T> __device__ __forceinline__ float round_to(float v);
 template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }
 template <> __device__ __forceinline__ float round_to<bf16_t>(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
 
+// (a, b) rotated by the angle whose cosine and sine are given.  One explicit sequence of
+// operations, shared by every kernel that rotates, so that all of them give the same bits.
+__device__ __forceinline__ void rotate_pair(float& a, float& b, float cs, float sn) {
+  const float ra = __fmaf_rn(a, cs, -__fmul_rn(b, sn));
+  const float rb = __fmaf_rn(b, cs, __fmul_rn(a, sn));
+  a = ra;
+  b = rb;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

@@ -253,8 +253,8 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
           sincosf(pos * inv_freq[j], &sn, &cs);
         }
         const int c = h * hd + j;
-        const float a = value(c), b = value(c + half);
-        const float ra = a * cs - b * sn, rb = b * cs + a * sn;
+        float ra = value(c), rb = value(c + half);
+        rotate_pair(ra, rb, cs, sn);
         if (!prow || is_q) {
           store_f(row + c, ra);
           store_f(row + c + half, rb);
@@ -327,10 +327,7 @@ __global__ void __launch_bounds__(256)
       for (int e = 0; e < 8; ++e) sincosf(pos * inv_freq[j0 + e], &sn[e], &cs[e]);
     }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float ra = a[e] * cs[e] - b[e] * sn[e], rb = b[e] * cs[e] + a[e] * sn[e];
-      a[e] = ra; b[e] = rb;
-    }
+    for (int e = 0; e < 8; ++e) rotate_pair(a[e], b[e], cs[e], sn[e]);
     store4<T>(row + j0, a); store4<T>(row + j0 + 4, a + 4);
     store4<T>(row + half + j0, b); store4<T>(row + half + j0 + 4, b + 4);
   }

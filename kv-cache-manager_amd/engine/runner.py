@@ -134,6 +134,13 @@ class StepContext:
     def attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window=0):
         self.runner.attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window)
 
+    def decode_attention_fused(self, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):
+        """Rotation by ``cos_sin``, page write at ``slots`` and attention in one launch, straight
+        from the QKV projection's result; False when this step or shape has no such kernel (then
+        the caller runs them one after the other: the same values up to rounding)."""
+        return self.runner.decode_attention_fused(self, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window,
+                                                  cos_sin, slots)
+
 
 class ModelRunner:
     def __init__(self, model: Model, core: HostCore, storages, limits: ModelLimits, dtype, device, attn="auto"):
@@ -163,12 +170,30 @@ class ModelRunner:
     # Rows up to which a step is treated as decode-shaped by the partitioned attention kernel.
     DECODE_ATTENTION_MAX_ROWS = 512
 
+    # The one-launch decode kernel walks a row's context chunk by chunk inside one workgroup:
+    # right when contexts are moderate or there are enough rows to fill the chip; a few rows with
+    # very long contexts are better cut into partitions that run in parallel.
+    FUSED_DECODE_MAX_CONTEXT = 4096
+    FUSED_DECODE_FULL_CHIP = 192
+
+    def decode_attention_fused(self, step, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):
+        ops = self.ops
+        if (self.attn != "auto" or window != 0 or step.max_run != 1 or out.dtype != torch.bfloat16
+                or step.rows > self.DECODE_ATTENTION_MAX_ROWS
+                or not ops.attention_decode_fused_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
+            return False
+        if step.max_context_bound > self.FUSED_DECODE_MAX_CONTEXT and step.rows * nkv < self.FUSED_DECODE_FULL_CHIP:
+            return False
+        ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
+                                   step.ctx_lens, nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=step.rows)
+        return True
+
     def attention(self, step, q, out, kcache, vcache, g, nh, nkv, hd, scale, window):
         """attn = "v1": the generic kernel, one pass over the whole context per (row, head); "v2" and
         "auto": for bfloat16, decode-shaped steps take the kernel that cuts contexts into partitions
         and merges them, steps with runs of positions take the tiled kernel; "v2" insists on the
-        partitioned kernel for decode steps.  The 32-bit path always takes v1, whose result does
-        not depend on the batch."""
+        partitioned kernel for decode steps, "auto" prefers the one-launch kernel above where it
+        applies.  The 32-bit path always takes v1, whose result does not depend on the batch."""
         ops = self.ops
         partitioned = (self.attn != "v1" and window == 0 and step.max_run == 1
                        and step.rows <= self.DECODE_ATTENTION_MAX_ROWS

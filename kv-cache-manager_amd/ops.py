@@ -34,6 +34,8 @@ def _declare(lib):
     fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp, vp)
     fn("kvcm_rope_table", vp, vp, vp, i, i, vp)
     fn("kvcm_attention_decode_info", i, i, i, vp)
+    fn("kvcm_attention_decode_fused_supported", i, i, i, i)
+    fn("kvcm_attention_decode_fused", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, vp, i, vp)
     fn("kvcm_attention_generic_info", i, vp)
     fn("kvcm_gemm_skinny_swiglu_supported", i, i, i)
     fn("kvcm_gemm_skinny_swiglu", vp, vp, vp, i, i, i, i, i, i, i, vp)
@@ -347,6 +349,44 @@ def attention_decode(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_
                                        _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh, nkv, hd,
                                        kcache.shape[2], float(scale), int(max_context), _ptr(scratch), scratch.numel(),
                                        _stream()))
+
+
+def attention_decode_fused_supported(nh, nkv, hd, dtype, block_size=16):
+    return dtype == torch.bfloat16 and bool(lib().kvcm_attention_decode_fused_supported(nh, nkv, hd, block_size))
+
+
+def attention_decode_fused(projection, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, nh, nkv, hd, scale,
+                           cos_sin=None, slots=None, rows=None):
+    """One launch from the QKV projection to the attention output for rows of different sequences
+    (bfloat16): ``projection`` is the fused [q | k | v] rows or their un-added split-K sums
+    (PartialSums); q and k are rotated by ``cos_sin`` [rows, hd/2, 2] (None: not rotated), k and v
+    stored at ``slots`` (None: nothing stored), and every row attends over its whole context."""
+    partial = isinstance(projection, PartialSums)
+    rows_t = projection.out if partial else projection
+    T = rows_t.shape[0] if rows is None else rows
+    _dev(rows_t, out, kcache, vcache, tables, row_seq, ctx_lens, cos_sin, slots)
+    _rows2d(out, "out")
+    width = (nh + 2 * nkv) * hd
+    _need(out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "attention_decode_fused is bfloat16 only")
+    _check_caches(kcache, vcache, nkv, hd)
+    if partial:
+        _need(projection.cols == width and projection.rows == T, "the partial sums are not [splits, rows, (nh + 2 nkv) * hd]")
+    else:
+        _rows2d(rows_t, "qkv")
+        _need(rows_t.dtype == torch.bfloat16 and rows_t.shape[1] >= width and rows_t.shape[0] >= T, "qkv must be bfloat16 [rows, (nh + 2 nkv) * hd]")
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.numel() >= T * hd, "cos_sin must be float32 [rows, hd/2, 2]")
+    if slots is not None:
+        _i32(slots, "slots", T)
+    _i32(row_seq, "row_seq", T)
+    _i32(ctx_lens, "ctx_lens", T)
+    _i32(tables, "tables")
+    _need(out.shape[0] >= T and out.shape[1] >= nh * hd, "out must be [rows, nh * hd]")
+    _check(lib().kvcm_attention_decode_fused(
+        _ptr(projection.data) if partial else 0, projection.splits if partial else 0,
+        0 if partial else _ptr(rows_t), 0 if partial else rows_t.stride(0), _ptr(cos_sin), _ptr(slots), _ptr(kcache),
+        _ptr(vcache), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh, nkv, hd, kcache.shape[2],
+        float(scale), _ptr(out), out.stride(0), _stream()))
 
 
 def attention_prefill_supported(nh, nkv, hd, dtype, block_size=16):

@@ -57,21 +57,26 @@ class Rotary(PositionEncoding):
 
     accepts_partial_sums = True
 
+    def rotation_table(self, step, head_dim):
+        """(cos, sin) of every row's angles [rows, head_dim/2, 2], or None where the step cannot
+        share work between layers.  The angles depend on the row only: the first layer of a step
+        computes them, the others (same theta and dim) read them."""
+        shared = getattr(step, "shared", None)
+        if shared is None or head_dim != self.params["dim"]:
+            return None
+        key = ("rotary", float(self.params["theta"]), head_dim)
+        table = shared.get(key)
+        if table is None:
+            table = step.ws("rotary_cos_sin_%d" % head_dim, (step.rows, head_dim), torch.float32).view(step.rows, head_dim // 2, 2)
+            self.ctx.ops.rope_table(step.positions, self.inv_freq, table, rows=step.rows)
+            shared[key] = table
+        return table
+
     def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None, source=None):
         if head_dim != self.params["dim"]:
             raise ValueError("rotary: this kernel rotates the whole head (dim must equal head_dim)")
         k, v = cache if cache is not None else (None, None)
-        # the angles depend on the row only: the first layer of a step computes cos and sin, the
-        # others (same theta and dim) read them
-        table = None
-        shared = getattr(step, "shared", None)
-        if shared is not None:
-            key = ("rotary", float(self.params["theta"]), head_dim)
-            table = shared.get(key)
-            if table is None:
-                table = step.ws("rotary_cos_sin_%d" % head_dim, (step.rows, head_dim), torch.float32).view(step.rows, head_dim // 2, 2)
-                self.ctx.ops.rope_table(step.positions, self.inv_freq, table, rows=step.rows)
-                shared[key] = table
+        table = self.rotation_table(step, head_dim)
         self.ctx.ops.rope_cache(qkv, num_heads, num_kv_heads, head_dim, positions=step.positions,
                                 inv_freq=self.inv_freq, slots=slots, kcache=k, vcache=v,
                                 block_size=self.ctx.block_size, rows=step.rows, source=source, cos_sin=table)
@@ -80,6 +85,8 @@ class Rotary(PositionEncoding):
 
 @POSITIONS.register("none")
 class NoPosition(PositionEncoding):
+    rotates = False
+
     def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None):
         return False
 
@@ -122,13 +129,26 @@ class GQAAttention(Mixer):
         res = _linear(self.ctx, step, h, self.w["wqkv"], "qkv", keep_partial=fused)
         qkv = step.ws("qkv", (step.rows, self.q_dim + 2 * self.kv_dim))
         slots = step.slots(g) if self.cache_owner else None
+        attn = step.ws("attn", (step.rows, self.q_dim))
+        # decode-shaped steps: rotation, page write and attention in one launch, where the position
+        # encoding is a rotation by pairs (or none) and the step offers that kernel
+        fused_attention = getattr(step, "decode_attention_fused", None)
+        if fused_attention is not None:
+            pos, table, fusable = self.position, None, False
+            if getattr(pos, "rotates", True) is False:
+                fusable = True
+            elif hasattr(pos, "rotation_table"):
+                table = pos.rotation_table(step, self.hd)
+                fusable = table is not None
+            if fusable and fused_attention(res, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window,
+                                           table, slots):
+                return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
         extra = {"source": res} if hasattr(res, "materialize") else {}
         stored = self.position.apply(step, qkv, self.nh, self.nkv, self.hd,
                                      cache=(kc, vc) if self.cache_owner else None, slots=slots, **extra)
         if self.cache_owner and not stored:
             ops.rope_cache(qkv, self.nh, self.nkv, self.hd, slots=slots, kcache=kc, vcache=vc,
                            block_size=self.ctx.block_size, rows=step.rows)
-        attn = step.ws("attn", (step.rows, self.q_dim))
         step.attention(qkv, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window)
         return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
 

@@ -644,6 +644,94 @@ def test_partitioned_decode_attention_padding_rows_and_far_key(ops):
     assert not ops.attention_decode_supported(32, 4, 64, torch.float32)
 
 
+# ------------------------------------------ rotation + page write + attention in one launch
+@pytest.mark.parametrize("nh,nkv,hd,B", [(32, 4, 64, 16), (8, 8, 64, 8), (16, 4, 128, 16), (6, 2, 64, 64), (5, 1, 128, 16)])
+@pytest.mark.parametrize("source", ["rows", "partial_sums"])
+def test_fused_decode_attention_equals_rope_write_attend(ops, nh, nkv, hd, B, source):
+    rng = np.random.default_rng(nh + hd + B)
+    lens = [700, 256, 257, 1, 255, 33, 513, 1024]       # 1..4 chunks, chunk edges, the first token of a sequence
+    P = _paged_problem(rng, lens, nh, nkv, hd, B, all_rows=False)
+    R, W = P["R"], (nh + 2 * nkv) * hd
+    pos = (P["ctx"] - 1).astype(np.int32)
+    k_new = _bf16_grid(rng.normal(size=(R, nkv, hd)))
+    v_new = _bf16_grid(rng.normal(size=(R, nkv, hd)))
+    rows = np.concatenate([P["Q"].reshape(R, -1), k_new.reshape(R, -1), v_new.reshape(R, -1)], axis=1)
+    slots = np.array([P["tables"][s, p // B] * B + p % B for s, p in zip(P["row_seq"], pos)], dtype=np.int32)
+    inv = _t(_inv_freq(hd, 1e4), torch.float32)
+    table = torch.empty(R, hd // 2, 2, device=DEV)
+    ops.rope_table(_t(pos, torch.int32), inv, table)
+    args = dict(tables=_t(P["tables"], torch.int32), row_seq=_t(P["row_seq"], torch.int32), ctx=_t(P["ctx"], torch.int32))
+
+    # the last token of every sequence is not in the cache yet: both ways have to put it there
+    def caches():
+        kc, vc = P["Kc"].copy(), P["Vc"].copy()
+        for s_, p_ in zip(P["row_seq"], pos):
+            kc[P["tables"][s_, p_ // B], :, p_ % B] = 0
+            vc[P["tables"][s_, p_ // B], :, p_ % B] = 0
+        return _t(kc, torch.bfloat16), _vt(vc, torch.bfloat16)
+
+    # separately: rotation + page write, then the one-pass kernel
+    kc1, vc1 = caches()
+    q1 = _t(rows, torch.bfloat16)
+    ops.rope_cache(q1, nh, nkv, hd, positions=_t(pos, torch.int32), inv_freq=inv, slots=_t(slots, torch.int32),
+                   kcache=kc1, vcache=vc1, block_size=B, cos_sin=table)
+    want = torch.zeros(R, nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention(q1, want, kc1, vc1, args["tables"], P["max_blocks"], args["row_seq"], args["ctx"], nh, nkv, hd, 1.0 / math.sqrt(hd))
+
+    kc2, vc2 = caches()
+    if source == "rows":
+        proj = _t(rows, torch.bfloat16)
+    else:   # three splits whose sum is the row, none of them on the bfloat16 grid
+        noise = rng.normal(size=(2, R, W)) * 0.37
+        parts = np.stack([noise[0], noise[1], rows - noise[0] - noise[1]]).astype(np.float32)
+        parts[2] += (rows - parts.astype(np.float64).sum(0)).astype(np.float32)
+        proj = ops.PartialSums(_t(parts, torch.float32), 3, R, W, torch.zeros(R, W, dtype=torch.bfloat16, device=DEV))
+        ref_rows = proj.materialize().clone()
+        ops.rope_cache(ref_rows, nh, nkv, hd, positions=_t(pos, torch.int32), inv_freq=inv, slots=_t(slots, torch.int32),
+                       kcache=kc1, vcache=vc1, block_size=B, cos_sin=table)
+        ops.attention(ref_rows, want, kc1, vc1, args["tables"], P["max_blocks"], args["row_seq"], args["ctx"], nh, nkv, hd,
+                      1.0 / math.sqrt(hd))
+    got = torch.full((R, nh * hd), 5.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode_fused(proj, got, kc2, vc2, args["tables"], P["max_blocks"], args["row_seq"], args["ctx"], nh, nkv, hd,
+                               1.0 / math.sqrt(hd), cos_sin=table, slots=_t(slots, torch.int32))
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)                      # the same keys and values reached the pages
+    np.testing.assert_allclose(_np(got), _np(want), atol=2 ** -6, rtol=0)        # two kernels, a rounding apart
+
+
+def test_fused_decode_attention_against_plain_far_key_padding_and_no_store(ops):
+    rng = np.random.default_rng(91)
+    nh, nkv, hd, B = 8, 2, 64, 16
+    P = _paged_problem(rng, [900, 300], nh, nkv, hd, B, all_rows=False)
+    far = 3                                                   # in the first chunk, while the row spans four
+    P["Q"][0, 5] = 0.0
+    P["Q"][0, 5, 7] = 40.0
+    kvec = np.zeros(hd)
+    kvec[7] = 40.0
+    P["Kl"][0][far, 1] = kvec
+    P["Kc"][P["tables"][0, far // B], 1, far % B] = kvec
+    ref = _ref_attention(P, nh, nkv, hd, scale=1.0)
+    # no rotation, nothing stored: the cache already holds every token, k and v of the rows are ignored
+    rows = np.concatenate([P["Q"].reshape(2, -1), rng.normal(size=(2, 2 * nkv * hd))], axis=1)
+    rows = np.concatenate([rows, np.ones((1, rows.shape[1]))])                  # + a padding row without context
+    ctx = np.array([900, 300, 0], dtype=np.int32)
+    kc, vc = _t(P["Kc"], torch.bfloat16), _vt(P["Vc"], torch.bfloat16)
+    kc0, vc0 = kc.clone(), vc.clone()
+    out = torch.full((3, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode_fused(_t(rows, torch.bfloat16), out, kc, vc, _t(P["tables"], torch.int32), P["max_blocks"],
+                               _t([0, 1, 0], torch.int32), _t(ctx, torch.int32), nh, nkv, hd, 1.0)
+    got = _np(out).reshape(3, nh, hd)
+    np.testing.assert_allclose(got[:2], ref, atol=1e-2, rtol=0)
+    np.testing.assert_allclose(got[0, 5], P["Vl"][0][far, 1], atol=1e-2)
+    assert not got[2].any() and torch.equal(kc, kc0) and torch.equal(vc, vc0)
+    # slot -1 stores nothing either
+    ops.attention_decode_fused(_t(rows, torch.bfloat16), out, kc, vc, _t(P["tables"], torch.int32), P["max_blocks"],
+                               _t([0, 1, 0], torch.int32), _t(ctx, torch.int32), nh, nkv, hd, 1.0,
+                               slots=_t([-1, -1, -1], torch.int32))
+    assert torch.equal(kc, kc0) and torch.equal(vc, vc0)
+    assert not ops.attention_decode_fused_supported(12, 1, 64, torch.bfloat16) and not ops.attention_decode_fused_supported(4, 2, 48, torch.bfloat16)
+    assert not ops.attention_decode_fused_supported(32, 4, 64, torch.float32)
+
+
 # ------------------------------------------------------------------- tiled prefill attention
 def _run_prefill(ops, P, runs, nh, nkv, hd, scale=None):
     """runs: per sequence (first position, number of rows); rows of P are those positions in order."""
