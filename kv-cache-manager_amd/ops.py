@@ -272,7 +272,7 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
 def gemm_swiglu(x, w_gate_up, out):
     """out[M, I] = swiglu(x[M, K] @ w_gate_up[2 I, K]^T) in one launch, or False when this shape
     has no fused kernel (then the caller runs the product and ``swiglu`` one after the other:
-    the same values)."""
+    the same values up to the order of the sums)."""
     _dev(x, w_gate_up, out)
     for t, n in ((x, "x"), (w_gate_up, "w_gate_up"), (out, "out")):
         _rows2d(t, n)

@@ -577,7 +577,7 @@ def test_partial_sums_feed_the_fused_norm_and_rope(ops):
 
 def test_skinny_gemm_with_swiglu_epilogue_equals_product_then_swiglu(ops):
     rng = np.random.default_rng(77)
-    for M, I, K in ((8, 2560, 256), (1, 5632, 2048), (37, 2568, 192), (64, 2560, 128)):
+    for M, I, K in ((8, 2560, 256), (1, 5632, 2048), (37, 2568, 192), (64, 5120, 128), (20, 5120, 192), (40, 5152, 64), (33, 10240, 64)):
         x = _t(rng.normal(size=(M, K)), torch.bfloat16)
         w = _t(rng.normal(size=(2 * I, K)) * 0.1, torch.bfloat16)
         act = torch.zeros(M, I, dtype=torch.bfloat16, device=DEV)
@@ -586,7 +586,12 @@ def test_skinny_gemm_with_swiglu_epilogue_equals_product_then_swiglu(ops):
         ops.gemm(x, w, gu)                                   # unsplit: no scratch given
         ref = torch.zeros_like(act)
         ops.swiglu(gu, ref)
-        assert torch.equal(act, ref)
+        if M <= 16:
+            assert torch.equal(act, ref)
+        else:   # more than 16 rows: workgroups walk K from different starting points in the two launches
+            a, b = _np(act), _np(ref)
+            assert np.mean(a == b) > 0.98
+            np.testing.assert_allclose(a, b, rtol=2 ** -6, atol=2e-3)
     small = torch.zeros(8, 256, dtype=torch.bfloat16, device=DEV)      # too few columns to fill the chip unsplit
     assert not ops.gemm_swiglu(_t(rng.normal(size=(8, 64)), torch.bfloat16), _t(rng.normal(size=(512, 64)), torch.bfloat16), small)
     big = torch.zeros(65, 2560, dtype=torch.bfloat16, device=DEV)      # too many rows for the streaming kernel
