@@ -20,6 +20,12 @@
 //
 // The only mask is causal: a row at position p sees tokens t <= p.  Rows of different sequences
 // never share a workgroup.  Head sizes 64 and 128; pages of 8, 16, 32, ... tokens (a power of two).
+//
+// Long contexts are cut into segments of 1,024 keys (at absolute multiples of 1,024) that run as
+// workgroups of their own: without that the launch lasts as long as its last rows need to walk
+// all their keys, while the workgroups of early rows have long finished.  A tile whose rows see
+// one segment stores its result; otherwise every segment leaves (o / l, m, l) per row in scratch
+// and a second kernel merges them in segment order.
 #include <cfloat>
 
 #include "common.h"
@@ -43,6 +49,7 @@ constexpr int kPfWaveRows = 16 * kPfRT;
 constexpr int kPfRows = kPfWaveRows * kPfWaves;  // query rows per workgroup
 constexpr int kPfChunk = 64;                     // keys per trip
 constexpr int kPfPad = 8;                        // bfloat16 of padding per LDS row (keeps 16-byte alignment)
+constexpr int kPfSeg = 1024;                     // keys per segment
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   union { bf16x2_t v; uint32_t u; } r;
@@ -64,12 +71,18 @@ __global__ void __launch_bounds__(kPfThreads)
     attention_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                              const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                              const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
-                             const int* __restrict__ seq_start, int nh, int nkv, int B, int b_shift, float scale) {
+                             const int* __restrict__ seq_start, int nh, int nkv, int B, int b_shift, float scale,
+                             int max_segs, float* __restrict__ scratch) {
   constexpr int KSTEPS = HD / 32;                          // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;                              // 16-dim tiles of the output
   constexpr int PIECES = kPfChunk * HD / 8 / kPfThreads;   // 16-byte pieces of a chunk per thread (keys; as many of values)
   constexpr int KPITCH = HD + kPfPad, VPITCH = kPfChunk + kPfPad;
-  const int tile = gridDim.x - 1 - blockIdx.x, seq = blockIdx.y, head = blockIdx.z;   // long rows first
+  // Workgroups are handed out in the order of blockIdx.x, round-robin over the chip's eight parts:
+  // neighbours in that order are the heads of one (tile, segment), so that every part gets the
+  // same mix of long and short walks, and the long ones (late rows) start first.
+  const int head = blockIdx.x % nh, seq = blockIdx.y;
+  const int unit = gridDim.x / nh - 1 - blockIdx.x / nh;
+  const int tile = unit / max_segs, seg = unit % max_segs;
   const int row0 = run_start[seq], n_rows = run_start[seq + 1] - row0;
   const int block_first = tile * kPfRows;
   if (block_first >= n_rows) return;
@@ -81,7 +94,11 @@ __global__ void __launch_bounds__(kPfThreads)
   const size_t head_elems = size_t(B) * HD, page_elems = head_elems * nkv;
   const uint16_t* kbase = kcache + kvh * head_elems;
   const uint16_t* vbase = vcache + kvh * head_elems;
-  const int block_last_pos = pos0 + min(block_first + kPfRows, n_rows) - 1;
+  const int tile_last_pos = pos0 + min(block_first + kPfRows, n_rows) - 1;
+  const int seg_first = seg * kPfSeg;
+  if (seg_first > tile_last_pos) return;
+  const int n_segs = tile_last_pos / kPfSeg + 1;
+  const int block_last_pos = min(tile_last_pos, seg_first + kPfSeg - 1);   // the last key this workgroup reads
   const int first = block_first + wave * kPfWaveRows;   // first row of this wave inside the run
   const bool wave_on = first < n_rows;
   const int wave_last_pos = pos0 + min(first + kPfWaveRows, n_rows) - 1;
@@ -94,7 +111,8 @@ __global__ void __launch_bounds__(kPfThreads)
   // the sequence's page ids up to the workgroup's last position: the address of a piece is one
   // LDS read away instead of one more trip to global memory
   extern __shared__ int page_lds[];
-  for (int i = threadIdx.x; i <= (block_last_pos >> b_shift); i += kPfThreads) page_lds[i] = table[i];
+  const int page_lo = seg_first >> b_shift;
+  for (int i = threadIdx.x; i <= (block_last_pos >> b_shift) - page_lo; i += kPfThreads) page_lds[i] = table[page_lo + i];
 
   // B operand of the scores: lane holds 8 dims of query row n16 of each tile (rows past the run
   // repeat its last row; they are never stored).  That row's position is what the lane may see.
@@ -123,38 +141,30 @@ __global__ void __launch_bounds__(kPfThreads)
   // pieces of keys (8 dims of one token) and as many of values (8 tokens of one dim).  Tokens past
   // the workgroup's last position are read from that position's place instead (always valid
   // memory); the mask keeps them out.
-  uint4 kreg[PIECES], vreg[PIECES];
-  auto request = [&](int c0) {
+  struct Pieces { uint4 k[PIECES], v[PIECES]; };
+  auto request = [&](int c0, Pieces& pc) {
+    c0 = min(c0, block_last_pos & ~(kPfChunk - 1));   // past the last chunk: the last chunk again (no load behind a branch)
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
       const int e = threadIdx.x + i * kPfThreads;
       const int t = min(c0 + e / (HD / 8), block_last_pos);
-      kreg[i] = *reinterpret_cast<const uint4*>(kbase + size_t(page_lds[t >> b_shift]) * page_elems +
+      pc.k[i] = *reinterpret_cast<const uint4*>(kbase + size_t(page_lds[(t >> b_shift) - page_lo]) * page_elems +
                                                 size_t(t & b_mask) * HD + (e % (HD / 8)) * 8);
       const int tv = min(c0 + (e % 8) * 8, block_last_pos & ~7);
-      vreg[i] = *reinterpret_cast<const uint4*>(vbase + size_t(page_lds[tv >> b_shift]) * page_elems +
+      pc.v[i] = *reinterpret_cast<const uint4*>(vbase + size_t(page_lds[(tv >> b_shift) - page_lo]) * page_elems +
                                                 size_t(e / 8) * B + (tv & b_mask));
     }
   };
-  auto stage = [&](int buf) {
+  auto stage = [&](int buf, const Pieces& pc) {
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
       const int e = threadIdx.x + i * kPfThreads;
-      *reinterpret_cast<uint4*>(&k_lds[buf][e / (HD / 8)][(e % (HD / 8)) * 8]) = kreg[i];
-      *reinterpret_cast<uint4*>(&v_lds[buf][e / 8][(e % 8) * 8]) = vreg[i];
+      *reinterpret_cast<uint4*>(&k_lds[buf][e / (HD / 8)][(e % (HD / 8)) * 8]) = pc.k[i];
+      *reinterpret_cast<uint4*>(&v_lds[buf][e / 8][(e % 8) * 8]) = pc.v[i];
     }
   };
 
-  request(0);
-  stage(0);
-  __syncthreads();
-  int buf = 0;
-  for (int c0 = 0; c0 <= block_last_pos; c0 += kPfChunk, buf ^= 1) {
-    // The next chunk's loads are in flight while this one is multiplied.  After the last chunk
-    // the same chunk is asked for again: no branch around the loads (the compiler would wait for
-    // them at once), and nobody reads what is staged then.
-    request(c0 + kPfChunk <= block_last_pos ? c0 + kPfChunk : c0);
-
+  auto compute = [&](int c0, int buf) {
     if (wave_on && c0 <= wave_last_pos) {
       // ---- S^T: s[rt][j][i] = k[token c0 + 16 j + 4 kq + i] . q[row n16 of tile rt]
       f32x4 s[kPfRT][4];
@@ -171,37 +181,54 @@ __global__ void __launch_bounds__(kPfThreads)
             s[rt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c].v, qf[rt][c].v, s[rt][j], 0, 0, 0);
         }
       }
-      // ---- running maximum and sum of the lane's query row; probabilities stay in registers
-      const bool diagonal = c0 + kPfChunk - 1 > wave_first_pos;   // some row of the wave cannot see the whole chunk
+      // ---- running maximum and sum of the lane's query row; probabilities stay in registers.
+      // Scores stay raw: the scale (in units of log2) goes into the exponent's multiply-add, the
+      // maximum is taken of raw scores (the scale is positive).  Only a chunk that some row of the
+      // wave cannot see completely is masked.
+      const bool diagonal = c0 + kPfChunk - 1 > wave_first_pos;
       PFrag pf[kPfRT][2];   // B operands of the two 32-token steps
 #pragma unroll
       for (int rt = 0; rt < kPfRT; ++rt) {
         float mx = -FLT_MAX;
+        if (diagonal) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+          for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int t = c0 + j * 16 + 4 * kq + i;
-            s[rt][j][i] = (!diagonal || t <= pos[rt]) ? s[rt][j][i] * scale_log2 : -FLT_MAX;
-            mx = fmaxf(mx, s[rt][j][i]);
-          }
+            for (int i = 0; i < 4; ++i) {
+              const int t = c0 + j * 16 + 4 * kq + i;
+              s[rt][j][i] = t <= pos[rt] ? s[rt][j][i] : -FLT_MAX;
+              mx = fmaxf(mx, s[rt][j][i]);
+            }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[rt][j][i]);
+        }
         mx = quad_rows_max(mx);
-        const float m_new = fmaxf(m[rt], mx);   // finite from the first trip on: token 0 is visible to every row
-        const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_new);
+        // m is finite once the row has seen a key; a row that starts before this segment's first
+        // key has seen none of it yet (m_new = -FLT_MAX): its probabilities are zero
+        const float m_new = fmaxf(m[rt], mx);
+        const bool seen = m_new > -0.5f * FLT_MAX;
+        const float shift = seen ? -m_new * scale_log2 : -FLT_MAX;       // exp2(s * scale + shift)
+        const float alpha = seen ? __builtin_amdgcn_exp2f((m[rt] - m_new) * scale_log2) : 1.0f;
         m[rt] = m_new;
         float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            s[rt][j][i] = __builtin_amdgcn_exp2f(s[rt][j][i] - m_new);   // masked: exp2(-huge) = 0
+            // masked scores are -FLT_MAX: the product overflows to -inf, exp2 gives 0
+            s[rt][j][i] = __builtin_amdgcn_exp2f(fmaf(s[rt][j][i], scale_log2, shift));
             sum += s[rt][j][i];
           }
         l[rt] = l[rt] * alpha + quad_rows_sum(sum);
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // the maximum moves in few chunks
 #pragma unroll
-        for (int d = 0; d < DT; ++d)
+          for (int d = 0; d < DT; ++d)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o[rt][d][i] *= alpha;
+            for (int i = 0; i < 4; ++i) o[rt][d][i] *= alpha;
+        }
         // step c covers tiles 2c and 2c+1: reduction index e < 4 -> token 16(2c) + 4kq + e, e >= 4 -> 16(2c+1) + 4kq + e-4
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
@@ -223,8 +250,28 @@ __global__ void __launch_bounds__(kPfThreads)
           for (int rt = 0; rt < kPfRT; ++rt) o[rt][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][c].v, o[rt][d], 0, 0, 0);
         }
     }
-    stage(buf ^ 1);
+  };
+
+  // Two chunks are on their way from the cache while one is multiplied: chunk i+1 sits in
+  // registers (asked for one trip earlier) and goes to the other LDS buffer after the products,
+  // chunk i+2 is asked for before them.
+  {
+    Pieces pa, pb;
+    request(seg_first, pa);
+    request(seg_first + kPfChunk, pb);
+    stage(0, pa);
     __syncthreads();
+    for (int c0 = seg_first; c0 <= block_last_pos; c0 += 2 * kPfChunk) {
+      request(c0 + 2 * kPfChunk, pa);
+      compute(c0, 0);
+      stage(1, pb);
+      __syncthreads();
+      if (c0 + kPfChunk > block_last_pos) break;
+      request(c0 + 3 * kPfChunk, pb);
+      compute(c0 + kPfChunk, 1);
+      stage(0, pa);
+      __syncthreads();
+    }
   }
 
   if (!wave_on) return;
@@ -232,16 +279,61 @@ __global__ void __launch_bounds__(kPfThreads)
   for (int rt = 0; rt < kPfRT; ++rt) {
     const int r = first + rt * 16 + n16;
     if (r >= n_rows) continue;
-    uint16_t* orow = out + size_t(row0 + r) * out_stride + size_t(head) * HD + 4 * kq;
-    const float inv = 1.0f / l[rt];
+    const float inv = l[rt] > 0.f ? 1.0f / l[rt] : 0.f;
+    if (n_segs == 1) {
+      uint16_t* orow = out + size_t(row0 + r) * out_stride + size_t(head) * HD + 4 * kq;
 #pragma unroll
-    for (int d = 0; d < DT; ++d) {
-      uint2 v;
-      v.x = pack_bf16(o[rt][d][0] * inv, o[rt][d][1] * inv);
-      v.y = pack_bf16(o[rt][d][2] * inv, o[rt][d][3] * inv);
-      *reinterpret_cast<uint2*>(orow + d * 16) = v;
+      for (int d = 0; d < DT; ++d) {
+        uint2 v;
+        v.x = pack_bf16(o[rt][d][0] * inv, o[rt][d][1] * inv);
+        v.y = pack_bf16(o[rt][d][2] * inv, o[rt][d][3] * inv);
+        *reinterpret_cast<uint2*>(orow + d * 16) = v;
+      }
+    } else {   // this segment's share of the row: o / l, then m (in units of log2) and l
+      float* dst = scratch + ((size_t(row0 + r) * nh + head) * max_segs + seg) * (HD + 4);
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+        *reinterpret_cast<float4*>(dst + d * 16 + 4 * kq) =
+            float4{o[rt][d][0] * inv, o[rt][d][1] * inv, o[rt][d][2] * inv, o[rt][d][3] * inv};
+      if (kq == 0) { dst[HD] = m[rt] > -0.5f * FLT_MAX ? m[rt] * scale_log2 : -FLT_MAX; dst[HD + 1] = l[rt]; }
     }
   }
+}
+
+// Rows whose tile was cut into several segments: out = sum_s w_s o_s / sum_s w_s with
+// w_s = l_s 2^(m_s - m), segments in order.  HD / 4 threads per row, four dims each.
+template <int HD>
+__global__ void __launch_bounds__(256)
+    attention_prefill_merge_kernel(const float* __restrict__ scratch, uint16_t* __restrict__ out, int out_stride,
+                                   const int* __restrict__ run_start, const int* __restrict__ seq_start, int nh,
+                                   int max_segs) {
+  const int seq = blockIdx.y, head = blockIdx.z;
+  const int row0 = run_start[seq], n_rows = run_start[seq + 1] - row0;
+  constexpr int PER_ROW = HD / 4;
+  const int r = blockIdx.x * (256 / PER_ROW) + threadIdx.x / PER_ROW, piece = threadIdx.x % PER_ROW;
+  if (r >= n_rows) return;
+  const int tile = r / kPfRows;
+  const int tile_last_pos = seq_start[seq] + min((tile + 1) * kPfRows, n_rows) - 1;
+  const int n_segs = tile_last_pos / kPfSeg + 1;
+  if (n_segs == 1) return;   // stored directly
+  const float* base = scratch + (size_t(row0 + r) * nh + head) * max_segs * (HD + 4);
+  float m = -FLT_MAX;
+  for (int s = 0; s < n_segs; ++s) m = fmaxf(m, base[s * (HD + 4) + HD]);
+  float4 num = {0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+  for (int s = 0; s < n_segs; ++s) {
+    const float* p = base + s * (HD + 4);
+    const float l = p[HD + 1];
+    const float w = l > 0.f ? l * __builtin_amdgcn_exp2f(p[HD] - m) : 0.f;
+    const float4 o = *reinterpret_cast<const float4*>(p + piece * 4);
+    num.x = fmaf(w, o.x, num.x); num.y = fmaf(w, o.y, num.y); num.z = fmaf(w, o.z, num.z); num.w = fmaf(w, o.w, num.w);
+    den += w;
+  }
+  const float inv = 1.0f / den;
+  uint2 v;
+  v.x = pack_bf16(num.x * inv, num.y * inv);
+  v.y = pack_bf16(num.z * inv, num.w * inv);
+  *reinterpret_cast<uint2*>(out + size_t(row0 + r) * out_stride + size_t(head) * HD + piece * 4) = v;
 }
 
 }  // namespace kvcm
@@ -254,34 +346,59 @@ int kvcm_attention_prefill_supported(int nh, int nkv, int hd, int B) {
   return nkv > 0 && nh % nkv == 0 && (hd == 64 || hd == 128) && B >= 8 && (B & (B - 1)) == 0;
 }
 
+// Floats of scratch a launch needs: none while no row's context exceeds one segment of 1,024 keys.
+long long kvcm_attention_prefill_scratch(int T, int nh, int hd, int max_context) {
+  const long long segs = (max_context + kPfSeg - 1) / kPfSeg;
+  return segs <= 1 ? 0 : static_cast<long long>(T) * nh * segs * (hd + 4);
+}
+
 // run_start [S+1]: first row of each sequence's run of consecutive positions (rows of a run are
 // consecutive); seq_start [S]: position of a run's first row; tables [S][table_stride];
-// max_run: the longest run (it sizes the launch).
+// max_run: the longest run (it sizes the launch); T: rows in all (run_start[S]); max_context: an
+// upper bound of every row's context length (position + 1); scratch: see above.
 int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                            const void* vcache, const int* tables, int table_stride, const int* run_start,
-                           const int* seq_start, int S, int max_run, int nh, int nkv, int hd, int B, float scale,
-                           hipStream_t s) {
+                           const int* seq_start, int S, int max_run, int T, int max_context, int nh, int nkv, int hd,
+                           int B, float scale, float* scratch, long long scratch_floats, hipStream_t s) {
   if (S == 0 || max_run == 0) return 0;
   KVCM_REQUIRE(kvcm_attention_prefill_supported(nh, nkv, hd, B),
                "attention_prefill: unsupported shape heads=%d kv_heads=%d head_dim=%d page=%d", nh, nkv, hd, B);
-  KVCM_REQUIRE(S > 0 && max_run > 0 && S <= 65535 && nh <= 65535, "attention_prefill: bad sizes S=%d max_run=%d", S, max_run);
+  KVCM_REQUIRE(S > 0 && max_run > 0 && S <= 65535 && nh <= 65535 && T >= max_run && max_context >= 1,
+               "attention_prefill: bad sizes S=%d max_run=%d T=%d max_context=%d", S, max_run, T, max_context);
+  KVCM_REQUIRE(scale > 0.f, "attention_prefill: the scale must be positive");
   KVCM_REQUIRE(q_stride >= nh * hd && out_stride >= nh * hd && q_stride % 8 == 0, "attention_prefill: bad row strides");
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(vcache) % 16 == 0, "attention_prefill: operands must be 16-byte aligned");
   KVCM_REQUIRE(out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0, "attention_prefill: output must be 8-byte aligned");
+  const int max_segs = (max_context + kPfSeg - 1) / kPfSeg;
+  const long long need = kvcm_attention_prefill_scratch(T, nh, hd, max_context);
+  KVCM_REQUIRE(need == 0 || (scratch && scratch_floats >= need && reinterpret_cast<uintptr_t>(scratch) % 16 == 0),
+               "attention_prefill: scratch too small (%lld floats needed)", need);
   int b_shift = 0;
   while ((1 << b_shift) < B) ++b_shift;
-  const dim3 grid((max_run + kPfRows - 1) / kPfRows, S, nh);
-  const size_t page_bytes = sizeof(int) * size_t(table_stride);
-  KVCM_REQUIRE(page_bytes <= 48 * 1024, "attention_prefill: page tables of %d entries do not fit LDS", table_stride);
+  const long long units = static_cast<long long>((max_run + kPfRows - 1) / kPfRows) * max_segs * nh;
+  KVCM_REQUIRE(units < (1ll << 31), "attention_prefill: too many workgroups");
+  const dim3 grid(static_cast<unsigned>(units), S, 1);
+  const size_t page_bytes = sizeof(int) * size_t(kPfSeg / B + 2);   // the pages of one segment
   const uint16_t *qq = static_cast<const uint16_t*>(q), *kc = static_cast<const uint16_t*>(kcache),
                  *vc = static_cast<const uint16_t*>(vcache);
-  if (hd == 64)
+  const int merge_rows = 256 / (hd / 4);   // rows per workgroup of the merge
+  const dim3 mgrid((max_run + merge_rows - 1) / merge_rows, S, nh);
+  if (hd == 64) {
     attention_prefill_kernel<64><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
-                                                             tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale);
-  else
+                                                             tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale,
+                                                             max_segs, scratch);
+    if (max_segs > 1)
+      attention_prefill_merge_kernel<64><<<mgrid, 256, 0, s>>>(scratch, static_cast<uint16_t*>(out), out_stride, run_start,
+                                                              seq_start, nh, max_segs);
+  } else {
     attention_prefill_kernel<128><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
-                                                              tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale);
+                                                              tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale,
+                                                              max_segs, scratch);
+    if (max_segs > 1)
+      attention_prefill_merge_kernel<128><<<mgrid, 256, 0, s>>>(scratch, static_cast<uint16_t*>(out), out_stride, run_start,
+                                                               seq_start, nh, max_segs);
+  }
   return launch_status("attention_prefill");
 }
 

@@ -212,8 +212,11 @@ class ModelRunner:
         if (self.attn != "v1" and window == 0 and step.max_run > 1
                 and ops.attention_prefill_supported(nh, nkv, hd, q.dtype, kcache.shape[2])):
             # runs of consecutive positions: keys are read once per 64 query rows, on the matrix cores
+            need = ops.attention_prefill_scratch(step.real_rows, nh, hd, step.max_context)
+            scratch = self.workspace.flat("prefill_partials", need) if need else None
             ops.attention_prefill(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.run_start,
-                                  step.seq_start, step.real_seqs, step.max_run, nh, nkv, hd, scale)
+                                  step.seq_start, step.real_seqs, step.max_run, nh, nkv, hd, scale,
+                                  rows=step.real_rows, max_context=step.max_context, scratch=scratch)
             return
         ops.attention(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
                       step.ctx_lens, nh, nkv, hd, scale, window, rows=step.rows)

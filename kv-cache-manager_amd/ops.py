@@ -50,7 +50,9 @@ def _declare(lib):
     fn("kvcm_sample", vp, i, vp, vp, vp, vp, vp, i, i, vp)
     fn("kvcm_attention_decode_supported", i, i, i, i)
     fn("kvcm_attention_prefill_supported", i, i, i, i)
-    fn("kvcm_attention_prefill", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, i, f, vp)
+    fn("kvcm_attention_prefill", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, i, i, i, f, vp, C.c_longlong, vp)
+    lib.kvcm_attention_prefill_scratch.restype = C.c_longlong
+    lib.kvcm_attention_prefill_scratch.argtypes = [i, i, i, i]
     lib.kvcm_attention_decode_scratch.restype = C.c_longlong
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
@@ -393,12 +395,28 @@ def attention_prefill_supported(nh, nkv, hd, dtype, block_size=16):
     return dtype == torch.bfloat16 and bool(lib().kvcm_attention_prefill_supported(nh, nkv, hd, block_size))
 
 
+def attention_prefill_scratch(rows, nh, hd, max_context):
+    """Floats of scratch ``attention_prefill`` needs (0 while contexts fit one segment of keys)."""
+    return int(lib().kvcm_attention_prefill_scratch(rows, nh, hd, max_context))
+
+
 def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, seq_start, num_seqs, max_run, nh, nkv, hd,
-                      scale):
+                      scale, rows=None, max_context=None, scratch=None):
     """Causal attention for runs of consecutive positions (bfloat16): sequence s owns rows
     run_start[s] .. run_start[s+1]-1, the first of them at position seq_start[s]; every row sees the
-    sequence's cached tokens up to its own position.  The same result as ``attention``."""
-    _dev(q, out, kcache, vcache, tables, run_start, seq_start)
+    sequence's cached tokens up to its own position.  The same result as ``attention``.
+    ``rows``: rows in all; ``max_context``: a bound of every row's context length (default: what the
+    block tables can hold); contexts beyond 1,024 keys need ``scratch`` (float32,
+    attention_prefill_scratch elements; allocated here when not given)."""
+    _dev(q, out, kcache, vcache, tables, run_start, seq_start, scratch)
+    T = q.shape[0] if rows is None else rows
+    if max_context is None:
+        max_context = table_stride * kcache.shape[2]
+    need = attention_prefill_scratch(T, nh, hd, max_context)
+    if need and scratch is None:
+        scratch = torch.empty(need, dtype=torch.float32, device=q.device)
+    if scratch is not None:
+        _need(scratch.dtype == torch.float32 and scratch.is_contiguous(), "scratch must be contiguous float32")
     _rows2d(q, "q")
     _rows2d(out, "out")
     _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "attention_prefill is bfloat16 only")
@@ -408,7 +426,8 @@ def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, s
     _i32(tables, "tables", num_seqs * table_stride)
     _check(lib().kvcm_attention_prefill(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
                                         _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), num_seqs, max_run,
-                                        nh, nkv, hd, kcache.shape[2], float(scale), _stream()))
+                                        T, int(max_context), nh, nkv, hd, kcache.shape[2], float(scale), _ptr(scratch),
+                                        scratch.numel() if scratch is not None else 0, _stream()))
 
 
 def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_index=None):

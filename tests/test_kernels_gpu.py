@@ -801,9 +801,34 @@ def test_prefill_attention_long_prompt(ops):
     runs = [(0, 1500), (1000, 300)]
     P = _runs_problem(rng, runs, nh, nkv, hd, B)
     got = _run_prefill(ops, P, runs, nh, nkv, hd)
-    rows = [0, 1, 63, 64, 700, 1499, 1500, 1799]
+    # contexts beyond 1,024 keys are cut into segments that are merged afterwards: rows around the
+    # cut, a tile that the cut goes through (the second run starts at 1000), tile edges
+    rows = [0, 1, 63, 64, 700, 1023, 1024, 1025, 1151, 1152, 1499, 1500, 1523, 1524, 1627, 1628, 1799]
     ref = np.zeros((len(rows), nh, hd))
     for k, r in enumerate(rows):
         s, c = P["row_seq"][r], P["ctx"][r]
         ref[k] = plain.attention(P["Q"][r:r + 1], P["Kl"][s][:c], P["Vl"][s][:c], [c - 1], np.arange(c), 1.0 / math.sqrt(hd))[0]
+    np.testing.assert_allclose(got[rows], ref, atol=1e-2, rtol=0)
+
+
+def test_prefill_attention_three_segments_far_key(ops):
+    """A row deep in the third segment of keys must still find one outstanding key of the first."""
+    rng = np.random.default_rng(52)
+    nh, nkv, hd, B = 4, 1, 128, 16
+    runs = [(0, 2300)]
+    P = _runs_problem(rng, runs, nh, nkv, hd, B)
+    far = 5
+    P["Q"][2200:, 2] = 0.0
+    P["Q"][2200:, 2, 11] = 30.0
+    kvec = np.zeros(hd)
+    kvec[11] = 30.0
+    P["Kl"][0][far, 0] = kvec
+    P["Kc"][P["tables"][0, far // B], 0, far % B] = kvec
+    got = _run_prefill(ops, P, runs, nh, nkv, hd, scale=1.0)
+    np.testing.assert_allclose(got[2200:, 2], np.broadcast_to(P["Vl"][0][far, 0], got[2200:, 2].shape), atol=2e-2)
+    rows = [2047, 2048, 2175, 2176, 2299]
+    ref = np.zeros((len(rows), nh, hd))
+    for k, r in enumerate(rows):
+        c = P["ctx"][r]
+        ref[k] = plain.attention(P["Q"][r:r + 1], P["Kl"][0][:c], P["Vl"][0][:c], [c - 1], np.arange(c), 1.0)[0]
     np.testing.assert_allclose(got[rows], ref, atol=1e-2, rtol=0)
