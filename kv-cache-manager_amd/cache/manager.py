@@ -161,6 +161,7 @@ class HostCore:
         self.prefill_chunk = prefill_chunk
         self.prefix_caching = bool(prefix_caching) and policy == "paged"
         self._desc = np.zeros(self._lib.kvcm_batch_desc_len(self._h), dtype=np.int32)
+        self._summary = np.zeros(5, dtype=np.int64)
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -274,6 +275,18 @@ class HostCore:
             seed.ctypes.data_as(u64p), cap))
         return [PlanEntry(int(ids[k]), int(start[k]), int(count[k]), bool(flags[k] & 1), bool(flags[k] & 2),
                           int(gen[k]), float(temp[k]), int(seed[k])) for k in range(n)]
+
+    def schedule_summary(self, now=0.0):
+        """Runs the scheduler; -> (entries, prompt tokens, decoding sequences, entries that sample,
+        decode_shaped) without building the plan's entries in Python (``plan()`` still gives them)."""
+        check(self._lib.kvcm_sched_schedule_summary(self._h, float(now), self._summary.ctypes.data_as(i64p)))
+        s = self._summary
+        return int(s[0]), int(s[1]), int(s[2]), int(s[3]), bool(s[4])
+
+    def update_sampled(self, ids, now=0.0):
+        """The ids sampled this step, in the order of the plan's sampling entries."""
+        t = np.ascontiguousarray(ids, dtype=np.int32)
+        check(self._lib.kvcm_sched_update_sampled(self._h, t.ctypes.data_as(i32p), len(t), float(now)))
 
     def update(self, next_tokens, now=0.0):
         t = _i32(next_tokens)

@@ -61,6 +61,8 @@ def _declare(lib):
     fn("kvcm_sched_schedule", i, vp, dbl)
     fn("kvcm_sched_plan", i, vp, i64p, i32p, i32p, i32p, i32p, f32p, u64p, i)
     fn("kvcm_sched_update", i, vp, i32p, i, dbl)
+    fn("kvcm_sched_schedule_summary", i, vp, dbl, i64p)
+    fn("kvcm_sched_update_sampled", i, vp, i32p, i, dbl)
     fn("kvcm_sched_collect_finished", i, vp)
     fn("kvcm_finished_get", i, vp, i, i64p, f64p, i32p, i)
     fn("kvcm_finished_clear", None, vp)

@@ -340,6 +340,41 @@ int kvcm_sched_plan(void* c, int64_t* ids, int32_t* start, int32_t* count, int32
     return static_cast<int64_t>(plan.size());
   }));
 }
+// Runs the scheduler and says what it planned without handing the entries over:
+// out = {entries, prompt tokens, decoding sequences, entries that sample, 1 if every entry is a
+// single token that samples (a decode-shaped step)}.
+int kvcm_sched_schedule_summary(void* c, double now, int64_t* out) {
+  return static_cast<int>(guarded([&]() -> int64_t {
+    const auto& plan = static_cast<Core*>(c)->sched->schedule(now);
+    int64_t prefill = 0, decode = 0, sampling = 0, single = 1;
+    for (const auto& p : plan) {
+      if (p.is_prefill) prefill += p.num_tokens; else ++decode;
+      if (p.samples) ++sampling;
+      if (p.num_tokens != 1 || !p.samples) single = 0;
+    }
+    out[0] = static_cast<int64_t>(plan.size()); out[1] = prefill; out[2] = decode; out[3] = sampling;
+    out[4] = plan.empty() ? 0 : single;
+    return static_cast<int64_t>(plan.size());
+  }));
+}
+// The step's sampled ids, in the order of the plan's sampling entries; entries that did not
+// sample get none.
+int kvcm_sched_update_sampled(void* c, const int32_t* ids, int n, double now) {
+  return static_cast<int>(guarded([&]() -> int64_t {
+    auto* core = static_cast<Core*>(c);
+    const auto& plan = core->sched->plan();
+    std::vector<int32_t> next(plan.size(), -1);
+    int k = 0;
+    for (size_t i = 0; i < plan.size(); ++i)
+      if (plan[i].samples) {
+        if (k >= n) throw std::invalid_argument("update_sampled: fewer ids than sampling entries");
+        next[i] = ids[k++];
+      }
+    if (k != n) throw std::invalid_argument("update_sampled: more ids than sampling entries");
+    core->sched->update(next, now);
+    return 0;
+  }));
+}
 int kvcm_sched_update(void* c, const int32_t* next, int n, double now) {
   return static_cast<int>(guarded([&]() -> int64_t {
     auto* core = static_cast<Core*>(c);

@@ -76,18 +76,12 @@ class Engine:
     def step(self) -> StepInfo:
         info = StepInfo()
         t_start = self.now()
-        plan = self.core.schedule(t_start)
-        if not plan:
+        n, info.prefill_tokens, info.decode_seqs, sampling, decode_shaped = self.core.schedule_summary(t_start)
+        if n == 0:
             return info
-        for p in plan:
-            if p.is_prefill:
-                info.prefill_tokens += p.count
-            else:
-                info.decode_seqs += 1
-        sampling = [p for p in plan if p.samples]
-        if self.decode_graphs is not None and self.decode_graphs.usable(plan):
-            ids = self.decode_graphs.run(plan)
-            info.rows = info.seqs = len(plan)
+        if self.decode_graphs is not None and decode_shaped and self.decode_graphs.fits(n):
+            ids = self.decode_graphs.run(n)
+            info.rows = info.seqs = n
         else:
             layout = self.core.build_batch_from_plan(self.runner.host_buffer())
             logits = self.runner.execute(layout)
@@ -97,15 +91,8 @@ class Engine:
                 ids = self.sampler.sample_on_device(logits, self.runner.last_step.sampling_params())
             else:
                 torch.cuda.current_stream().synchronize()
-        nxt, k = [], 0
-        for p in plan:
-            if p.samples:
-                nxt.append(int(ids[k]))
-                k += 1
-            else:
-                nxt.append(-1)
         t_end = self.now()
-        self.core.update(nxt, t_end)
+        self.core.update_sampled(ids, t_end)
         info.ms = (t_end - t_start) * 1e3
         return info
 

@@ -29,12 +29,15 @@ class DecodeGraphs:
         self.buckets = [b for b in _BUCKETS if b <= min(lim.max_seqs, lim.max_logit_rows, lim.max_tokens)]
         self.table_stride = lim.max_blocks_per_seq
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
+        self._views = {}      # bucket -> (device view, pinned view, ints) of the metadata a replay uploads
         self.enabled = bool(self.buckets)
 
+    def fits(self, n: int) -> bool:
+        """May a decode-shaped step of n sequences be replayed from a graph?"""
+        return self.enabled and 0 < n <= self.buckets[-1]
+
     def usable(self, plan) -> bool:
-        if not self.enabled or not plan or len(plan) > self.buckets[-1]:
-            return False
-        return all(p.count == 1 and p.samples for p in plan)
+        return self.fits(len(plan)) and all(p.count == 1 and p.samples for p in plan)
 
     def _bucket(self, n: int) -> int:
         for b in self.buckets:
@@ -60,17 +63,20 @@ class DecodeGraphs:
         t, seeds, ids, idx = step.sampling_params()
         self.runner.ops.sample(logits, self.sampler.out[:bucket], t, seeds, ids, idx)
 
-    def run(self, plan) -> np.ndarray:
-        n = len(plan)
+    def run(self, n: int) -> np.ndarray:
+        """Runs the scheduler's current plan (n decode-shaped entries); returns the n sampled ids."""
         bucket = self._bucket(n)
         runner, s = self.runner, self.sampler
         layout = self.core.build_batch_from_plan(runner.host_buffer(), pad_rows=bucket, pad_seqs=bucket,
                                                  pad_logit_rows=bucket, table_stride=self.table_stride)
         runner._check(layout)
-        total = layout.total
-        runner.meta_dev[:total].copy_(runner._pinned[:total], non_blocking=True)
-        runner._upload_done.record()
-        runner._upload_pending = True
+        views = self._views.get(bucket)
+        if views is None or views[2] != layout.total:
+            views = self._views[bucket] = (runner.meta_dev[:layout.total], runner._pinned[:layout.total], layout.total)
+        views[0].copy_(views[1], non_blocking=True)
+        # no event: the synchronous download below ends after this upload, so the pinned buffer
+        # is free again when the next step fills it
+        runner._upload_pending = False
         graph = self.graphs.get(bucket)
         if graph is None:
             self._forward(layout, bucket)                 # eager once: creates every work buffer

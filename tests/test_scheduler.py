@@ -1,6 +1,7 @@
 """The scheduler's decisions with a fake model (every sampled token is 42), as the reference
 tests them (tests/test_scheduler.cpp), plus portions of prompts under a token budget."""
 import numpy as np
+import pytest
 from kvcm_amd.cache.manager import HostCore
 
 
@@ -215,3 +216,26 @@ def test_plan_batch_carries_sampling_parameters_for_every_logit_row():
     L = core.build_batch_from_plan(out)
     o, R = L.sampling, L.logit_rows_padded
     np.testing.assert_array_equal(out[o + R:o + 2 * R], [1, 1])                          # second generated token
+
+
+def test_schedule_summary_and_update_by_sampled_ids():
+    core = HostCore(num_blocks=64, block_size=4, max_seq_len=64, max_num_seqs=8, max_batched_tokens=64, prefill_chunk=4)
+    core.sched_add(1, [5, 6, 7], 3)              # fits one portion: samples in the first step
+    core.sched_add(2, list(range(10, 19)), 3)    # 9 tokens: three portions, samples in the third
+    n, prefill, decode, sampling, shaped = core.schedule_summary()
+    assert (n, prefill, decode, sampling, shaped) == (2, 7, 0, 1, False)
+    assert [(p.id, p.count, p.samples) for p in core.plan()] == [(1, 3, True), (2, 4, False)]
+    with pytest.raises(Exception):
+        core.update_sampled([42, 43])            # one sampling entry, two ids
+    core.update_sampled([42])
+    n, prefill, decode, sampling, shaped = core.schedule_summary()
+    assert (n, prefill, decode, sampling, shaped) == (2, 4, 1, 1, False)       # request 1 decodes beside a portion of 2
+    core.update_sampled([43])
+    n, prefill, decode, sampling, shaped = core.schedule_summary()
+    assert (n, prefill, decode, sampling, shaped) == (2, 0, 2, 2, True)        # a prompt's last single token runs like a decode
+    core.update_sampled([44, 50])
+    n, prefill, decode, sampling, shaped = core.schedule_summary()
+    assert (n, prefill, decode, sampling, shaped) == (1, 0, 1, 1, True)        # request 1 is done, request 2 decodes
+    core.update_sampled([51])
+    done = {f.id: f.generated for f in core.take_finished()}
+    assert done[1] == [42, 43, 44]
