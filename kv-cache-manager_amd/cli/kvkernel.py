@@ -4,9 +4,11 @@ page sizes, with the reference tool's flags and columns (src/main_kernel_bench.c
   --ctx 128,256,512,1024,2048  --batch 1,8,32,128  --block-size 16  --heads 32  --kv-heads 4
   --head-dim 64  --iters 100  --out FILE.csv  [--graph]
 
-Four variants per point: v1 (one pass over the context per row and head) and v2 (contexts cut
-into partitions that run in parallel and are merged), each through a shuffled block table
-("paged") and through a table of consecutive pages ("contiguous").  5 warm-up calls, then
+Six variants per point: v1 (one pass over the context per row and head), v2 (contexts cut into
+partitions that run in parallel and are merged) and, not in the reference, "fused" (the kernel
+decode steps run: one launch that also takes q, k, v from the projection and writes the new key
+and value to their page), each through a shuffled block table ("paged") and through a table of
+consecutive pages ("contiguous").  5 warm-up calls, then
 ``--iters`` timed calls between two events; GB/s = 2 * batch * ctx * kv_heads * head_dim * 2 bytes
 / time, the keys and values a call has to read once.  Zero-filled bfloat16 cache, scale 0.125.
 With --graph (not in the reference) the timed calls are replays of one captured HIP graph that
@@ -75,10 +77,19 @@ def main(argv=None):
                 def v2(tab):
                     ops.attention_decode(Q, O, K, V, tab, mb, rows, lens, heads, kvh, hd, 0.125, ctx, scratch)
 
-                for version, call in (("v1", v1), ("v2", v2)):
+                fused_ok = ops.attention_decode_fused_supported(heads, kvh, hd, bf16, B)
+                QKV = torch.zeros(batch, (heads + 2 * kvh) * hd, dtype=bf16, device=dev)
+                slots = {k: (t.view(batch, mb)[:, (ctx - 1) // B] * B + (ctx - 1) % B).to(torch.int32).contiguous()
+                         for k, t in tables.items()}
+
+                def fused(tab):
+                    ops.attention_decode_fused(QKV, O, K, V, tab, mb, rows, lens, heads, kvh, hd, 0.125,
+                                               slots=slots["paged" if tab is tables["paged"] else "contiguous"])
+
+                for version, call in (("v1", v1), ("v2", v2), ("fused", fused)):
                     for layout in ("paged", "contiguous"):
                         name = f"{layout}-{version}"
-                        if version == "v2" and not v2_ok:
+                        if (version == "v2" and not v2_ok) or (version == "fused" and not fused_ok):
                             print("%5d %6d %6d %-16s %10s" % (B, batch, ctx, name, "unsupported"))
                             continue
                         tab = tables[layout]
@@ -108,7 +119,7 @@ def main(argv=None):
                         waves = info["threads"] // 64
                         occ = 100.0 * info["workgroups_per_cu"] * waves / WAVE_SLOTS_PER_CU
                         wgs = ((batch * heads + 3) // 4 if version == "v1"
-                               else kvh * batch * ((ctx + 255) // 256))
+                               else kvh * batch * ((ctx + 255) // 256) if version == "v2" else kvh * batch)
                         rounds = wgs / float(max(info["workgroups_per_cu"], 1) * cus)
                         print("%5d %6d %6d %-16s %10.2f %9.1f %6.1f%% %5d %6dB %6d %5.0f%% %7.2f" % (
                             B, batch, ctx, name, us, gbs, 100 * gbs / PEAK_GBS, info["regs"], info["lds_bytes"],

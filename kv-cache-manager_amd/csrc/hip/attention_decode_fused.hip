@@ -262,6 +262,28 @@ __global__ void __launch_bounds__(kFusWaves* kWave)
   }
 }
 
+template <int HD, int GROUP>
+int fused_kernel_info(int* out) {
+  hipFuncAttributes a;
+  int per_cu = 0;
+  if (hipFuncGetAttributes(&a, reinterpret_cast<const void*>(&attention_decode_fused_kernel<HD, GROUP>)) != hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attention_decode_fused_kernel<HD, GROUP>, kFusWaves * kWave, 0) != hipSuccess)
+    return -1;
+  out[0] = a.numRegs; out[1] = static_cast<int>(a.sharedSizeBytes); out[2] = per_cu; out[3] = kFusWaves * kWave;
+  return 0;
+}
+
+template <int HD>
+int dispatch_fused_info(int group, int* out) {
+  switch (group) {
+    case 1: return fused_kernel_info<HD, 1>(out); case 2: return fused_kernel_info<HD, 2>(out);
+    case 3: return fused_kernel_info<HD, 3>(out); case 4: return fused_kernel_info<HD, 4>(out);
+    case 5: return fused_kernel_info<HD, 5>(out); case 6: return fused_kernel_info<HD, 6>(out);
+    case 7: return fused_kernel_info<HD, 7>(out); case 8: return fused_kernel_info<HD, 8>(out);
+    default: return -1;
+  }
+}
+
 template <int HD>
 int dispatch_fused(int group, dim3 grid, hipStream_t s, const float* partials, int S, size_t pstride, const uint16_t* qkv,
                    int qkv_stride, const float2* cos_sin, const int* slots, uint16_t* kc, uint16_t* vc,
@@ -292,6 +314,15 @@ int kvcm_attention_decode_fused_supported(int nh, int nkv, int hd, int B) {
   if (nkv <= 0 || nh % nkv || B <= 0 || B % 8) return 0;
   const int g = nh / nkv;
   return (hd == 64 || hd == 128) && g >= 1 && g <= 8;
+}
+
+// What the compiled kernel for this shape uses: out = {vector registers per lane, bytes of LDS
+// per workgroup, workgroups that fit on one CU, threads per workgroup}.
+int kvcm_attention_decode_fused_info(int nh, int nkv, int hd, int* out) {
+  KVCM_REQUIRE(kvcm_attention_decode_fused_supported(nh, nkv, hd, 8), "attention_decode_fused_info: unsupported shape");
+  const int rc = hd == 64 ? dispatch_fused_info<64>(nh / nkv, out) : dispatch_fused_info<128>(nh / nkv, out);
+  KVCM_REQUIRE(rc == 0, "attention_decode_fused_info: the runtime gave no attributes");
+  return 0;
 }
 
 // Rows of T different sequences.  The projection's result is either `partials` (split-K sums

@@ -37,6 +37,7 @@ def _declare(lib):
     fn("kvcm_attention_decode_fused_supported", i, i, i, i)
     fn("kvcm_attention_decode_fused", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, vp, i, vp)
     fn("kvcm_attention_generic_info", i, vp)
+    fn("kvcm_attention_decode_fused_info", i, i, i, vp)
     fn("kvcm_gemm_skinny_swiglu_supported", i, i, i)
     fn("kvcm_gemm_skinny_swiglu", vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_gemm_skinny_splits", i, i, i)
@@ -320,10 +321,13 @@ def attention_decode_supported(nh, nkv, hd, dtype, block_size=16):
 
 def attention_kernel_info(variant, nh, nkv, hd):
     """{"regs", "lds_bytes", "workgroups_per_cu", "threads"} of the compiled bfloat16 attention
-    kernel: variant "v1" (one pass per row and head) or "v2" (partitioned)."""
+    kernel: variant "v1" (one pass per row and head), "v2" (partitioned) or "fused" (one launch
+    with rotation and page write)."""
     out = (C.c_int * 4)()
     if variant == "v1":
         _check(lib().kvcm_attention_generic_info(hd, out))
+    elif variant == "fused":
+        _check(lib().kvcm_attention_decode_fused_info(nh, nkv, hd, out))
     else:
         _check(lib().kvcm_attention_decode_info(nh, nkv, hd, out))
     return dict(regs=out[0], lds_bytes=out[1], workgroups_per_cu=out[2], threads=out[3])

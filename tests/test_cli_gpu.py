@@ -26,13 +26,14 @@ def test_kvkernel_writes_one_row_per_variant(tmp_path):
     p = _run("kvkernel", "--ctx", "100,300", "--batch", "2", "--block-size", "16", "--iters", "3", "--out", out)
     assert p.returncode == 0, p.stderr
     rows = list(csv.DictReader(open(out)))
-    assert len(rows) == 8 and {r["variant"] for r in rows} == {"paged-v1", "contiguous-v1", "paged-v2", "contiguous-v2"}
+    assert len(rows) == 12 and {r["variant"] for r in rows} == {"paged-v1", "contiguous-v1", "paged-v2", "contiguous-v2",
+                                                                 "paged-fused", "contiguous-fused"}
     for r in rows:
         assert float(r["us"]) > 0 and float(r["gbps"]) > 0 and int(r["regs"]) > 0 and int(r["wgs_per_cu"]) >= 1
     assert "unsupported" not in p.stdout
     # a shape the partitioned kernel does not take is reported, not silently replaced
     p = _run("kvkernel", "--ctx", "64", "--batch", "1", "--heads", "12", "--kv-heads", "1", "--iters", "1")
-    assert p.returncode == 0 and p.stdout.count("unsupported") == 2
+    assert p.returncode == 0 and p.stdout.count("unsupported") == 4
 
 
 def test_kvbench_runs_a_small_workload(tmp_path):
