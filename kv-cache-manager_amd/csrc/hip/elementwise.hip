@@ -241,8 +241,8 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
   const bool is_q = h < nh, is_k = !is_q && h < nh + nkv;
   if (is_q || is_k) {
     T* cache_row = (is_k && slot >= 0) ? kcache + ((page * nkv + (h - nh)) * B + off) * hd : nullptr;
-    if (inv_freq) {
-      const float pos = float(positions[t]);
+    if (inv_freq || cos_sin) {
+      const float pos = cos_sin ? 0.f : float(positions[t]);
       for (int j = threadIdx.x; j < half; j += blockDim.x) {
         float sn, cs;
         if (cos_sin) {   // computed once per step by rope_table_kernel, the same values
@@ -312,7 +312,7 @@ __global__ void __launch_bounds__(256)
   float a[8], b[8];
   load4<T>(row + j0, a); load4<T>(row + j0 + 4, a + 4);
   load4<T>(row + half + j0, b); load4<T>(row + half + j0 + 4, b + 4);
-  if (inv_freq) {
+  if (inv_freq || cos_sin) {
     float cs[8], sn[8];
     if (cos_sin) {
       const float4* tab = reinterpret_cast<const float4*>(cos_sin + size_t(t) * half + j0);
@@ -452,8 +452,7 @@ int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, 
   KVCM_REQUIRE(hd > 0 && hd % 2 == 0, "rope: head_dim %d must be even", hd);
   KVCM_REQUIRE(nh >= 0 && nkv >= 0 && row_stride >= (nh + 2 * nkv) * hd, "rope: row stride %d too small", row_stride);
   KVCM_REQUIRE(!slots || (kcache && vcache && B > 0), "rope: cache write without a cache");
-  KVCM_REQUIRE(!inv_freq || positions, "rope: rotation without positions");
-  KVCM_REQUIRE(!cos_sin || inv_freq, "rope: a cos/sin table without rotation");
+  KVCM_REQUIRE(!inv_freq || positions || cos_sin, "rope: rotation without positions");
   KVCM_REQUIRE(!partials || S >= 1, "rope: partial sums need their split count");
   KVCM_REQUIRE(nh + 2 * nkv <= 65535 && nh + 2 * nkv > 0, "rope: too many heads");
   const bool aligned = reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&

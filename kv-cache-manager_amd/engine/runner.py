@@ -87,6 +87,7 @@ class StepContext:
         # to the largest context the engine allows, so that the launch fits every replay
         self.max_context_bound = max(L.max_context, 1)
         self.shared = {}    # what parts of one step compute once and share (keyed by the part kind)
+        self._leading = None
         d, h = runner.meta_dev, runner.meta_host
         T, S, R = self.rows, self.seqs, self.logit_rows_padded
         self.tokens = d[L.tokens:L.tokens + T]
@@ -104,6 +105,17 @@ class StepContext:
         self.host_seq_start = h[L.seq_start:L.seq_start + S]
         self.host_seq_end = h[L.seq_end:L.seq_end + S]
         self.host_state_slots = h[L.state_slots:L.state_slots + S]
+
+    def leading_single_runs(self):
+        """How many of the step's first sequences run exactly one token (the scheduler puts the
+        decoding requests first); their rows are the step's first rows."""
+        if self._leading is None:
+            rs = self.host_run_start[:self.real_seqs + 1]
+            n = 0
+            while n < self.real_seqs and rs[n + 1] - rs[n] == 1:
+                n += 1
+            self._leading = n
+        return self._leading
 
     def sampling_params(self):
         """(temperature f32, seeds i64 bit patterns, request ids i64, token index i32), one entry per
@@ -149,7 +161,8 @@ class ModelRunner:
         self.ops = model.ctx.ops
         self.workspace = Workspace(device, dtype, limits, self.ops)
         G = core.num_groups
-        ints = (4 * limits.max_tokens + 4 * limits.max_seqs + 1 + 7 * limits.max_logit_rows
+        # (logits of every row may be asked for and fetched in portions: room for that many indices)
+        ints = (4 * limits.max_tokens + 4 * limits.max_seqs + 1 + 7 * max(limits.max_logit_rows, limits.max_tokens)
                 + G * (limits.max_tokens + limits.max_seqs * limits.max_blocks_per_seq) + 64)
         self._pinned = torch.empty(ints, dtype=torch.int32, pin_memory=True)
         self.meta_host = self._pinned.numpy()
@@ -177,15 +190,38 @@ class ModelRunner:
     FUSED_DECODE_FULL_CHIP = 192
 
     def decode_attention_fused(self, step, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):
+        """From the QKV projection to the attention output.  Decode-shaped steps: one launch.  Mixed
+        steps (the scheduler puts decoding requests first): the leading single-token runs take that
+        launch too, the rows after them are rotated and stored, then attended by the tiled kernel;
+        a single-token run there would otherwise cost a whole tile of its own."""
         ops = self.ops
-        if (self.attn != "auto" or window != 0 or step.max_run != 1 or out.dtype != torch.bfloat16
-                or step.rows > self.DECODE_ATTENTION_MAX_ROWS
+        if (self.attn != "auto" or window != 0 or out.dtype != torch.bfloat16
                 or not ops.attention_decode_fused_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
             return False
-        if step.max_context_bound > self.FUSED_DECODE_MAX_CONTEXT and step.rows * nkv < self.FUSED_DECODE_FULL_CHIP:
+        if step.max_run == 1:
+            if step.rows > self.DECODE_ATTENTION_MAX_ROWS:
+                return False
+            if step.max_context_bound > self.FUSED_DECODE_MAX_CONTEXT and step.rows * nkv < self.FUSED_DECODE_FULL_CHIP:
+                return False
+            ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
+                                       step.ctx_lens, nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=step.rows)
+            return True
+        D, T, S = step.leading_single_runs(), step.real_rows, step.real_seqs
+        if (D == 0 or D > self.DECODE_ATTENTION_MAX_ROWS or isinstance(projection, ops.PartialSums)
+                or not ops.attention_prefill_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
             return False
-        ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
-                                   step.ctx_lens, nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=step.rows)
+        stride = step.table_stride(g)
+        ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), stride, step.row_seq, step.ctx_lens,
+                                   nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=D)
+        if (cos_sin is not None or slots is not None) and T > D:
+            ops.rope_cache(projection[D:T], nh, nkv, hd, cos_sin=cos_sin[D:T] if cos_sin is not None else None,
+                           slots=slots[D:T] if slots is not None else None, kcache=kcache, vcache=vcache,
+                           block_size=kcache.shape[2], rows=T - D)
+        need = ops.attention_prefill_scratch(T, nh, hd, step.max_context)
+        scratch = self.workspace.flat("prefill_partials", need) if need else None
+        ops.attention_prefill(projection, out, kcache, vcache, step.tables(g)[D * stride:], stride, step.run_start[D:],
+                              step.seq_start[D:], S - D, step.max_run, nh, nkv, hd, scale, rows=T,
+                              max_context=step.max_context, scratch=scratch)
         return True
 
     def attention(self, step, q, out, kcache, vcache, g, nh, nkv, hd, scale, window):
@@ -222,10 +258,11 @@ class ModelRunner:
                       step.ctx_lens, nh, nkv, hd, scale, window, rows=step.rows)
 
     # ------------------------------------------------------------------------------ steps
-    def _check(self, layout: BatchLayout):
+    def _check(self, layout: BatchLayout, logits_in_portions=False):
         lim = self.limits
         if (layout.rows_padded > lim.max_tokens or layout.seqs_padded > lim.max_seqs
-                or layout.logit_rows_padded > lim.max_logit_rows or layout.max_context > lim.max_context_len
+                or (layout.logit_rows_padded > lim.max_logit_rows and not logits_in_portions)
+                or layout.max_context > lim.max_context_len
                 or max(layout.table_stride + [0]) > lim.max_blocks_per_seq):
             raise RuntimeError(
                 f"step: batch exceeds model limits (rows {layout.rows_padded}/{lim.max_tokens}, sequences "
@@ -235,8 +272,8 @@ class ModelRunner:
         if layout.rows and (toks.min() < 0 or toks.max() >= self.vocab_size):
             raise ValueError(f"step: token id outside the vocabulary of {self.vocab_size}")
 
-    def _begin(self, layout: BatchLayout) -> StepContext:
-        self._check(layout)
+    def _begin(self, layout: BatchLayout, logits_in_portions=False) -> StepContext:
+        self._check(layout, logits_in_portions)
         n = layout.total
         self.meta_dev[:n].copy_(self._pinned[:n], non_blocking=True)
         self._upload_done.record()
@@ -264,7 +301,7 @@ class ModelRunner:
         at most max_logit_rows and the logits are gathered in host memory [logit_rows, vocab]."""
         if layout.rows == 0:
             return None
-        step = self._begin(layout)
+        step = self._begin(layout, logits_in_portions=True)
         x, pending = self.model.run_layers(step)
         R = layout.logit_rows
         if R == 0:

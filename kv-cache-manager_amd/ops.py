@@ -177,9 +177,11 @@ def rope_table(positions, inv_freq, out, rows=None):
 
 def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcache=None, vcache=None,
                block_size=0, rows=None, source=None, cos_sin=None):
-    """Rotates the q and k heads of the fused rows in place (inv_freq given) and copies k (rotated)
-    and v to the paged cache (slots given).  Cache layout [pages, nkv, block_size, hd].  With
-    ``source`` (PartialSums of the projection) the rows are read from there; q lands in ``qkv``."""
+    """Rotates the q and k heads of the fused rows in place (by the angles position * inv_freq, or
+    by a table ``cos_sin`` [rows, hd/2, 2] computed beforehand; neither: no rotation) and copies k
+    (rotated) and v to the paged cache (slots given).  Keys [pages, nkv, block_size, hd], values
+    [pages, nkv, hd, block_size].  With ``source`` (PartialSums of the projection) the rows are read
+    from there; q lands in ``qkv``."""
     _dev(qkv, positions, inv_freq, slots, kcache, vcache)
     _rows2d(qkv, "qkv")
     T = qkv.shape[0] if rows is None else rows
@@ -190,11 +192,12 @@ def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcac
     if inv_freq is not None:
         _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == hd // 2 and inv_freq.is_contiguous(),
               "inv_freq must hold head_dim/2 float32 values")
-        _i32(positions, "positions", T)
-        _need(positions is not None, "rotation needs positions")
+        if cos_sin is None:
+            _need(positions is not None, "rotation needs positions")
+            _i32(positions, "positions", T)
     if cos_sin is not None:
-        _need(inv_freq is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
-              and cos_sin.numel() >= T * hd, "cos_sin must be float32 [rows, head_dim/2, 2]")
+        _need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.numel() >= T * hd
+              and cos_sin.is_cuda, "cos_sin must be float32 [rows, head_dim/2, 2]")
     if slots is not None:
         _i32(slots, "slots", T)
         _need(kcache is not None and kcache.dtype == qkv.dtype and kcache.is_contiguous() and kcache.dim() == 4

@@ -19,9 +19,19 @@ TINY_B = dict(architectures=["LlamaForCausalLM"], vocab_size=384, hidden_size=96
 TINY_C = dict(architectures=["LlamaForCausalLM"], vocab_size=331, hidden_size=80, intermediate_size=136,
               num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=3, head_dim=48,
               max_position_embeddings=512, rope_theta=250000.0, rms_norm_eps=3e-6, tie_word_embeddings=False)
-BLOCK_SIZE = {"A": 16, "B": 8, "C": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-WEIGHT_SEED = {"A": 0, "B": 2, "C": 5}
+# sizes that the matrix-core kernels of the bfloat16 path take (head_dim 64, K a multiple of 64 and
+# long enough to be split): what the other three run through the general kernels, this one runs
+# through the kernels a served model meets, with contexts beyond one chunk of 256 and one segment of 1,024 keys
+TINY_D = dict(architectures=["LlamaForCausalLM"], vocab_size=300, hidden_size=256, intermediate_size=320,
+              num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+              max_position_embeddings=2048, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+BLOCK_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+WEIGHT_SEED = {"A": 0, "B": 2, "C": 5, "D": 7}
+# factor on the q and k projections: chosen per width so that scores have a spread of a few units
+# in every configuration (they grow with hidden_size * sqrt(head_dim); a spread of tens would make
+# the 32-bit rounding of the scores themselves, amplified by exp, the largest error in the test)
+SHARPEN = {"A": 12.0, "B": 12.0, "C": 12.0, "D": 6.0}
 
 
 def make_model_dir(path, raw, seed, dtype, sharpen=12.0):

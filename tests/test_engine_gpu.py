@@ -90,6 +90,53 @@ def test_temperature_generation_config_b_chunked(models, dtype):
         assert again == done
 
 
+def test_mixed_steps_at_matrix_core_sizes(tmp_path):
+    """head_dim 64, bfloat16: decoding requests (the scheduler puts them first) take the one-launch
+    decode kernel inside steps that also carry long prompt portions for the tiled kernel; graphs
+    replay the pure decode steps.  Greedy tokens must be those of the plain implementation."""
+    d = str(tmp_path / "m")
+    H.make_model_dir(d, H.TINY_D, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=H.SHARPEN["D"])
+    pm = plain.load_model_dir(d, plain.round_bf16)
+    prompts = _prompts(H.TINY_D, [40, 12, 700, 90, 1200, 25], seed=9)
+    eng = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, prefill_chunk=160, max_batched_tokens=200)
+    ids = [eng.add_request(p, 10) for p in prompts]
+    # which attention kernels the steps take (a silent fall back to the general kernel would pass the comparison)
+    ops, calls = eng.runner.ops, {"fused": 0, "fused_in_mixed": 0, "tiled": 0, "general": 0}
+    real = (ops.attention_decode_fused, ops.attention_prefill, ops.attention)
+
+    def fused(*a, **k):
+        calls["fused"] += 1
+        return real[0](*a, **k)
+
+    def tiled(*a, **k):
+        calls["tiled"] += 1
+        return real[1](*a, **k)
+
+    def general(*a, **k):
+        calls["general"] += 1
+        return real[2](*a, **k)
+
+    ops.attention_decode_fused, ops.attention_prefill, ops.attention = fused, tiled, general
+    try:
+        mixed_big, done = 0, {}
+        while not eng.idle():
+            before = dict(calls)
+            info = eng.step()
+            if info.decode_seqs > 0 and info.prefill_tokens >= 100:
+                mixed_big += 1
+                calls["fused_in_mixed"] += calls["fused"] > before["fused"] and calls["tiled"] > before["tiled"]
+            for f in eng.take_finished():
+                done[f.id] = f.generated
+    finally:
+        ops.attention_decode_fused, ops.attention_prefill, ops.attention = real
+    assert mixed_big > 3, "no step mixed decoding requests with a long prompt portion"
+    assert calls["fused_in_mixed"] == mixed_big and calls["general"] == 0, calls
+    for rid, p in zip(ids, prompts):
+        want, margins = pm.generate(p, 10)
+        assert _same_up_to_near_ties(done[rid], want, margins, 5e-2), (rid, done[rid], want, margins)
+    assert eng.core.blocks_in_use() == 0
+
+
 def test_preemption_recomputes_and_gives_the_same_tokens(models):
     d, pm = models[("A", "float32")]
     prompts = _prompts(H.TINY_A, [20, 25, 18, 30, 22, 19], seed=5)

@@ -17,7 +17,8 @@ import helpers as H
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LENGTHS = {"A": [7, 70, 13, 45, 5, 100, 33, 64], "B": [1, 9, 17, 33, 40, 130, 2, 65], "C": [50, 3, 97, 16, 31]}
+LENGTHS = {"A": [7, 70, 13, 45, 5, 100, 33, 64], "B": [1, 9, 17, 33, 40, 130, 2, 65], "C": [50, 3, 97, 16, 31],
+           "D": [300, 20, 1100, 65, 257]}
 
 
 def tolerance(dtype, ref):
@@ -35,7 +36,8 @@ def setups(tmp_path_factory):
     for name, raw in H.CONFIGS.items():
         for dtype in ("float32", "bfloat16"):
             d = str(tmp_path_factory.mktemp(f"model_{name}_{dtype}"))
-            H.make_model_dir(d, raw, H.WEIGHT_SEED[name], torch.float32 if dtype == "float32" else torch.bfloat16)
+            H.make_model_dir(d, raw, H.WEIGHT_SEED[name], torch.float32 if dtype == "float32" else torch.bfloat16,
+                             sharpen=H.SHARPEN[name])
             reqs = H.requests_for(raw, LENGTHS[name], seed=1 + H.WEIGHT_SEED[name])
             ref, _ = H.plain_logits(d, reqs, bf16=dtype == "bfloat16")
             rp = TraceReplayer(d, dtype, max_tokens=H.tokens_needed(reqs), block_size=H.BLOCK_SIZE[name])
@@ -43,7 +45,7 @@ def setups(tmp_path_factory):
     return out
 
 
-CASES = [(n, d) for n in ("A", "B", "C") for d in ("float32", "bfloat16")]
+CASES = [(n, d) for n in ("A", "B", "C", "D") for d in ("float32", "bfloat16")]
 
 
 def check(setups, case, steps):
@@ -81,7 +83,7 @@ def test_mixed_batches_with_reused_pages(setups, case, seed):
     check(setups, case, steps)
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_32bit_logits_do_not_depend_on_the_cutting(setups, name):
     """In 32-bit every kernel computes a row by a fixed sequence of operations, so the cuttings
     agree to the last bit, not just within rounding."""
