@@ -227,6 +227,24 @@ def test_graph_replays_equal_eager_steps(models, dtype):
     assert [done[i] for i in ids] == eager
 
 
+def test_graph_replays_at_matrix_core_sizes(tmp_path):
+    """head_dim 64, bfloat16: replayed decode steps (split products whose sums the one-launch decode
+    kernel and the norms add up, batch padded to a bucket, launch sized for the longest context
+    allowed) give the plain implementation's tokens, also while contexts cross chunks of 256."""
+    d = str(tmp_path / "m")
+    H.make_model_dir(d, H.TINY_D, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=H.SHARPEN["D"])
+    pm = plain.load_model_dir(d, plain.round_bf16)
+    prompts = _prompts(H.TINY_D, [250, 20, 505, 65, 1019], seed=11)
+    eng = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, max_batched_tokens=2048, use_graphs=True)
+    got = eng.generate(prompts, 24)
+    assert eng.decode_graphs.graphs, "no graph was captured"
+    for p, g in zip(prompts, got):
+        want, margins = pm.generate(p, 24)
+        assert _same_up_to_near_ties(g, want, margins, 5e-2), (len(p), g, want, margins)
+    eager = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, max_batched_tokens=2048, use_graphs=False)
+    assert eager.generate(prompts, 24) == got
+
+
 # -------------------------------------------------------------------------- parts, alone
 def _ctx(dtype, hidden):
     from kvcm_amd import ops
