@@ -136,91 +136,97 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// The same product for 17 .. 64 rows.  With that many rows X is no longer small: every 16-column
-// tile needs all of it, and re-reading it from L2 per tile would cost four times the weights'
-// bytes.  Here a workgroup owns 64 columns (one 16-column tile per wave) and a slice of K, and
-// its waves share X through LDS: per step of 64 k the workgroup stages X[rows][64] once
-// (double-buffered, the next step's global loads are issued before the current step's products),
-// every wave streams its own 16 weight rows from HBM and multiplies them with the staged rows.
-// No reduction between waves; split-K partial sums as above.  SWIGLU: a wave's tile is 8 gate + 8
-// up rows, the workgroup stores 32 activation columns.
+// The same product for more than 16 rows.  With that many rows X is no longer small: every
+// 16-column tile needs all of it, and re-reading it from L2 per tile would cost several times the
+// weights' bytes.  Here a workgroup owns 64 columns (one 16-column tile per wave), up to 128 rows
+// and a slice of K, and its waves share X through LDS: per trip of DEPTH x 64 k the workgroup
+// stages X[rows][DEPTH * 64] once (double-buffered; the next trip's global loads are issued before
+// the current trip's products), every wave streams its own 16 weight rows from HBM and multiplies
+// them with the staged rows.  No reduction between waves; split-K partial sums as above.  More
+// than 128 rows run as row blocks of 128 (blockIdx.z), each streaming the weights again.
+// SWIGLU: a wave's tile is 8 gate + 8 up rows, the workgroup stores 32 activation columns.
 constexpr int kXPad = 8;    // bfloat16 of padding per staged row, so that rows spread over the banks
-constexpr int kDepth = 4;   // units of 64 k per trip: what a lane has in flight is 4 x (32 B of W + 32 B of X)
+constexpr int kRowBlock = 128;
 
-// KH = 2: eight waves, the second four take the second half of the workgroup's K slice with X
-// buffers of their own, and the halves are added through LDS at the end (first half + second
-// half).  For launches with far fewer workgroups than CUs (a product that may not be split and
-// has few columns): twice the waves at work per CU.
-template <int MT, int KH, class TO, bool SWIGLU>
-__global__ void __launch_bounds__(256 * KH)
-    gemm_rows64_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ partials,
-                       TO* __restrict__ out, int M, int N, int K, int ldx, int ldw, int ldo, int S) {
-  __shared__ __attribute__((aligned(16))) uint16_t xs[KH][2][MT * 16][kDepth * kUnit + kXPad];
-  const int kh = threadIdx.x / 256, tid = threadIdx.x % 256;
-  const int wave = tid / kWave, lane = tid % kWave;
+template <int MT, int DEPTH, class TO, bool SWIGLU>
+__global__ void __launch_bounds__(256)
+    gemm_rows_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ partials,
+                     TO* __restrict__ out, int M, int N, int K, int ldx, int ldw, int ldo, int S) {
+  constexpr int RP = (MT * 16 + 63) / 64;   // staging passes: 256 threads move 64 rows x 64 k at a time
+  __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][DEPTH * kUnit + kXPad];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int r = lane % 16, kq = lane / 16;
   constexpr int kCols = SWIGLU ? 8 : 16;
   const int c0 = blockIdx.x * (4 * kCols) + wave * kCols;   // this wave's first output column
   const int s = blockIdx.y;
+  const int row_base = blockIdx.z * kRowBlock;
   const int units = K / kUnit;
-  const int s_lo = int((long long)units * s / S), s_hi = int((long long)units * (s + 1) / S);
-  const int u_lo = s_lo + (s_hi - s_lo) * kh / KH, u_hi = s_lo + (s_hi - s_lo) * (kh + 1) / KH;
-  // every wave of the workgroup runs the same number of trips (and barriers): that of the longer half
-  const int trips = ((s_hi - s_lo + KH - 1) / KH + kDepth - 1) / kDepth;
+  const int u_lo = int((long long)units * s / S), u_hi = int((long long)units * (s + 1) / S);
+  const int trips = (u_hi - u_lo + DEPTH - 1) / DEPTH;
 
   const uint16_t* wrow = W + size_t(SWIGLU ? (r < 8 ? c0 + r : N + c0 + r - 8) : c0 + r) * ldw + kq * 16;
-  // staging: thread -> (row tid / 4, 16 elements at (tid % 4) * 16 of every unit); rows beyond M
-  // read row 0 and are dropped at the store
-  const int srow = tid / 4, sseg = (tid % 4) * 16;
-  const bool stages = srow < MT * 16;                         // uniform per wave
-  const uint16_t* xsrc = X + size_t(srow < M ? srow : 0) * ldx + sseg;
+  // staging: thread -> (row tid / 4 + 64 p, 16 elements at (tid % 4) * 16 of every unit); rows
+  // beyond M read the block's first row and are dropped at the store
+  const int srow = threadIdx.x / 4, sseg = (threadIdx.x % 4) * 16;
+  const uint16_t* xsrc[RP];
+#pragma unroll
+  for (int p = 0; p < RP; ++p) {
+    const int m = row_base + srow + 64 * p;
+    xsrc[p] = X + size_t(m < M ? m : row_base) * ldx + sseg;
+  }
 
   f32x4 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // A trip's operands: kDepth units of this wave's weight rows and of this thread's piece of X.
+  // A trip's operands: DEPTH units of this wave's weight rows and of this thread's pieces of X.
   // Units beyond the slice repeat its last unit (no load behind a branch) and are not multiplied.
   struct Trip {
-    Frag b[kDepth][2];
-    uint4 x[kDepth][2];
+    Frag b[DEPTH][2];
+    uint4 x[DEPTH][RP][2];
   };
   // Workgroups walk their slice from different starting points (and wrap around): if all of them
   // read the same k at the same time, their rows, a multiple of 4 KB apart, would queue up at the
   // same few memory channels.
-  const int span = u_hi - u_lo > 0 ? u_hi - u_lo : 1;   // (an empty half cannot happen: a slice has at least KH units)
-  const int phase = (blockIdx.x * 5) % span;   // the same for all waves that share staged X
+  const int span = u_hi - u_lo > 0 ? u_hi - u_lo : 1;
+  const int phase = (blockIdx.x * 5) % span;   // the same for all waves: they share staged X
   auto fetch = [&](int j0, Trip& tr) {
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
+    for (int d = 0; d < DEPTH; ++d) {
       const int j = j0 + d < span ? j0 + d : span - 1;
       const int u = u_lo + (j + phase) % span;
       const uint16_t* p = wrow + size_t(u) * kUnit;
       tr.b[d][0].u = *reinterpret_cast<const uint4*>(p);
       tr.b[d][1].u = *reinterpret_cast<const uint4*>(p + 8);
-      const uint16_t* q = xsrc + size_t(u) * kUnit;
-      tr.x[d][0] = *reinterpret_cast<const uint4*>(q);
-      tr.x[d][1] = *reinterpret_cast<const uint4*>(q + 8);
+#pragma unroll
+      for (int q = 0; q < RP; ++q) {
+        const uint16_t* xp = xsrc[q] + size_t(u) * kUnit;
+        tr.x[d][q][0] = *reinterpret_cast<const uint4*>(xp);
+        tr.x[d][q][1] = *reinterpret_cast<const uint4*>(xp + 8);
+      }
     }
   };
   auto stage = [&](int buf, const Trip& tr) {
-    if (stages) {
 #pragma unroll
-      for (int d = 0; d < kDepth; ++d) {
-        *reinterpret_cast<uint4*>(&xs[kh][buf][srow][d * kUnit + sseg]) = tr.x[d][0];
-        *reinterpret_cast<uint4*>(&xs[kh][buf][srow][d * kUnit + sseg + 8]) = tr.x[d][1];
+    for (int q = 0; q < RP; ++q) {
+      if (srow + 64 * q < MT * 16) {   // uniform per wave
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+          *reinterpret_cast<uint4*>(&xs[buf][srow + 64 * q][d * kUnit + sseg]) = tr.x[d][q][0];
+          *reinterpret_cast<uint4*>(&xs[buf][srow + 64 * q][d * kUnit + sseg + 8]) = tr.x[d][q][1];
+        }
       }
     }
   };
   auto multiply = [&](int buf, int j0, const Trip& tr) {
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
+    for (int d = 0; d < DEPTH; ++d) {
       if (j0 + d >= span) break;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         Frag a0, a1;
-        a0.u = *reinterpret_cast<const uint4*>(&xs[kh][buf][t * 16 + r][d * kUnit + kq * 16]);
-        a1.u = *reinterpret_cast<const uint4*>(&xs[kh][buf][t * 16 + r][d * kUnit + kq * 16 + 8]);
+        a0.u = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + r][d * kUnit + kq * 16]);
+        a1.u = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + r][d * kUnit + kq * 16 + 8]);
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0.v, tr.b[d][0].v, acc[t], 0, 0, 0);
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1.v, tr.b[d][1].v, acc[t], 0, 0, 0);
       }
@@ -229,35 +235,20 @@ __global__ void __launch_bounds__(256 * KH)
   // Two trips in registers: while one is multiplied, the next one's loads are on their way.  LDS
   // buffer i holds the X of the trip in register set i; a buffer is written one barrier after its
   // last read.
-  {
+  if (u_lo < u_hi) {
     Trip ta, tb;
     fetch(0, ta);
     for (int i = 0; i < trips; i += 2) {
-      const int j0 = i * kDepth;
-      fetch(j0 + kDepth, tb);
+      const int j0 = i * DEPTH;
+      fetch(j0 + DEPTH, tb);
       stage(0, ta);
       __syncthreads();
       multiply(0, j0, ta);
       if (i + 1 >= trips) break;
-      fetch(j0 + 2 * kDepth, ta);
+      fetch(j0 + 2 * DEPTH, ta);
       stage(1, tb);
       __syncthreads();
-      multiply(1, j0 + kDepth, tb);
-    }
-  }
-  if constexpr (KH == 2) {   // second half -> LDS -> first half
-    __syncthreads();         // nobody reads staged X any more
-    f32x4* red = reinterpret_cast<f32x4*>(&xs[0][0][0][0]);
-    if (kh == 1) {
-#pragma unroll
-      for (int t = 0; t < MT; ++t) red[(wave * MT + t) * kWave + lane] = acc[t];
-    }
-    __syncthreads();
-    if (kh == 1) return;
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const f32x4 o = red[(wave * MT + t) * kWave + lane];
-      acc[t][0] += o[0]; acc[t][1] += o[1]; acc[t][2] += o[2]; acc[t][3] += o[3];
+      multiply(1, j0 + DEPTH, tb);
     }
   }
   // accumulator: column = r of the wave's tile, rows = 4 kq + i
@@ -270,7 +261,7 @@ __global__ void __launch_bounds__(256 * KH)
       if (r >= 8) continue;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int m = t * 16 + kq * 4 + i;
+        const int m = row_base + t * 16 + kq * 4 + i;
         if (m >= M) continue;
         const float x = round_to<TO>(acc[t][i]);
         const float act = x / (1.0f + expf(-x));
@@ -283,7 +274,7 @@ __global__ void __launch_bounds__(256 * KH)
   for (int t = 0; t < MT; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int m = t * 16 + kq * 4 + i;
+      const int m = row_base + t * 16 + kq * 4 + i;
       if (m >= M) continue;
       if (S > 1) partials[(size_t(s) * M + m) * N + c0 + r] = acc[t][i];
       else store_f(out + size_t(m) * ldo + c0 + r, acc[t][i]);
@@ -304,22 +295,46 @@ __global__ void reduce_store_kernel(const float* __restrict__ partials, TO* __re
 
 using namespace kvcm;
 
-extern "C" {
+constexpr int kMaxSharedRows = 512;
 
 // More than 16 rows and whole groups of 64 columns: the kernel whose waves share X through LDS.
-static bool shares_rows(int M, int N) { return M > 16 && N % 64 == 0; }
+static bool shares_rows(int M, int N) { return M > 16 && M <= kMaxSharedRows && N % 64 == 0; }
+static int row_blocks(int M) { return (M + kRowBlock - 1) / kRowBlock; }
+
+// One launch of the shared-rows kernel: MT row tiles per block (8 for every block when there are
+// several), two k-depths: four units per trip up to 64 rows, two beyond (LDS holds rows x depth).
+template <class TO, bool SWIGLU>
+static void launch_rows(dim3 grid, hipStream_t st, const uint16_t* x, const uint16_t* w, float* partials, TO* out, int M,
+                        int N, int K, int ldx, int ldw, int ldo, int S) {
+  const int mt = M > kRowBlock ? kRowBlock / 16 : (M + 15) / 16;
+#define KVCM_ROWS(MT, DEPTH) \
+  gemm_rows_kernel<MT, DEPTH, TO, SWIGLU><<<grid, 256, 0, st>>>(x, w, partials, out, M, N, K, ldx, ldw, ldo, S)
+  switch (mt) {
+    case 1: case 2: KVCM_ROWS(2, 4); break;
+    case 3: KVCM_ROWS(3, 4); break;
+    case 4: KVCM_ROWS(4, 4); break;
+    case 5: case 6: KVCM_ROWS(6, 2); break;
+    default: KVCM_ROWS(8, 2); break;
+  }
+#undef KVCM_ROWS
+}
+
+
+extern "C" {
 
 // How many splits of K a launch of this shape uses (0: the shape is not supported by this kernel).
 int kvcm_gemm_skinny_splits(int M, int N, int K) {
-  if (M <= 0 || M > 64 || N % 16 != 0 || K % kUnit != 0 || N <= 0 || K <= 0) return 0;
+  if (M <= 0 || N % 16 != 0 || K % kUnit != 0 || N <= 0 || K <= 0) return 0;
   if (shares_rows(M, N)) {
-    const int groups = N / 64, units = K / kUnit;
+    const int groups = (N / 64) * row_blocks(M), units = K / kUnit;
     if (groups >= 256) return 1;
     int S = (512 + groups - 1) / groups;       // aim at two workgroups per CU ...
-    if (S > units / 4) S = units / 4;          // ... of at least four steps each ...
-    if (S > 8) S = 8;                          // ... and partial sums that stay small beside the weights
+    if (S > units / 4) S = units / 4;          // ... of at least four units each ...
+    if (S > K / (4 * M)) S = K / (4 * M);      // ... and partial sums (S*M*N floats) that stay below the weights' bytes
+    if (S > 8) S = 8;
     return S < 1 ? 1 : S;
   }
+  if (M > 64) return 0;
   const int tiles = N / 16, units = K / kUnit;
   int S = (640 + tiles - 1) / tiles;           // aim at >= 640 workgroups (2.5 per CU)
   if (S > units / 2) S = units / 2;            // at least two units per split ...
@@ -339,38 +354,23 @@ int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, i
                "gemm_skinny: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
   KVCM_REQUIRE(ldx >= K && ldw >= K, "gemm_skinny: leading dimensions too small");
   KVCM_REQUIRE(S == 1 ? (out != nullptr && ldo >= N) : partials != nullptr, "gemm_skinny: missing output buffer");
+  KVCM_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "gemm_skinny: unknown output dtype %d", out_dtype);
   const uint16_t* x = static_cast<const uint16_t*>(X);
   const uint16_t* w = static_cast<const uint16_t*>(W);
   const int mt = (M + 15) / 16;
   if (shares_rows(M, N)) {
-    const dim3 grid64(N / 64, S);
-    const bool two_halves = (N / 64) * S < 128 && K / kUnit / S >= 4 * kDepth;   // far fewer workgroups than CUs
-#define KVCM_ROWS64(MT, TO) \
-  do {                                                                                                             \
-    if (two_halves)                                                                                                \
-      gemm_rows64_kernel<MT, 2, TO, false><<<grid64, 512, 0, st>>>(x, w, partials, static_cast<TO*>(out), M, N, K, ldx, ldw, ldo, S); \
-    else                                                                                                           \
-      gemm_rows64_kernel<MT, 1, TO, false><<<grid64, 256, 0, st>>>(x, w, partials, static_cast<TO*>(out), M, N, K, ldx, ldw, ldo, S); \
-  } while (0)
-    if (out_dtype == kBF16) {
-      if (mt == 2) KVCM_ROWS64(2, bf16_t); else if (mt == 3) KVCM_ROWS64(3, bf16_t); else KVCM_ROWS64(4, bf16_t);
-    } else if (out_dtype == kF32) {
-      if (mt == 2) KVCM_ROWS64(2, float); else if (mt == 3) KVCM_ROWS64(3, float); else KVCM_ROWS64(4, float);
-    } else {
-      KVCM_REQUIRE(false, "gemm_skinny: unknown output dtype %d", out_dtype);
-    }
-#undef KVCM_ROWS64
-    return launch_status("gemm_rows64");
+    const dim3 grid(N / 64, S, row_blocks(M));
+    if (out_dtype == kBF16) launch_rows<bf16_t, false>(grid, st, x, w, partials, static_cast<bf16_t*>(out), M, N, K, ldx, ldw, ldo, S);
+    else launch_rows<float, false>(grid, st, x, w, partials, static_cast<float*>(out), M, N, K, ldx, ldw, ldo, S);
+    return launch_status("gemm_rows");
   }
   const dim3 grid(N / 16, S);
 #define KVCM_SKINNY(MT, TO) \
   gemm_skinny_kernel<MT, TO, false><<<grid, 256, 0, st>>>(x, w, partials, static_cast<TO*>(out), M, N, K, ldx, ldw, ldo, S)
   if (out_dtype == kBF16) {
     if (mt == 1) KVCM_SKINNY(1, bf16_t); else if (mt == 2) KVCM_SKINNY(2, bf16_t); else if (mt == 3) KVCM_SKINNY(3, bf16_t); else KVCM_SKINNY(4, bf16_t);
-  } else if (out_dtype == kF32) {
-    if (mt == 1) KVCM_SKINNY(1, float); else if (mt == 2) KVCM_SKINNY(2, float); else if (mt == 3) KVCM_SKINNY(3, float); else KVCM_SKINNY(4, float);
   } else {
-    KVCM_REQUIRE(false, "gemm_skinny: unknown output dtype %d", out_dtype);
+    if (mt == 1) KVCM_SKINNY(1, float); else if (mt == 2) KVCM_SKINNY(2, float); else if (mt == 3) KVCM_SKINNY(3, float); else KVCM_SKINNY(4, float);
   }
 #undef KVCM_SKINNY
   return launch_status("gemm_skinny");
@@ -378,10 +378,10 @@ int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, i
 
 // May act = swiglu(X * [gate | up]^T) be computed in one launch?  I is the width of the result.
 int kvcm_gemm_skinny_swiglu_supported(int M, int I, int K) {
-  if (!(M > 0 && M <= 64 && I > 0 && I % 8 == 0 && K > 0 && K % kUnit == 0)) return 0;
+  if (!(M > 0 && I > 0 && I % 8 == 0 && K > 0 && K % kUnit == 0)) return 0;
   // with too few workgroups a split product fills the chip better than this unsplit one
-  if (M > 16 && I % 32 == 0) return I / 32 >= 160;
-  return I / 8 >= 320;
+  if (M > 16 && M <= kMaxSharedRows && I % 32 == 0) return (I / 32) * row_blocks(M) >= 160;
+  return M <= 64 && I / 8 >= 320;
 }
 
 // W [2 I, K] (gate rows, then up rows); out [M, I].
@@ -392,38 +392,23 @@ int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dty
                    reinterpret_cast<uintptr_t>(W) % 16 == 0,
                "gemm_skinny_swiglu: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
   KVCM_REQUIRE(ldx >= K && ldw >= K && out != nullptr && ldo >= I, "gemm_skinny_swiglu: leading dimensions too small");
+  KVCM_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "gemm_skinny_swiglu: unknown output dtype %d", out_dtype);
   const uint16_t* x = static_cast<const uint16_t*>(X);
   const uint16_t* w = static_cast<const uint16_t*>(W);
   const int mt = (M + 15) / 16;
-  if (M > 16 && I % 32 == 0) {
-    const dim3 grid32(I / 32, 1);
-    const bool two_halves = I / 32 < 128 && K / kUnit >= 4 * kDepth;   // far fewer workgroups than CUs
-#define KVCM_ROWS64(MT, TO) \
-  do {                                                                                                             \
-    if (two_halves)                                                                                                \
-      gemm_rows64_kernel<MT, 2, TO, true><<<grid32, 512, 0, st>>>(x, w, nullptr, static_cast<TO*>(out), M, I, K, ldx, ldw, ldo, 1); \
-    else                                                                                                           \
-      gemm_rows64_kernel<MT, 1, TO, true><<<grid32, 256, 0, st>>>(x, w, nullptr, static_cast<TO*>(out), M, I, K, ldx, ldw, ldo, 1); \
-  } while (0)
-    if (out_dtype == kBF16) {
-      if (mt == 2) KVCM_ROWS64(2, bf16_t); else if (mt == 3) KVCM_ROWS64(3, bf16_t); else KVCM_ROWS64(4, bf16_t);
-    } else if (out_dtype == kF32) {
-      if (mt == 2) KVCM_ROWS64(2, float); else if (mt == 3) KVCM_ROWS64(3, float); else KVCM_ROWS64(4, float);
-    } else {
-      KVCM_REQUIRE(false, "gemm_skinny_swiglu: unknown output dtype %d", out_dtype);
-    }
-#undef KVCM_ROWS64
-    return launch_status("gemm_rows64_swiglu");
+  if (M > 16 && M <= kMaxSharedRows && I % 32 == 0) {
+    const dim3 grid(I / 32, 1, row_blocks(M));
+    if (out_dtype == kBF16) launch_rows<bf16_t, true>(grid, st, x, w, nullptr, static_cast<bf16_t*>(out), M, I, K, ldx, ldw, ldo, 1);
+    else launch_rows<float, true>(grid, st, x, w, nullptr, static_cast<float*>(out), M, I, K, ldx, ldw, ldo, 1);
+    return launch_status("gemm_rows_swiglu");
   }
   const dim3 grid(I / 8, 1);
 #define KVCM_SKINNY(MT, TO) \
   gemm_skinny_kernel<MT, TO, true><<<grid, 256, 0, st>>>(x, w, nullptr, static_cast<TO*>(out), M, I, K, ldx, ldw, ldo, 1)
   if (out_dtype == kBF16) {
     if (mt == 1) KVCM_SKINNY(1, bf16_t); else if (mt == 2) KVCM_SKINNY(2, bf16_t); else if (mt == 3) KVCM_SKINNY(3, bf16_t); else KVCM_SKINNY(4, bf16_t);
-  } else if (out_dtype == kF32) {
-    if (mt == 1) KVCM_SKINNY(1, float); else if (mt == 2) KVCM_SKINNY(2, float); else if (mt == 3) KVCM_SKINNY(3, float); else KVCM_SKINNY(4, float);
   } else {
-    KVCM_REQUIRE(false, "gemm_skinny_swiglu: unknown output dtype %d", out_dtype);
+    if (mt == 1) KVCM_SKINNY(1, float); else if (mt == 2) KVCM_SKINNY(2, float); else if (mt == 3) KVCM_SKINNY(3, float); else KVCM_SKINNY(4, float);
   }
 #undef KVCM_SKINNY
   return launch_status("gemm_skinny_swiglu");

@@ -54,9 +54,16 @@ class Workspace:
         when that shape is not split.  Sized once for the most rows the split kernel takes."""
         key = ("scratch", name, n, k)
         if key not in self.buffers:
-            splits = self.ops.skinny_splits(min(64, max(rows, 1)), n, k) if self.ops is not None else 0
-            self.buffers[key] = (torch.empty(splits * 64 * n, dtype=torch.float32, device=self.device)
-                                 if splits > 1 else None)
+            # the number of splits changes with the rows: room for the worst of the row counts at
+            # which it can change
+            need = 0
+            if self.ops is not None:
+                for m in (1, 16, 17, 32, 64, 65, 128, 129, 256, 257, 512):
+                    m = min(m, self.limits.max_tokens)
+                    splits = self.ops.skinny_splits(m, n, k)
+                    if splits > 1:
+                        need = max(need, splits * m * n)
+            self.buffers[key] = torch.empty(need, dtype=torch.float32, device=self.device) if need else None
         return self.buffers[key]
 
     def flat(self, name, numel, dtype=torch.float32):
@@ -139,7 +146,7 @@ class StepContext:
         return self.runner.workspace.get(name, shape, dtype)
 
     def scratch(self, name, rows, n, k):
-        if rows > 64 or self.runner.dtype != torch.bfloat16:
+        if rows > 512 or self.runner.dtype != torch.bfloat16:
             return None
         return self.runner.workspace.scratch(name, rows, n, k)
 

@@ -239,8 +239,9 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
     """out[M, N] = x[M, K] @ w[N, K]^T.  float32 x float32 -> float32 (plain FMA, fixed k order), or
     bfloat16 x bfloat16 -> bfloat16 | float32 (MFMA, 32-bit accumulation).
 
-    For few rows (M <= 64) of a bfloat16 product the weight-streaming kernel is used; when it
-    splits K it needs ``scratch`` (float32, at least splits*M*N elements).  With ``keep_partial``
+    Rows below LIBRARY_GEMM_MIN_ROWS take the weight-streaming kernels (also more rows, up to 512,
+    while the library is switched off: inside a captured graph); when they split K they need
+    ``scratch`` (float32, at least splits*M*N elements).  With ``keep_partial``
     the un-added partial sums are returned as PartialSums (for a fused consumer) instead of ``out``.
     """
     _dev(x, w, out)
@@ -254,8 +255,9 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
         _check(lib().kvcm_gemm_f32(_ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0), _stream()))
         return out
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm operands must both be bfloat16")
-    S = skinny_splits(M, N, K) if (x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
-                                   and w.data_ptr() % 16 == 0) else 0
+    library = bool(LIBRARY_GEMM_MIN_ROWS) and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 and out.is_contiguous()
+    S = skinny_splits(M, N, K) if (not library and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+                                   and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0) else 0
     if S > 1 and (scratch is None or scratch.numel() < S * M * N):
         S = 1 if scratch is None else max(1, min(S, scratch.numel() // (M * N)))
     if S >= 1:
@@ -267,7 +269,7 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
             return out
         partial = PartialSums(scratch, S, M, N, out)
         return partial if keep_partial else partial.materialize()
-    if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 and out.is_contiguous():
+    if library:
         torch.matmul(x, w.t(), out=out)
         return out
     _check(lib().kvcm_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, x.stride(0), w.stride(0),
@@ -285,6 +287,8 @@ def gemm_swiglu(x, w_gate_up, out):
     M, K = x.shape
     I = out.shape[1]
     _need(w_gate_up.shape == (2 * I, K) and out.shape[0] == M, "gemm_swiglu shapes do not agree")
+    if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS:
+        return False          # many rows: the library product, then swiglu
     if not (x.dtype == w_gate_up.dtype == out.dtype == torch.bfloat16 and x.stride(0) % 8 == 0
             and w_gate_up.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
             and lib().kvcm_gemm_skinny_swiglu_supported(M, I, K)):

@@ -529,6 +529,40 @@ def test_gemm_skinny_with_and_without_splits(ops, M, N, K):
     np.testing.assert_allclose(_np(out), ref, rtol=0, atol=2e-5 * math.sqrt(K))
 
 
+@pytest.mark.parametrize("M", [65, 96, 100, 128, 129, 300, 512])
+@pytest.mark.parametrize("N,K", [(2048, 2048), (2560, 512), (192, 320)])
+def test_gemm_shared_rows_beyond_64_rows(ops, M, N, K):
+    """The weight-streaming kernel for up to 512 rows (row blocks of 128), which the engine uses
+    where the library product may not run: inside captured graphs."""
+    rng = np.random.default_rng(M + N)
+    x = _bf16_grid(rng.normal(size=(M, K)))
+    w = _bf16_grid(rng.normal(size=(N, K)) * 0.05)
+    ref = plain.linear(x, w)
+    xt, wt = _t(x, torch.bfloat16), _t(w, torch.bfloat16)
+    keep, ops.LIBRARY_GEMM_MIN_ROWS = ops.LIBRARY_GEMM_MIN_ROWS, 0
+    try:
+        S = ops.skinny_splits(M, N, K)
+        assert S >= 1
+        scratch = torch.zeros(S * M * N, dtype=torch.float32, device=DEV)
+        out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        ops.gemm(xt, wt, out, scratch=scratch)
+        np.testing.assert_allclose(_np(out), ref, rtol=2 ** -7, atol=1e-3)
+        out32 = torch.zeros(M, N, dtype=torch.float32, device=DEV)
+        ops.gemm(xt, wt, out32)                                             # unsplit
+        np.testing.assert_allclose(_np(out32), ref, rtol=0, atol=2e-5 * math.sqrt(K))
+        if N % 64 == 0 and N >= 2048:                                       # gate/up with the SwiGLU epilogue
+            I = N // 2
+            act = torch.zeros(M, I, dtype=torch.bfloat16, device=DEV)
+            if ops.gemm_swiglu(xt, wt, act):
+                want = torch.zeros_like(act)
+                ops.swiglu(out, want)
+                a, b = _np(act), _np(want)
+                assert np.mean(a == b) > 0.98
+                np.testing.assert_allclose(a, b, rtol=2 ** -6, atol=2e-3)
+    finally:
+        ops.LIBRARY_GEMM_MIN_ROWS = keep
+
+
 def test_partial_sums_feed_the_fused_norm_and_rope(ops):
     rng = np.random.default_rng(30)
     M, H, K = 5, 2048, 2048
