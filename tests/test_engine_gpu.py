@@ -245,6 +245,38 @@ def test_graph_replays_at_matrix_core_sizes(tmp_path):
     assert eager.generate(prompts, 24) == got
 
 
+@pytest.mark.parametrize("attn", ["v1", "v2"])
+def test_attention_variants_at_matrix_core_sizes(tmp_path, attn):
+    """--attn v1 (one-pass kernel everywhere) and v2 (partitions + merge for decode steps, after a
+    separate rotation + page write that reads the split sums) give the plain implementation's
+    tokens too; "auto" is covered by the tests above."""
+    d = str(tmp_path / "m")
+    H.make_model_dir(d, H.TINY_D, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=H.SHARPEN["D"])
+    pm = plain.load_model_dir(d, plain.round_bf16)
+    prompts = _prompts(H.TINY_D, [250, 33, 520], seed=12)
+    eng = _engine(d, dtype="bfloat16", num_blocks=100, max_seq_len=1024, max_batched_tokens=1024, attn=attn)
+    ops, calls = eng.runner.ops, {"fused": 0, "partitioned": 0}
+    real = (ops.attention_decode_fused, ops.attention_decode)
+
+    def fused(*a, **k):
+        calls["fused"] += 1
+        return real[0](*a, **k)
+
+    def partitioned(*a, **k):
+        calls["partitioned"] += 1
+        return real[1](*a, **k)
+
+    ops.attention_decode_fused, ops.attention_decode = fused, partitioned
+    try:
+        got = eng.generate(prompts, 12)
+    finally:
+        ops.attention_decode_fused, ops.attention_decode = real
+    assert calls["fused"] == 0 and (calls["partitioned"] > 0) == (attn == "v2"), calls
+    for p, g in zip(prompts, got):
+        want, margins = pm.generate(p, 12)
+        assert _same_up_to_near_ties(g, want, margins, 5e-2), (len(p), g, want, margins)
+
+
 # -------------------------------------------------------------------------- parts, alone
 def _ctx(dtype, hidden):
     from kvcm_amd import ops
