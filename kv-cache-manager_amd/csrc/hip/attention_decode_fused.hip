@@ -5,11 +5,13 @@
 // decode step is bound by the number of dependent launches, not by bytes, so they are one here.
 //
 // One workgroup per (kv head, row) serves the row's whole query group.  After a common prologue
-// (q to LDS, new key and value to their page) its four waves work on their own: the context is
-// walked in chunks of 256 tokens, wave w takes tokens 64 w .. 64 w + 63 of every chunk, keeps its
-// own running maximum, sum and output, and asks for the keys and values of its next chunk before
-// it computes the current one.  No barrier inside the loop; the four partial results are merged
-// through LDS at the end, always in wave order.
+// (q to LDS, new key and value to their page) its waves work on their own: the context is walked
+// in chunks of 256 tokens; with head_dim 64 there are eight waves, wave w takes tokens
+// 64 (w % 4) .. + 63 of every second chunk (starting at chunk w / 4), with head_dim 128 four waves
+// take every chunk (registers).  A wave keeps its own running maximum, sum and output, and asks
+// for the keys and values of its next chunk before it computes the current one.  No barrier
+// inside the loop; the waves' partial results are merged through LDS at the end, always in wave
+// order.
 //
 // Both products run on the matrix cores, transposed: S^T = K Q^T puts one query head in each
 // accumulator column, so a lane's softmax concerns one head only and its eight probabilities of a
@@ -25,7 +27,7 @@
 
 namespace kvcm {
 
-constexpr int kFusWaves = 4;
+template <int HD> struct FusWaves { static constexpr int N = HD == 64 ? 8 : 4; };
 constexpr int kFusChunk = 256;
 constexpr float kFusNone = -1.0e30f;   // "no score yet": finite, so that differences stay finite
 
@@ -44,7 +46,7 @@ __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
 }
 
 template <int HD, int GROUP>
-__global__ void __launch_bounds__(kFusWaves* kWave)
+__global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
     attention_decode_fused_kernel(const float* __restrict__ partials, int S, size_t pstride,
                                   const uint16_t* __restrict__ qkv, int qkv_stride,
                                   const float2* __restrict__ cos_sin, const int* __restrict__ slots,
@@ -55,9 +57,12 @@ __global__ void __launch_bounds__(kFusWaves* kWave)
   constexpr int KSTEPS = HD / 32;   // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;       // 16-dim tiles of the output
   constexpr int HALF = HD / 2;
+  constexpr int kFusWaves = FusWaves<HD>::N;
+  constexpr int STRIDE = kFusWaves / 4;   // a wave takes every STRIDE-th chunk
   const int kvh = blockIdx.x, row = blockIdx.y;
   const int ctx = ctx_lens[row];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int wq = wave % 4, wfirst = wave / 4;   // which quarter of a chunk, and the first chunk, are this wave's
 
   __shared__ __attribute__((aligned(16))) uint16_t q_lds[GROUP][HD];
   __shared__ __attribute__((aligned(16))) float red[kFusWaves][16][HD + 4];
@@ -80,7 +85,7 @@ __global__ void __launch_bounds__(kFusWaves* kWave)
   // masked out.  The lanes that need an offset get it by a shuffle.
   struct Where { uint32_t k, v; };
   auto lookup = [&](int c) {
-    const int t0 = c * kFusChunk + wave * 64 + lane;
+    const int t0 = c * kFusChunk + wq * 64 + lane;
     const int t = min(t0, ctx - 1), tv = min(t0, (ctx - 1) & ~7);
     const int pk = table[t / B], pv = table[tv / B];
     Where w;
@@ -88,8 +93,12 @@ __global__ void __launch_bounds__(kFusWaves* kWave)
     w.v = uint32_t((size_t(pv) * page_elems + kvh * head_elems + tv % B) / 8);
     return w;
   };
-  // lookups run two chunks ahead of the computation, so that their trip to memory is never waited for
-  Where wha = lookup(0), whb = lookup(min(1, last));
+  // this wave's chunks: wfirst, wfirst + STRIDE, ...; lookups run two of them ahead of the
+  // computation, so that their trip to memory is never waited for
+  const int mine = nchunks > wfirst ? (nchunks - wfirst + STRIDE - 1) / STRIDE : 0;
+  const int my_last = wfirst + STRIDE * (mine > 0 ? mine - 1 : 0);
+  auto nth = [&](int i) { return min(wfirst + STRIDE * i, my_last); };   // past the last: the last again, never used
+  Where wha = lookup(min(nth(0), last)), whb = lookup(min(nth(1), last));
 
   // ---- prologue: this row's q (GROUP heads), k and v (one kv head) from the projection
   const int width = (nh + 2 * nkv) * HD;
@@ -176,7 +185,7 @@ __global__ void __launch_bounds__(kFusWaves* kWave)
   const float scale2 = scale * 1.4426950408889634f;
 
   auto compute = [&](int c, const Chunk& ch) {
-    const int base = c * kFusChunk + wave * 64 + 8 * kq;   // this lane's first token of group 0
+    const int base = c * kFusChunk + wq * 64 + 8 * kq;   // this lane's first token of group 0
     float s[2][8];
     float mx = kFusNone;
 #pragma unroll
@@ -222,22 +231,24 @@ __global__ void __launch_bounds__(kFusWaves* kWave)
 
   // The chunk after the last repeats the last one, so that no load sits behind a branch; what it
   // brings is never used.
-  Chunk cha, chb;
-  request(wha, cha);
-  wha = lookup(min(2, last));
-  for (int c = 0; c < nchunks; c += 2) {
-    request(whb, chb);                 // chunk c + 1
-    whb = lookup(min(c + 3, last));
-    __builtin_amdgcn_sched_barrier(0);
-    compute(c, cha);
-    if (c + 1 >= nchunks) break;
-    request(wha, cha);                 // chunk c + 2
-    wha = lookup(min(c + 4, last));
-    __builtin_amdgcn_sched_barrier(0);
-    compute(c + 1, chb);
+  if (mine > 0) {
+    Chunk cha, chb;
+    request(wha, cha);
+    wha = lookup(nth(2));
+    for (int i = 0; i < mine; i += 2) {
+      request(whb, chb);                 // this wave's chunk i + 1
+      whb = lookup(nth(i + 3));
+      __builtin_amdgcn_sched_barrier(0);
+      compute(wfirst + STRIDE * i, cha);
+      if (i + 1 >= mine) break;
+      request(wha, cha);                 // chunk i + 2
+      wha = lookup(nth(i + 4));
+      __builtin_amdgcn_sched_barrier(0);
+      compute(wfirst + STRIDE * (i + 1), chb);
+    }
   }
 
-  // ---- the four waves' results, merged in wave order: out = sum_w e_w o_w / sum_w e_w l_w, e_w = 2^(m_w - m)
+  // ---- the waves' results, merged in wave order: out = sum_w e_w o_w / sum_w e_w l_w, e_w = 2^(m_w - m)
   l_run += __shfl_xor(l_run, 16, kWave);
   l_run += __shfl_xor(l_run, 32, kWave);
   if (kq == 0) { w_max[wave][n16] = m_run; w_sum[wave][n16] = l_run; }
@@ -267,9 +278,9 @@ int fused_kernel_info(int* out) {
   hipFuncAttributes a;
   int per_cu = 0;
   if (hipFuncGetAttributes(&a, reinterpret_cast<const void*>(&attention_decode_fused_kernel<HD, GROUP>)) != hipSuccess ||
-      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attention_decode_fused_kernel<HD, GROUP>, kFusWaves * kWave, 0) != hipSuccess)
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attention_decode_fused_kernel<HD, GROUP>, FusWaves<HD>::N * kWave, 0) != hipSuccess)
     return -1;
-  out[0] = a.numRegs; out[1] = static_cast<int>(a.sharedSizeBytes); out[2] = per_cu; out[3] = kFusWaves * kWave;
+  out[0] = a.numRegs; out[1] = static_cast<int>(a.sharedSizeBytes); out[2] = per_cu; out[3] = FusWaves<HD>::N * kWave;
   return 0;
 }
 
@@ -291,7 +302,7 @@ int dispatch_fused(int group, dim3 grid, hipStream_t s, const float* partials, i
                    float scale, uint16_t* out, int out_stride) {
 #define KVCM_FUSED(G)                                                                                                   \
   case G:                                                                                                               \
-    attention_decode_fused_kernel<HD, G><<<grid, kFusWaves * kWave, 0, s>>>(partials, S, pstride, qkv, qkv_stride,      \
+    attention_decode_fused_kernel<HD, G><<<grid, FusWaves<HD>::N * kWave, 0, s>>>(partials, S, pstride, qkv, qkv_stride,      \
                                                                            cos_sin, slots, kc, vc, tables, table_stride, \
                                                                            row_seq, ctx_lens, nh, nkv, B, scale, out,   \
                                                                            out_stride);                                 \
