@@ -74,7 +74,14 @@ def library_path():
     return _lib._name
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The current stream's handle (of device 0: the engine runs on one GPU).  The raw getter
+    costs a fraction of a microsecond; building a Stream object costs several, on every launch."""
+    if _raw_stream is not None:
+        return _raw_stream(0)
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -227,7 +234,11 @@ def add_residual(x, y):
 
 # Rows from which a bfloat16 product is handed to the library (hipBLASLt through torch.matmul); the
 # reference leaves every product to its vendor library.  0 = always use the kernels of this package.
-LIBRARY_GEMM_MIN_ROWS = 128
+# Below, the weight-streaming kernels of this package run: on the GPU the library wins from about
+# 128 rows on, but a call through torch costs the host about 15 us against 5 us for a kernel of
+# this package, and a step of a few hundred rows (88 products) is bound by the host: measured
+# end to end, a prompt portion is faster with this package's kernels up to about 300 rows.
+LIBRARY_GEMM_MIN_ROWS = 320
 
 
 def skinny_splits(M, N, K):
