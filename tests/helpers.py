@@ -25,13 +25,18 @@ TINY_C = dict(architectures=["LlamaForCausalLM"], vocab_size=331, hidden_size=80
 TINY_D = dict(architectures=["LlamaForCausalLM"], vocab_size=300, hidden_size=256, intermediate_size=320,
               num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
               max_position_embeddings=2048, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
-BLOCK_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
-WEIGHT_SEED = {"A": 0, "B": 2, "C": 5, "D": 7}
+# the other head size of the matrix-core kernels (128), a group of three query heads per KV head,
+# pages of 32, an odd vocabulary
+TINY_E = dict(architectures=["LlamaForCausalLM"], vocab_size=1001, hidden_size=192, intermediate_size=272,
+              num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=2, head_dim=128,
+              max_position_embeddings=512, rope_theta=50000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
+BLOCK_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 32}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+WEIGHT_SEED = {"A": 0, "B": 2, "C": 5, "D": 7, "E": 9}
 # factor on the q and k projections: chosen per width so that scores have a spread of a few units
 # in every configuration (they grow with hidden_size * sqrt(head_dim); a spread of tens would make
 # the 32-bit rounding of the scores themselves, amplified by exp, the largest error in the test)
-SHARPEN = {"A": 12.0, "B": 12.0, "C": 12.0, "D": 6.0}
+SHARPEN = {"A": 12.0, "B": 12.0, "C": 12.0, "D": 6.0, "E": 6.0}
 
 
 def make_model_dir(path, raw, seed, dtype, sharpen=12.0):

@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LENGTHS = {"A": [7, 70, 13, 45, 5, 100, 33, 64], "B": [1, 9, 17, 33, 40, 130, 2, 65], "C": [50, 3, 97, 16, 31],
-           "D": [300, 20, 1100, 65, 257]}
+           "D": [300, 20, 1100, 65, 257], "E": [40, 3, 300, 17, 129]}
 
 
 def tolerance(dtype, ref):
@@ -45,7 +45,7 @@ def setups(tmp_path_factory):
     return out
 
 
-CASES = [(n, d) for n in ("A", "B", "C", "D") for d in ("float32", "bfloat16")]
+CASES = [(n, d) for n in ("A", "B", "C", "D", "E") for d in ("float32", "bfloat16")]
 
 
 def check(setups, case, steps):
@@ -83,7 +83,7 @@ def test_mixed_batches_with_reused_pages(setups, case, seed):
     check(setups, case, steps)
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_32bit_logits_do_not_depend_on_the_cutting(setups, name):
     """In 32-bit every kernel computes a row by a fixed sequence of operations, so the cuttings
     agree to the last bit, not just within rounding."""
