@@ -226,3 +226,179 @@ def test_layer_list_may_repeat_a_layer_and_share_a_cache(tmp_path):
     b = rp.step({"step": 1, "entries": [{"id": "s", "tokens": toks[20:22], "want": [0, 1]}], "end": []})
     c = rp.step({"step": 2, "entries": [{"id": "s", "tokens": toks[22:], "want": list(range(15))}], "end": ["s"]})
     np.testing.assert_allclose(np.concatenate([a, b, c]), ref, atol=1e-4)
+
+
+# ------ full and windowed attention layers side by side, a routed feed-forward, another position encoding
+def _register_mixed():
+    from kvcm_amd.parts.base import FeedForward, LayerSpec, ModelSpec, ParamSpec, PartSpec, PositionEncoding
+    from kvcm_amd.registry import ARCHITECTURES, FEED_FORWARDS, POSITIONS, Architecture
+
+    if "toy_top1_experts" in FEED_FORWARDS:
+        return
+
+    @POSITIONS.register("toy_damped")
+    class Damped(PositionEncoding):
+        """q[.., d] and k[.., d] are multiplied by cos(position * base^(-d / head_dim)): absolute, not a
+        rotation, so the engine may not fuse it; v and the page write are left to the caller."""
+
+        def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None):
+            d = torch.arange(head_dim, dtype=torch.float32, device=qkv.device)
+            freq = torch.pow(torch.tensor(float(self.params["base"]), device=qkv.device), -d / head_dim)
+            factor = torch.cos(step.positions[:step.rows].float()[:, None] * freq[None, :])          # [rows, hd]
+            heads = num_heads + num_kv_heads
+            view = qkv[:step.rows, :heads * head_dim].view(step.rows, heads, head_dim)
+            view.copy_((view.float() * factor[:, None, :]).to(qkv.dtype))
+            return False
+
+    @FEED_FORWARDS.register("toy_top1_experts")
+    class Top1Experts(FeedForward):
+        """The expert with the largest router logit (32-bit) alone runs: w2[e] relu(w1[e] h)."""
+
+        def param_specs(self):
+            H, E, I, pre = self.ctx.hidden_size, self.params["experts"], self.params["inner"], self.prefix
+            return [ParamSpec("router", ((pre + "router.weight", (E, H)),)),
+                    ParamSpec("w1", ((pre + "experts.w1", (E * I, H)),)),
+                    ParamSpec("w2", ((pre + "experts.w2", (E * H, I)),))]
+
+        def forward(self, step, h):
+            H, E, I = self.ctx.hidden_size, self.params["experts"], self.params["inner"]
+            out = step.ws("ffn_out", (step.rows, H))
+            x = h[:step.rows].float()
+            choice = (x @ self.w["router"].float().T).argmax(-1)
+            w1, w2 = self.w["w1"].float().view(E, I, H), self.w["w2"].float().view(E, H, I)
+            mid = torch.relu(torch.einsum("rih,rh->ri", w1[choice], x))
+            out[:step.rows] = torch.einsum("rhi,ri->rh", w2[choice], mid).to(out.dtype)
+            return out
+
+    @dataclass(frozen=True)
+    class MixedConfig:
+        vocab_size: int
+        width: int
+        eps: float
+        layers: tuple          # per layer: dict(heads, kv_heads, head_dim, window, position, ffn)
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["vocab_size"], raw["width"], raw["eps"], tuple(raw["layers"]))
+
+        def to_dict(self):
+            return {"vocab_size": self.vocab_size, "width": self.width, "eps": self.eps, "layers": list(self.layers)}
+
+    def spec(cfg):
+        layers = []
+        for l, d in enumerate(cfg.layers):
+            pre = f"blocks.{l}."
+            attn = {"num_heads": d["heads"], "num_kv_heads": d["kv_heads"], "head_dim": d["head_dim"],
+                    "scale": d["head_dim"] ** -0.5, "window": d["window"], "position": PartSpec(*d["position"])}
+            layers.append(LayerSpec(f"b{l}", "prenorm_residual",
+                                    {"norm_mixer": PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, pre + "n1."),
+                                     "mixer": PartSpec("gqa_attention", attn, pre + "attn."),
+                                     "norm_ffn": PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, pre + "n2."),
+                                     "ffn": PartSpec(d["ffn"][0], d["ffn"][1], pre + "mlp.")}))
+        return ModelSpec("MixedWindowForCausalLM", cfg.width, cfg.vocab_size,
+                         PartSpec("token_embedding", {"vocab_size": cfg.vocab_size}, "emb."), tuple(layers),
+                         tuple(range(len(layers))), PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, "norm."),
+                         PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "tied": False}, "head."))
+
+    ARCHITECTURES.register("MixedWindowForCausalLM", Architecture("MixedWindowForCausalLM", MixedConfig, spec))
+
+
+_MIXED_LAYERS = [
+    dict(heads=4, kv_heads=2, head_dim=16, window=0, position=("rotary", {"theta": 10000.0, "dim": 16}),
+         ffn=("swiglu", {"intermediate_size": 80})),
+    dict(heads=4, kv_heads=2, head_dim=16, window=20, position=("rotary", {"theta": 300.0, "dim": 16}),
+         ffn=("toy_top1_experts", {"experts": 3, "inner": 24})),
+    dict(heads=3, kv_heads=1, head_dim=32, window=9, position=("toy_damped", {"base": 50.0}),
+         ffn=("swiglu", {"intermediate_size": 48})),
+    dict(heads=4, kv_heads=2, head_dim=16, window=0, position=("none", {}),
+         ffn=("toy_top1_experts", {"experts": 2, "inner": 40})),
+]
+
+
+def _mixed_plain_logits(raw, t, tokens):
+    n, pos = len(tokens), np.arange(len(tokens))
+    x = plain.embedding(t["emb.weight"], tokens)
+    for l, d in enumerate(raw["layers"]):
+        p, nh, nkv, hd = f"blocks.{l}.", d["heads"], d["kv_heads"], d["head_dim"]
+        h = plain.rms_norm(x, t[p + "n1.weight"], raw["eps"])
+        q = plain.linear(h, t[p + "attn.q_proj.weight"]).reshape(n, nh, hd)
+        k = plain.linear(h, t[p + "attn.k_proj.weight"]).reshape(n, nkv, hd)
+        v = plain.linear(h, t[p + "attn.v_proj.weight"]).reshape(n, nkv, hd)
+        kind, pp = d["position"]
+        if kind == "rotary":
+            q, k = plain.rotary(q, pos, pp["theta"]), plain.rotary(k, pos, pp["theta"])
+        elif kind == "toy_damped":
+            f = np.cos(pos[:, None] * np.power(pp["base"], -np.arange(hd) / hd)[None, :])
+            q, k = q * f[:, None, :], k * f[:, None, :]
+        a = plain.attention(q, k, v, pos, pos, hd ** -0.5, window=d["window"])
+        x = x + plain.linear(a.reshape(n, nh * hd), t[p + "attn.o_proj.weight"])
+        h = plain.rms_norm(x, t[p + "n2.weight"], raw["eps"])
+        if d["ffn"][0] == "swiglu":
+            gu = np.concatenate([plain.linear(h, t[p + "mlp.gate_proj.weight"]), plain.linear(h, t[p + "mlp.up_proj.weight"])], -1)
+            x = x + plain.linear(plain.swiglu(gu), t[p + "mlp.down_proj.weight"])
+        else:
+            E, I, H = d["ffn"][1]["experts"], d["ffn"][1]["inner"], raw["width"]
+            choice = np.argmax(h @ t[p + "mlp.router.weight"].T, -1)
+            w1, w2 = t[p + "mlp.experts.w1"].reshape(E, I, H), t[p + "mlp.experts.w2"].reshape(E, H, I)
+            y = np.stack([w2[e] @ np.maximum(w1[e] @ h[r], 0.0) for r, e in enumerate(choice)])
+            x = x + y
+    return plain.rms_norm(x, t["norm.weight"], raw["eps"]) @ t["head.weight"].T
+
+
+def test_full_and_windowed_layers_routed_ffn_and_another_position_encoding(tmp_path):
+    _register_mixed()
+    from kvcm_amd import Engine, EngineConfig
+    from kvcm_amd.engine.replay import TraceReplayer
+    from kvcm_amd.registry import ARCHITECTURES
+    from kvcm_amd.weights.random_init import write_model_dir
+
+    raw = dict(architectures=["MixedWindowForCausalLM"], vocab_size=131, width=56, eps=3e-6, layers=_MIXED_LAYERS)
+    cfg = ARCHITECTURES.get("MixedWindowForCausalLM").config_class.from_dict(raw)
+    d = write_model_dir(str(tmp_path / "mixed"), "MixedWindowForCausalLM", cfg, seed=21, dtype=torch.float32, std=0.25,
+                        norm_jitter=0.1)
+    t = plain.read_safetensors(os.path.join(d, "model.safetensors"))
+    rng = np.random.default_rng(5)
+    reqs = {"a": rng.integers(0, 131, size=90).tolist(), "b": rng.integers(0, 131, size=41).tolist(),
+            "c": rng.integers(0, 131, size=57).tolist()}
+    ref = {k: _mixed_plain_logits(raw, t, v) for k, v in reqs.items()}
+
+    # 12 pages of 16: a (6 pages) + b (3) + c (4) do not fit together, so c takes pages b gave back
+    rp = TraceReplayer(d, "float32", max_tokens=192)
+    kinds = [(g.kind, g.window) for g in rp.core.groups]
+    assert kinds == [("full", 0), ("window", 20), ("window", 9)]
+    assert [p.layers for p in rp.model.groups] == [["b0", "b3"], ["b1"], ["b2"]]
+    steps = [[("a", 0, 30), ("b", 0, 2)], [("a", 30, 33), ("b", 2, 41)], [("a", 33, 34), ("c", 0, 17)],
+             [("a", 34, 70), ("c", 17, 18)], [("c", 18, 57)], [("a", 70, 72)]] + [[("a", k, k + 1)] for k in range(72, 90)]
+    got = {k: [] for k in reqs}
+    for k, entries in enumerate(steps):
+        ended = [rid for rid, lo, hi in entries if hi == len(reqs[rid])]
+        out = rp.step({"step": k, "entries": [{"id": rid, "tokens": reqs[rid][lo:hi], "want": list(range(hi - lo))}
+                                              for rid, lo, hi in entries], "end": ended})
+        row = 0
+        for rid, lo, hi in entries:
+            got[rid].append(out[row:row + hi - lo])
+            row += hi - lo
+        if k == 3:
+            # a has 70 tokens: the next query (position 70) sees keys from 51 on with window 20, from 62 on with 9
+            sid = rp._ids[json.dumps("a")]
+            assert [p >= 0 for p in rp.core.seq_table(sid, 0)][:5] == [True] * 5
+            assert [p >= 0 for p in rp.core.seq_table(sid, 1)][:5] == [False, False, False, True, True]
+            assert [p >= 0 for p in rp.core.seq_table(sid, 2)][:5] == [False, False, False, True, True]
+            assert rp.core.blocks_in_use(1) < rp.core.blocks_in_use(0)
+    for rid in reqs:
+        err = np.abs(np.concatenate(got[rid]) - ref[rid]).max()
+        assert err < 1e-4, (rid, err)
+    assert all(rp.core.blocks_in_use(g) == 0 for g in range(3))
+
+    # through the scheduler, with few pages and prompts cut into portions
+    eng = Engine(d, EngineConfig(dtype="float32", block_size=16, num_blocks=9, max_seq_len=128, max_num_seqs=4,
+                                 max_batched_tokens=48, prefill_chunk=13, use_graphs=False))
+    prompts = [reqs["b"], reqs["c"][:30]]
+    outs = eng.generate(prompts, 24)
+    for p, g in zip(prompts, outs):
+        toks = list(p)
+        for k in range(24):
+            row = _mixed_plain_logits(raw, t, toks)[-1]
+            srt = np.sort(row)
+            assert g[k] == int(np.argmax(row)) or srt[-1] - srt[-2] < 1e-4, (k, g[k], int(np.argmax(row)))
+            toks.append(g[k])
