@@ -178,24 +178,56 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
 }
 
 // out = sum_p w_p o_p / sum_p w_p with w_p = sum_p * exp(max_p - max)   (paged_attention.cu:186-203)
+// One workgroup of 256 threads per (head, row): the maximum is found by all threads together,
+// then 256 / HD groups of HD threads each take every (256 / HD)-th partition and their sums meet
+// in LDS, so that a long context (hundreds of partitions) costs a few trips to memory, not one
+// per partition.
+constexpr int kMergeThreads = 256;
+
 template <int HD>
-__global__ void attention_decode_merge_kernel(const float* __restrict__ scratch, const int* __restrict__ ctx_lens,
-                                              uint16_t* __restrict__ out, int out_stride, int nh, int num_parts) {
-  const int head = blockIdx.x, row = blockIdx.y, d = threadIdx.x;
+__global__ void __launch_bounds__(kMergeThreads)
+attention_decode_merge_kernel(const float* __restrict__ scratch, const int* __restrict__ ctx_lens,
+                              uint16_t* __restrict__ out, int out_stride, int nh, int num_parts) {
+  constexpr int GROUPS = kMergeThreads / HD;
+  static_assert(GROUPS >= 1 && kMergeThreads % HD == 0, "head_dim must divide the merge workgroup");
+  __shared__ float wave_top[kMergeThreads / kWave];
+  __shared__ float sums[GROUPS][HD + 1];
+  const int head = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+  const int g = tid / HD, d = tid % HD;
   const int ctx = ctx_lens[row];
   uint16_t* o = out + size_t(row) * out_stride + size_t(head) * HD + d;
-  if (ctx <= 0) { *o = 0; return; }
+  if (ctx <= 0) {                                   // the whole workgroup leaves together
+    if (g == 0) *o = 0;
+    return;
+  }
   const int np = (ctx + kDecPart - 1) / kDecPart;
   const float* base = scratch + (size_t(row) * nh + head) * num_parts * (HD + 2);
   float m = -FLT_MAX;
-  for (int i = 0; i < np; ++i) m = fmaxf(m, base[i * (HD + 2) + HD]);
+  for (int i = tid; i < np; i += kMergeThreads) m = fmaxf(m, base[i * (HD + 2) + HD]);
+  m = wave_max(m);
+  if (tid % kWave == 0) wave_top[tid / kWave] = m;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kMergeThreads / kWave; ++w) m = fmaxf(m, wave_top[w]);
   float num = 0.f, den = 0.f;
-  for (int i = 0; i < np; ++i) {
-    const float w = base[i * (HD + 2) + HD + 1] * expf(base[i * (HD + 2) + HD] - m);
-    num = fmaf(w, base[i * (HD + 2) + d], num);
+#pragma unroll 4
+  for (int i = g; i < np; i += GROUPS) {
+    const float* part = base + size_t(i) * (HD + 2);
+    const float w = part[HD + 1] * expf(part[HD] - m);
+    num = fmaf(w, part[d], num);
     den += w;
   }
-  *o = float_to_bf16_bits(num / den);
+  sums[g][d] = num;
+  if (d == 0) sums[g][HD] = den;
+  __syncthreads();
+  if (g == 0) {
+#pragma unroll
+    for (int k = 1; k < GROUPS; ++k) {
+      num += sums[k][d];
+      den += sums[k][HD];
+    }
+    *o = float_to_bf16_bits(num / den);
+  }
 }
 
 template <int HD, int GROUP>
@@ -205,7 +237,7 @@ int launch_decode(const void* q, int q_stride, void* out, int out_stride, const 
   attention_decode_kernel<HD, GROUP><<<dim3(nkv, T, num_parts), kDecWaves * kWave, 0, s>>>(
       static_cast<const uint16_t*>(q), q_stride, static_cast<const uint16_t*>(kc), static_cast<const uint16_t*>(vc),
       tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale, num_parts, scratch);
-  attention_decode_merge_kernel<HD><<<dim3(nh, T), HD, 0, s>>>(scratch, ctx_lens, static_cast<uint16_t*>(out),
+  attention_decode_merge_kernel<HD><<<dim3(nh, T), kMergeThreads, 0, s>>>(scratch, ctx_lens, static_cast<uint16_t*>(out),
                                                                out_stride, nh, num_parts);
   return 0;
 }

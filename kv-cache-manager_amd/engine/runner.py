@@ -193,7 +193,7 @@ class ModelRunner:
     # The one-launch decode kernel walks a row's context chunk by chunk inside one workgroup:
     # right when contexts are moderate or there are enough rows to fill the chip; a few rows with
     # very long contexts are better cut into partitions that run in parallel.
-    FUSED_DECODE_MAX_CONTEXT = 4096
+    FUSED_DECODE_MAX_CONTEXT = 2048
     FUSED_DECODE_FULL_CHIP = 192
 
     def decode_attention_fused(self, step, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):

@@ -653,6 +653,34 @@ def test_partitioned_decode_attention(ops, nh, nkv, hd, B):
     np.testing.assert_allclose(_np(out).reshape(R, nh, hd), generic, atol=2 ** -6, rtol=0)   # v1 vs v2: a rounding apart
 
 
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (6, 2, 128)])
+def test_partitioned_decode_attention_many_partitions(ops, nh, nkv, hd):
+    """Twenty partitions and more: the merge takes them in groups; a key in a middle partition that
+    outweighs all others must come through alone, and plain rows must match the plain attention."""
+    rng = np.random.default_rng(41 + hd)
+    B, lens = 16, [5000, 2300, 257]
+    P = _paged_problem(rng, lens, nh, nkv, hd, B, all_rows=False)
+    far = 2600                                                # partition 10 of 20
+    P["Q"][0, 3] = 0.0
+    P["Q"][0, 3, 5] = 40.0
+    kvec = np.zeros(hd)
+    kvec[5] = 40.0
+    kvh = 3 // (nh // nkv)
+    P["Kl"][0][far, kvh] = kvec
+    P["Kc"][P["tables"][0, far // B], kvh, far % B] = kvec
+    ref = _ref_attention(P, nh, nkv, hd, scale=1.0 / math.sqrt(hd))
+    for bound in (5000, 8192):
+        out = torch.full((3, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+        scratch = torch.full((ops.attention_decode_scratch(3, nh, hd, bound),), float("nan"), dtype=torch.float32, device=DEV)
+        ops.attention_decode(_t(P["Q"].reshape(3, nh * hd), torch.bfloat16), out, _t(P["Kc"], torch.bfloat16),
+                             _vt(P["Vc"], torch.bfloat16), _t(P["tables"], torch.int32), P["max_blocks"],
+                             _t(P["row_seq"], torch.int32), _t(P["ctx"], torch.int32), nh, nkv, hd, 1.0 / math.sqrt(hd),
+                             bound, scratch)
+        got = _np(out).reshape(3, nh, hd)
+        np.testing.assert_allclose(got[0, 3], P["Vl"][0][far, kvh], atol=1e-2)
+        np.testing.assert_allclose(got, ref, atol=1e-2, rtol=0)
+
+
 def test_partitioned_decode_attention_padding_rows_and_far_key(ops):
     rng = np.random.default_rng(40)
     nh, nkv, hd, B = 8, 2, 64, 16
