@@ -20,6 +20,11 @@ class KVStorage:
                  dtype: torch.dtype, device):
         self.group, self.need = group, need
         self.num_layers, self.num_blocks, self.block_size = num_layers, num_blocks, block_size
+        per_layer = num_blocks * need.num_kv_heads * block_size * need.head_dim
+        if num_blocks * block_size >= 2 ** 31 or per_layer > 2 ** 35:
+            # slot numbers are 32-bit; the decode kernels keep offsets inside a layer's cache as 32 bits x 8 elements
+            raise ValueError(f"cache group {group}: {num_blocks} pages of {block_size} tokens are more than the kernels "
+                             f"address (at most 2^31 token slots and 2^35 elements of keys per layer)")
         self.data = torch.zeros(num_layers, 2, num_blocks, need.num_kv_heads, block_size, need.head_dim,
                                 dtype=dtype, device=device)
 

@@ -497,6 +497,7 @@ int kvcm_rope_table(const int* positions, const float* inv_freq, float* cos_sin,
 int kvcm_swiglu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  KVCM_REQUIRE(T <= 65535, "swiglu: too many rows for one launch (%d)", T);
   if (I % 8 == 0 && reinterpret_cast<uintptr_t>(gate_up) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
     const dim3 vgrid((I / 8 + 255) / 256, T);
     if (dtype == kF32) swiglu_vec_kernel<float><<<vgrid, 256, 0, s>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), I);

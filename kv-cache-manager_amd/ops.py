@@ -309,11 +309,15 @@ def gemm_swiglu(x, w_gate_up, out):
     return True
 
 
-def _check_caches(kcache, vcache, nkv, hd):
+def _check_caches(kcache, vcache, nkv, hd, packed_offsets=False):
     _need(kcache.dim() == 4 and kcache.is_contiguous() and kcache.shape[1] == nkv and kcache.shape[3] == hd,
           "key cache must be [pages, nkv, block_size, hd]")
     _need(vcache.dim() == 4 and vcache.is_contiguous() and tuple(vcache.shape) == (kcache.shape[0], nkv, hd, kcache.shape[2]),
           "value cache must be [pages, nkv, hd, block_size]")
+    _need(kcache.shape[0] * kcache.shape[2] < 2 ** 31, "a cache of 2^31 token slots or more does not fit 32-bit slot numbers")
+    # the decode kernels keep a token's offset inside one layer's cache as 32 bits in units of 8 elements
+    _need(not packed_offsets or kcache.numel() <= 2 ** 35,
+          "one layer's key cache beyond 2^35 elements (64 GiB of bfloat16) does not fit the decode kernels' page offsets")
 
 
 def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, nh, nkv, hd, scale, window=0,
@@ -364,7 +368,7 @@ def attention_decode(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_
     _rows2d(out, "out")
     T = q.shape[0] if rows is None else rows
     _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "attention_decode is bfloat16 only")
-    _check_caches(kcache, vcache, nkv, hd)
+    _check_caches(kcache, vcache, nkv, hd, packed_offsets=True)
     _need(scratch.dtype == torch.float32 and scratch.is_contiguous(), "scratch must be contiguous float32")
     _i32(row_seq, "row_seq", T)
     _i32(ctx_lens, "ctx_lens", T)
@@ -392,7 +396,7 @@ def attention_decode_fused(projection, out, kcache, vcache, tables, table_stride
     _rows2d(out, "out")
     width = (nh + 2 * nkv) * hd
     _need(out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "attention_decode_fused is bfloat16 only")
-    _check_caches(kcache, vcache, nkv, hd)
+    _check_caches(kcache, vcache, nkv, hd, packed_offsets=True)
     if partial:
         _need(projection.cols == width and projection.rows == T, "the partial sums are not [splits, rows, (nh + 2 nkv) * hd]")
     else:

@@ -450,3 +450,17 @@ def test_random_orders_with_groups_never_lose_a_page():
     for sid in list(live):
         m.release(sid)
     assert m.num_free_pages(0) == 96 and m.num_free_pages(1) == 48 and m.state_slots_free() == 8
+
+
+def test_storage_refuses_a_cache_beyond_the_kernels_addressing():
+    """Slot numbers are 32-bit and the decode kernels keep offsets inside a layer's cache in 32
+    bits (units of 8 elements): a pool beyond that is refused when it is made, not at its first step."""
+    import torch
+    from kvcm_amd.cache.storage import KVStorage
+    from kvcm_amd.parts.base import KVCacheNeed
+    ok = KVStorage(0, KVCacheNeed(8, 128), 2, 2 ** 21, 16, torch.bfloat16, "meta")       # 2^35 elements per layer
+    assert ok.k(1).shape == (2 ** 21, 8, 16, 128)
+    with pytest.raises(ValueError, match="more than the kernels address"):
+        KVStorage(0, KVCacheNeed(8, 128), 2, 2 ** 21 + 1, 16, torch.bfloat16, "meta")
+    with pytest.raises(ValueError, match="more than the kernels address"):
+        KVStorage(0, KVCacheNeed(1, 8), 1, 2 ** 27, 16, torch.bfloat16, "meta")             # 2^31 token slots
