@@ -49,7 +49,9 @@ constexpr int kPfWaveRows = 16 * kPfRT;
 constexpr int kPfRows = kPfWaveRows * kPfWaves;  // query rows per workgroup
 constexpr int kPfChunk = 64;                     // keys per trip
 constexpr int kPfPad = 8;                        // bfloat16 of padding per LDS row (keeps 16-byte alignment)
-constexpr int kPfSeg = 1024;                     // keys per segment
+constexpr int kPfSeg = 1024;                     // keys per segment: a multiple of this, chosen per launch
+constexpr int kPfSegMax = 16384;                 // at most (its page ids lie in LDS)
+constexpr long long kPfFill = 4096;              // workgroups a launch should have before segments grow
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   union { bf16x2_t v; uint32_t u; } r;
@@ -72,7 +74,7 @@ __global__ void __launch_bounds__(kPfThreads)
                              const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                              const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
                              const int* __restrict__ seq_start, int nh, int nkv, int B, int b_shift, float scale,
-                             int max_segs, float* __restrict__ scratch) {
+                             int seg_len, int max_segs, float* __restrict__ scratch) {
   constexpr int KSTEPS = HD / 32;                          // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;                              // 16-dim tiles of the output
   constexpr int PIECES = kPfChunk * HD / 8 / kPfThreads;   // 16-byte pieces of a chunk per thread (keys; as many of values)
@@ -95,10 +97,10 @@ __global__ void __launch_bounds__(kPfThreads)
   const uint16_t* kbase = kcache + kvh * head_elems;
   const uint16_t* vbase = vcache + kvh * head_elems;
   const int tile_last_pos = pos0 + min(block_first + kPfRows, n_rows) - 1;
-  const int seg_first = seg * kPfSeg;
+  const int seg_first = seg * seg_len;
   if (seg_first > tile_last_pos) return;
-  const int n_segs = tile_last_pos / kPfSeg + 1;
-  const int block_last_pos = min(tile_last_pos, seg_first + kPfSeg - 1);   // the last key this workgroup reads
+  const int n_segs = tile_last_pos / seg_len + 1;
+  const int block_last_pos = min(tile_last_pos, seg_first + seg_len - 1);   // the last key this workgroup reads
   const int first = block_first + wave * kPfWaveRows;   // first row of this wave inside the run
   const bool wave_on = first < n_rows;
   const int wave_last_pos = pos0 + min(first + kPfWaveRows, n_rows) - 1;
@@ -306,7 +308,7 @@ template <int HD>
 __global__ void __launch_bounds__(256)
     attention_prefill_merge_kernel(const float* __restrict__ scratch, uint16_t* __restrict__ out, int out_stride,
                                    const int* __restrict__ run_start, const int* __restrict__ seq_start, int nh,
-                                   int max_segs) {
+                                   int seg_len, int max_segs) {
   const int seq = blockIdx.y, head = blockIdx.z;
   const int row0 = run_start[seq], n_rows = run_start[seq + 1] - row0;
   constexpr int PER_ROW = HD / 4;
@@ -314,7 +316,7 @@ __global__ void __launch_bounds__(256)
   if (r >= n_rows) return;
   const int tile = r / kPfRows;
   const int tile_last_pos = seq_start[seq] + min((tile + 1) * kPfRows, n_rows) - 1;
-  const int n_segs = tile_last_pos / kPfSeg + 1;
+  const int n_segs = tile_last_pos / seg_len + 1;
   if (n_segs == 1) return;   // stored directly
   const float* base = scratch + (size_t(row0 + r) * nh + head) * max_segs * (HD + 4);
   float m = -FLT_MAX;
@@ -346,9 +348,22 @@ int kvcm_attention_prefill_supported(int nh, int nkv, int hd, int B) {
   return nkv > 0 && nh % nkv == 0 && (hd == 64 || hd == 128) && B >= 8 && (B & (B - 1)) == 0;
 }
 
-// Floats of scratch a launch needs: none while no row's context exceeds one segment of 1,024 keys.
-long long kvcm_attention_prefill_scratch(int T, int nh, int hd, int max_context) {
-  const long long segs = (max_context + kPfSeg - 1) / kPfSeg;
+// Keys per segment of a launch: 1,024 while that gives the chip fewer than kPfFill workgroups,
+// longer (in multiples of 1,024) when tiles x heads x sequences already fill it, since every segment
+// beyond the first costs a partial result per row and head in scratch.
+int kvcm_attention_prefill_segment(int max_run, int S, int nh, int max_context) {
+  if (max_run <= 0 || S <= 0 || nh <= 0 || max_context <= 0) return kPfSeg;
+  const long long base = static_cast<long long>((max_run + kPfRows - 1) / kPfRows) * nh * S;
+  const long long want = (kPfFill + base - 1) / base;
+  long long len = (max_context + want - 1) / want;
+  len = (len + kPfSeg - 1) / kPfSeg * kPfSeg;
+  return static_cast<int>(len < kPfSeg ? kPfSeg : len > kPfSegMax ? kPfSegMax : len);
+}
+
+// Floats of scratch a launch needs: none while no row's context exceeds one segment.
+long long kvcm_attention_prefill_scratch(int T, int nh, int hd, int max_context, int max_run, int S) {
+  const int seg_len = kvcm_attention_prefill_segment(max_run, S, nh, max_context);
+  const long long segs = (max_context + seg_len - 1) / seg_len;
   return segs <= 1 ? 0 : static_cast<long long>(T) * nh * segs * (hd + 4);
 }
 
@@ -370,8 +385,9 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(vcache) % 16 == 0, "attention_prefill: operands must be 16-byte aligned");
   KVCM_REQUIRE(out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0, "attention_prefill: output must be 8-byte aligned");
-  const int max_segs = (max_context + kPfSeg - 1) / kPfSeg;
-  const long long need = kvcm_attention_prefill_scratch(T, nh, hd, max_context);
+  const int seg_len = kvcm_attention_prefill_segment(max_run, S, nh, max_context);
+  const int max_segs = (max_context + seg_len - 1) / seg_len;
+  const long long need = kvcm_attention_prefill_scratch(T, nh, hd, max_context, max_run, S);
   KVCM_REQUIRE(need == 0 || (scratch && scratch_floats >= need && reinterpret_cast<uintptr_t>(scratch) % 16 == 0),
                "attention_prefill: scratch too small (%lld floats needed)", need);
   int b_shift = 0;
@@ -379,7 +395,7 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
   const long long units = static_cast<long long>((max_run + kPfRows - 1) / kPfRows) * max_segs * nh;
   KVCM_REQUIRE(units < (1ll << 31), "attention_prefill: too many workgroups");
   const dim3 grid(static_cast<unsigned>(units), S, 1);
-  const size_t page_bytes = sizeof(int) * size_t(kPfSeg / B + 2);   // the pages of one segment
+  const size_t page_bytes = sizeof(int) * size_t(seg_len / B + 2);   // the pages of one segment
   const uint16_t *qq = static_cast<const uint16_t*>(q), *kc = static_cast<const uint16_t*>(kcache),
                  *vc = static_cast<const uint16_t*>(vcache);
   const int merge_rows = 256 / (hd / 4);   // rows per workgroup of the merge
@@ -387,17 +403,17 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
   if (hd == 64) {
     attention_prefill_kernel<64><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
                                                              tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale,
-                                                             max_segs, scratch);
+                                                             seg_len, max_segs, scratch);
     if (max_segs > 1)
       attention_prefill_merge_kernel<64><<<mgrid, 256, 0, s>>>(scratch, static_cast<uint16_t*>(out), out_stride, run_start,
-                                                              seq_start, nh, max_segs);
+                                                              seq_start, nh, seg_len, max_segs);
   } else {
     attention_prefill_kernel<128><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
                                                               tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale,
-                                                              max_segs, scratch);
+                                                              seg_len, max_segs, scratch);
     if (max_segs > 1)
       attention_prefill_merge_kernel<128><<<mgrid, 256, 0, s>>>(scratch, static_cast<uint16_t*>(out), out_stride, run_start,
-                                                               seq_start, nh, max_segs);
+                                                               seq_start, nh, seg_len, max_segs);
   }
   return launch_status("attention_prefill");
 }

@@ -224,7 +224,7 @@ class ModelRunner:
             ops.rope_cache(projection[D:T], nh, nkv, hd, cos_sin=cos_sin[D:T] if cos_sin is not None else None,
                            slots=slots[D:T] if slots is not None else None, kcache=kcache, vcache=vcache,
                            block_size=kcache.shape[2], rows=T - D)
-        need = ops.attention_prefill_scratch(T, nh, hd, step.max_context)
+        need = ops.attention_prefill_scratch(T, nh, hd, step.max_context, step.max_run, S - D)
         scratch = self.workspace.flat("prefill_partials", need) if need else None
         ops.attention_prefill(projection, out, kcache, vcache, step.tables(g)[D * stride:], stride, step.run_start[D:],
                               step.seq_start[D:], S - D, step.max_run, nh, nkv, hd, scale, rows=T,
@@ -255,7 +255,7 @@ class ModelRunner:
         if (self.attn != "v1" and window == 0 and step.max_run > 1
                 and ops.attention_prefill_supported(nh, nkv, hd, q.dtype, kcache.shape[2])):
             # runs of consecutive positions: keys are read once per 64 query rows, on the matrix cores
-            need = ops.attention_prefill_scratch(step.real_rows, nh, hd, step.max_context)
+            need = ops.attention_prefill_scratch(step.real_rows, nh, hd, step.max_context, step.max_run, step.real_seqs)
             scratch = self.workspace.flat("prefill_partials", need) if need else None
             ops.attention_prefill(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.run_start,
                                   step.seq_start, step.real_seqs, step.max_run, nh, nkv, hd, scale,

@@ -53,7 +53,9 @@ def _declare(lib):
     fn("kvcm_attention_prefill_supported", i, i, i, i)
     fn("kvcm_attention_prefill", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, i, i, i, f, vp, C.c_longlong, vp)
     lib.kvcm_attention_prefill_scratch.restype = C.c_longlong
-    lib.kvcm_attention_prefill_scratch.argtypes = [i, i, i, i]
+    lib.kvcm_attention_prefill_scratch.argtypes = [i, i, i, i, i, i]
+    lib.kvcm_attention_prefill_segment.restype = i
+    lib.kvcm_attention_prefill_segment.argtypes = [i, i, i, i]
     lib.kvcm_attention_decode_scratch.restype = C.c_longlong
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
@@ -421,9 +423,15 @@ def attention_prefill_supported(nh, nkv, hd, dtype, block_size=16):
     return dtype == torch.bfloat16 and bool(lib().kvcm_attention_prefill_supported(nh, nkv, hd, block_size))
 
 
-def attention_prefill_scratch(rows, nh, hd, max_context):
-    """Floats of scratch ``attention_prefill`` needs (0 while contexts fit one segment of keys)."""
-    return int(lib().kvcm_attention_prefill_scratch(rows, nh, hd, max_context))
+def attention_prefill_scratch(rows, nh, hd, max_context, max_run, num_seqs):
+    """Floats of scratch ``attention_prefill`` needs for a launch of these sizes (0 while contexts
+    fit one segment of keys)."""
+    return int(lib().kvcm_attention_prefill_scratch(rows, nh, hd, max_context, max_run, num_seqs))
+
+
+def attention_prefill_segment(max_run, num_seqs, nh, max_context):
+    """Keys per segment that a launch of these sizes cuts contexts into."""
+    return int(lib().kvcm_attention_prefill_segment(max_run, num_seqs, nh, max_context))
 
 
 def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, seq_start, num_seqs, max_run, nh, nkv, hd,
@@ -432,13 +440,13 @@ def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, s
     run_start[s] .. run_start[s+1]-1, the first of them at position seq_start[s]; every row sees the
     sequence's cached tokens up to its own position.  The same result as ``attention``.
     ``rows``: rows in all; ``max_context``: a bound of every row's context length (default: what the
-    block tables can hold); contexts beyond 1,024 keys need ``scratch`` (float32,
+    block tables can hold); contexts beyond one segment of keys need ``scratch`` (float32,
     attention_prefill_scratch elements; allocated here when not given)."""
     _dev(q, out, kcache, vcache, tables, run_start, seq_start, scratch)
     T = q.shape[0] if rows is None else rows
     if max_context is None:
         max_context = table_stride * kcache.shape[2]
-    need = attention_prefill_scratch(T, nh, hd, max_context)
+    need = attention_prefill_scratch(T, nh, hd, max_context, max_run, num_seqs)
     if need and scratch is None:
         scratch = torch.empty(need, dtype=torch.float32, device=q.device)
     if scratch is not None:

@@ -894,3 +894,33 @@ def test_prefill_attention_three_segments_far_key(ops):
         c = P["ctx"][r]
         ref[k] = plain.attention(P["Q"][r:r + 1], P["Kl"][0][:c], P["Vl"][0][:c], [c - 1], np.arange(c), 1.0)[0]
     np.testing.assert_allclose(got[rows], ref, atol=1e-2, rtol=0)
+
+
+def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops):
+    """Many heads and sequences fill the chip without short segments: the launch then cuts contexts
+    into segments of 2,048 keys.  Rows on both sides of that cut, and a far key of the first segment."""
+    rng = np.random.default_rng(53)
+    nh, nkv, hd, B = 32, 4, 64, 16
+    runs = [(2000 + 13 * i, 300) for i in range(22)]
+    assert ops.attention_prefill_segment(300, len(runs), nh, max(s + n for s, n in runs)) == 2048
+    assert ops.attention_prefill_segment(300, 2, nh, 2600) == 1024 and ops.attention_prefill_segment(4096, 1, 32, 32768) == 8192
+    P = _paged_problem(rng, [s + n for s, n in runs], nh, nkv, hd, B, all_rows=False)
+    R = sum(n for _, n in runs)
+    Q = _bf16_grid(rng.normal(size=(R, nh, hd)))
+    far, seq, head = 40, 3, 9                                   # kv head 1
+    row_lo = sum(n for _, n in runs[:seq])
+    Q[row_lo + 100:row_lo + 300, head] = 0.0
+    Q[row_lo + 100:row_lo + 300, head, 3] = 30.0
+    kvec = np.zeros(hd)
+    kvec[3] = 30.0
+    P["Kl"][seq][far, 1] = kvec
+    P["Kc"][P["tables"][seq, far // B], 1, far % B] = kvec
+    P["Q"], P["R"] = Q, R
+    got = _run_prefill(ops, P, runs, nh, nkv, hd, scale=1.0)
+    np.testing.assert_allclose(got[row_lo + 100:row_lo + 300, head],
+                               np.broadcast_to(P["Vl"][seq][far, 1], (200, hd)), atol=2e-2)
+    for s, r in ((0, 0), (0, 47), (0, 48), (0, 299), (3, 5), (3, 6), (21, 0), (21, 299), (10, 128)):
+        pos = runs[s][0] + r                                   # the cut lies between positions 2047 and 2048
+        row = sum(n for _, n in runs[:s]) + r
+        ref = plain.attention(Q[row:row + 1], P["Kl"][s][:pos + 1], P["Vl"][s][:pos + 1], [pos], np.arange(pos + 1), 1.0)[0]
+        np.testing.assert_allclose(got[row], ref, atol=1e-2, rtol=0, err_msg=f"sequence {s} row {r}")
