@@ -8,6 +8,11 @@ reference launches every kernel of every step from the host, src/model/llama.cpp
 
 Padding rows have context length 0 and slot -1: they write no key, attend to nothing, and their
 sampled ids are dropped.  Nothing inside a graph clears memory or allocates.
+
+A captured launch must fit every step that replays it, so kernels that size their grid by the
+context are captured for a bound on it.  There is one graph per (bucket, context class): a step
+replays the graph of the smallest class that holds its longest context, so that an engine that
+allows long sequences still runs short ones with the launches made for short ones.
 """
 from typing import Dict, List
 
@@ -17,6 +22,7 @@ import torch
 from .runner import StepContext
 
 _BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256, 384, 512)
+_CONTEXT_CLASSES = (2048, 8192, 32768)       # and the longest context the engine allows
 
 
 class DecodeGraphs:
@@ -28,7 +34,8 @@ class DecodeGraphs:
         lim = self.runner.limits
         self.buckets = [b for b in _BUCKETS if b <= min(lim.max_seqs, lim.max_logit_rows, lim.max_tokens)]
         self.table_stride = lim.max_blocks_per_seq
-        self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
+        self.context_classes = [c for c in _CONTEXT_CLASSES if c < lim.max_context_len] + [lim.max_context_len]
+        self.graphs: Dict[tuple, torch.cuda.CUDAGraph] = {}      # (bucket, context class) -> graph
         self._views = {}      # bucket -> (device view, pinned view, ints) of the metadata a replay uploads
         self.enabled = bool(self.buckets)
 
@@ -45,19 +52,25 @@ class DecodeGraphs:
                 return b
         raise RuntimeError("no bucket")
 
-    def _forward(self, layout, bucket):
+    def _context_class(self, context: int) -> int:
+        for c in self.context_classes:
+            if context <= c:
+                return c
+        raise RuntimeError(f"a context of {context} tokens exceeds what the engine allows")
+
+    def _forward(self, layout, bucket, bound):
         """Only kernels of this package inside a graph: a library product may record nodes that
         clear memory, which do not replay reliably."""
         ops = self.runner.ops
         keep, ops.LIBRARY_GEMM_MIN_ROWS = ops.LIBRARY_GEMM_MIN_ROWS, 0
         try:
-            self._forward_inner(layout, bucket)
+            self._forward_inner(layout, bucket, bound)
         finally:
             ops.LIBRARY_GEMM_MIN_ROWS = keep
 
-    def _forward_inner(self, layout, bucket):
+    def _forward_inner(self, layout, bucket, bound):
         step = StepContext(self.runner, layout)
-        step.max_context_bound = self.runner.limits.max_context_len
+        step.max_context_bound = bound
         logits = self.runner.model.forward(step)
         # the sampling parameters lie in the metadata buffer (padding rows: temperature 0, dropped)
         t, seeds, ids, idx = step.sampling_params()
@@ -77,13 +90,14 @@ class DecodeGraphs:
         # no event: the synchronous download below ends after this upload, so the pinned buffer
         # is free again when the next step fills it
         runner._upload_pending = False
-        graph = self.graphs.get(bucket)
+        bound = self._context_class(layout.max_context)
+        graph = self.graphs.get((bucket, bound))
         if graph is None:
-            self._forward(layout, bucket)                 # eager once: creates every work buffer
+            self._forward(layout, bucket, bound)          # eager once: creates every work buffer
             torch.cuda.current_stream().synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                self._forward(layout, bucket)
-            self.graphs[bucket] = graph
+                self._forward(layout, bucket, bound)
+            self.graphs[(bucket, bound)] = graph
         graph.replay()
         return s.download(n)

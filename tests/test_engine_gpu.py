@@ -245,6 +245,24 @@ def test_graph_replays_at_matrix_core_sizes(tmp_path):
     assert eager.generate(prompts, 24) == got
 
 
+def test_graphs_follow_the_context_across_classes(tmp_path):
+    """An engine that allows 4,096 tokens captures decode graphs per context class: steps whose
+    longest context is at most 2,048 replay the one-launch attention, longer ones the partitioned
+    kernel sized for 4,096.  A request that crosses 2,048 while decoding changes class on the way."""
+    d = str(tmp_path / "m")
+    H.make_model_dir(d, H.TINY_D, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=H.SHARPEN["D"])
+    pm = plain.load_model_dir(d, plain.round_bf16)
+    prompts = _prompts(H.TINY_D, [2030, 100], seed=13)
+    kw = dict(dtype="bfloat16", num_blocks=300, max_seq_len=4096, max_batched_tokens=4096)
+    eng = _engine(d, use_graphs=True, **kw)
+    got = eng.generate(prompts, 40)
+    assert sorted(eng.decode_graphs.graphs) == [(2, 2048), (2, 4096)]
+    assert _engine(d, use_graphs=False, **kw).generate(prompts, 40) == got
+    for p, g in zip(prompts, got):
+        want, margins = pm.generate(p, 40)
+        assert _same_up_to_near_ties(g, want, margins, 5e-2), (len(p), g, want, margins)
+
+
 @pytest.mark.parametrize("attn", ["v1", "v2"])
 def test_attention_variants_at_matrix_core_sizes(tmp_path, attn):
     """--attn v1 (one-pass kernel everywhere) and v2 (partitions + merge for decode steps, after a
