@@ -7,7 +7,8 @@ implementation.  With --refs FILE the reference's KVPR file format is read inste
 (main_correct.cpp:34-59).  Checks, as in the reference:
   1. greedy output of each prompt alone equals the yardstick's; a divergence is tolerated only
      where the yardstick's two best logits are closer than --tie-margin;
-  2. teacher-forced top-1 agreement >= 98 %, top-5 logit error reported;
+  2. teacher-forced top-1 agreement >= 98 % (positions whose two best reference logits are closer
+     than 1 % of the logit scale are set aside as near-ties), top-5 logit error <= 2 % of that scale;
   3. paged and contiguous policies give identical tokens (scattered physical pages);
   4. all prompts in one batch give the tokens of the solo runs;
   5. prefix caching on: hits happen and outputs stay identical.
@@ -139,19 +140,33 @@ def main(argv=None):
             solo[policy] = outs
             if policy == "paged":
                 print("\n== paged: teacher-forced logits")
-                agree = total = 0
+                # A position whose two best reference logits are closer than 1 % of the logit scale
+                # is a near-tie: which of the two wins there says nothing (random weights give
+                # almost flat logits; with trained weights the scale is some 25 and this is half of
+                # the reference's --tie-margin).  Such positions are reported, not counted.
+                scale = max(float(np.abs(r["top_logits"]).max()) for r in refs)
+                near = 0.01 * scale
+                agree = total = ties = strict = 0
                 errs = []
                 for r in refs:
                     toks = r["prompt"] + r["greedy"][:steps - 1]
                     logits = eng.score(toks)
                     for k in range(steps):
                         row = logits[len(r["prompt"]) - 1 + k]
-                        agree += int(np.argmax(row)) == int(r["top_ids"][k][0])
-                        total += 1
+                        same = int(np.argmax(row)) == int(r["top_ids"][k][0])
+                        strict += same
                         errs.extend(np.abs(row[r["top_ids"][k]] - r["top_logits"][k]).tolist())
-                print(f"  top-1 agreement {agree}/{total} ({100.0 * agree / total:.2f}%), top-{topk} logit |err| "
-                      f"mean {np.mean(errs):.4f} max {np.max(errs):.4f}")
-                check(agree >= 0.98 * total, "teacher-forced top-1 agreement >= 98%")
+                        if topk > 1 and r["top_logits"][k][0] - r["top_logits"][k][1] < near:
+                            ties += 1
+                            continue
+                        agree += same
+                        total += 1
+                print(f"  top-1 agreement {strict}/{steps * len(refs)} over all positions; {agree}/{total} "
+                      f"({100.0 * agree / max(total, 1):.2f}%) over those whose two best reference logits differ by "
+                      f">= {near:.3f} ({ties} near-ties set aside)")
+                print(f"  top-{topk} logit |err| mean {np.mean(errs):.4f} max {np.max(errs):.4f} (logit scale {scale:.2f})")
+                check(agree >= 0.98 * total, "teacher-forced top-1 agreement >= 98% outside near-ties")
+                check(np.max(errs) <= 0.02 * scale, "teacher-forced top-k logit error <= 2% of the logit scale")
                 print(f"\n== paged: all {N} prompts in one batch")
                 outs = eng.generate([r["prompt"] for r in refs], steps)
                 same = sum(o == s for o, s in zip(outs, solo["paged"]))
