@@ -82,9 +82,13 @@ def main(argv=None):
                 slots = {k: (t.view(batch, mb)[:, (ctx - 1) // B] * B + (ctx - 1) % B).to(torch.int32).contiguous()
                          for k, t in tables.items()}
 
+                fneed = ops.attention_decode_fused_scratch(batch, heads, kvh, hd, ctx) if fused_ok else 0
+                fscratch = torch.zeros(fneed, dtype=torch.float32, device=dev) if fneed else None
+
                 def fused(tab):
                     ops.attention_decode_fused(QKV, O, K, V, tab, mb, rows, lens, heads, kvh, hd, 0.125,
-                                               slots=slots["paged" if tab is tables["paged"] else "contiguous"])
+                                               slots=slots["paged" if tab is tables["paged"] else "contiguous"],
+                                               max_context=ctx, scratch=fscratch)
 
                 for version, call in (("v1", v1), ("v2", v2), ("fused", fused)):
                     for layout in ("paged", "contiguous"):

@@ -187,7 +187,7 @@ constexpr int kMergeThreads = 256;
 template <int HD>
 __global__ void __launch_bounds__(kMergeThreads)
 attention_decode_merge_kernel(const float* __restrict__ scratch, const int* __restrict__ ctx_lens,
-                              uint16_t* __restrict__ out, int out_stride, int nh, int num_parts) {
+                              uint16_t* __restrict__ out, int out_stride, int nh, int num_parts, int part_tokens) {
   constexpr int GROUPS = kMergeThreads / HD;
   static_assert(GROUPS >= 1 && kMergeThreads % HD == 0, "head_dim must divide the merge workgroup");
   __shared__ float wave_top[kMergeThreads / kWave];
@@ -200,7 +200,7 @@ attention_decode_merge_kernel(const float* __restrict__ scratch, const int* __re
     if (g == 0) *o = 0;
     return;
   }
-  const int np = (ctx + kDecPart - 1) / kDecPart;
+  const int np = (ctx + part_tokens - 1) / part_tokens;
   const float* base = scratch + (size_t(row) * nh + head) * num_parts * (HD + 2);
   float m = -FLT_MAX;
   for (int i = tid; i < np; i += kMergeThreads) m = fmaxf(m, base[i * (HD + 2) + HD]);
@@ -238,7 +238,21 @@ int launch_decode(const void* q, int q_stride, void* out, int out_stride, const 
       static_cast<const uint16_t*>(q), q_stride, static_cast<const uint16_t*>(kc), static_cast<const uint16_t*>(vc),
       tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale, num_parts, scratch);
   attention_decode_merge_kernel<HD><<<dim3(nh, T), kMergeThreads, 0, s>>>(scratch, ctx_lens, static_cast<uint16_t*>(out),
-                                                               out_stride, nh, num_parts);
+                                                               out_stride, nh, num_parts, kDecPart);
+  return 0;
+}
+
+// The merge alone, for the one-launch decode kernel when it cuts long contexts into parts.
+int launch_decode_merge(const float* scratch, const int* ctx_lens, void* out, int out_stride, int nh, int T, int hd,
+                        int num_parts, int part_tokens, hipStream_t s) {
+  if (hd == 64)
+    attention_decode_merge_kernel<64><<<dim3(nh, T), kMergeThreads, 0, s>>>(scratch, ctx_lens, static_cast<uint16_t*>(out),
+                                                                   out_stride, nh, num_parts, part_tokens);
+  else if (hd == 128)
+    attention_decode_merge_kernel<128><<<dim3(nh, T), kMergeThreads, 0, s>>>(scratch, ctx_lens, static_cast<uint16_t*>(out),
+                                                                    out_stride, nh, num_parts, part_tokens);
+  else
+    return -1;
   return 0;
 }
 

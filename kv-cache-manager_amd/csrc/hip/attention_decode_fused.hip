@@ -21,11 +21,20 @@
 // 16-byte fragments.
 // Only steps whose rows all belong to different sequences may use it: a row's new key is written
 // by its own workgroup and read by nobody else.
+//
+// A few rows with long contexts cannot fill the chip with one workgroup per (kv head, row): then
+// the context is cut into parts of whole chunks (blockIdx.z), every part repeats the small
+// prologue for q, the part that holds the row's newest token stores it, each part leaves
+// (o / l, maximum, l) in scratch and the merge kernel of the partitioned attention adds them up.
 #include <cfloat>
 
 #include "common.h"
 
 namespace kvcm {
+
+// attention_decode.hip: out = sum_p w_p o_p / sum_p w_p over parts of part_tokens tokens
+int launch_decode_merge(const float* scratch, const int* ctx_lens, void* out, int out_stride, int nh, int T, int hd,
+                        int num_parts, int part_tokens, hipStream_t s);
 
 template <int HD> struct FusWaves { static constexpr int N = HD == 64 ? 8 : 4; };
 constexpr int kFusChunk = 256;
@@ -53,7 +62,8 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
                                   uint16_t* __restrict__ kcache, uint16_t* __restrict__ vcache,
                                   const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
                                   const int* __restrict__ ctx_lens, int nh, int nkv, int B, float scale,
-                                  uint16_t* __restrict__ out, int out_stride) {
+                                  uint16_t* __restrict__ out, int out_stride, int part_chunks, int num_parts,
+                                  float* __restrict__ scratch) {
   constexpr int KSTEPS = HD / 32;   // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;       // 16-dim tiles of the output
   constexpr int HALF = HD / 2;
@@ -68,15 +78,22 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   __shared__ __attribute__((aligned(16))) float red[kFusWaves][16][HD + 4];
   __shared__ float w_max[kFusWaves][16], w_sum[kFusWaves][16];
 
-  if (ctx <= 0) {   // a padding row: zeros, nothing read or stored
-    for (int i = threadIdx.x; i < GROUP * HD; i += kFusWaves * kWave)
-      out[size_t(row) * out_stride + size_t(kvh) * GROUP * HD + i] = 0;
+  if (ctx <= 0) {   // a padding row: zeros (from the merge when there are parts), nothing read or stored
+    if (num_parts == 1)
+      for (int i = threadIdx.x; i < GROUP * HD; i += kFusWaves * kWave)
+        out[size_t(row) * out_stride + size_t(kvh) * GROUP * HD + i] = 0;
     return;
   }
   const int* table = tables + size_t(row_seq[row]) * table_stride;
   const size_t head_elems = size_t(B) * HD, page_elems = head_elems * nkv;
   const int nchunks = (ctx + kFusChunk - 1) / kFusChunk;
   const int last = nchunks - 1;
+  // this workgroup's chunks: [c_lo, c_hi); the part that reaches the row's end stores its new token
+  const int c_lo = num_parts == 1 ? 0 : int(blockIdx.z) * part_chunks;
+  if (c_lo >= nchunks) return;   // the row ends before this part (the same for the whole workgroup)
+  const int c_hi = num_parts == 1 ? nchunks : min(nchunks, c_lo + part_chunks);
+  const int n_local = c_hi - c_lo;
+  const bool stores = c_hi == nchunks;
 
   // Where this wave's 64 tokens of chunk c live: lane l looks up token 64 w + l, the offset of its
   // key row and of its group of 8 value slots, both inside this kv head's part of the cache and in
@@ -95,9 +112,9 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   };
   // this wave's chunks: wfirst, wfirst + STRIDE, ...; lookups run two of them ahead of the
   // computation, so that their trip to memory is never waited for
-  const int mine = nchunks > wfirst ? (nchunks - wfirst + STRIDE - 1) / STRIDE : 0;
-  const int my_last = wfirst + STRIDE * (mine > 0 ? mine - 1 : 0);
-  auto nth = [&](int i) { return min(wfirst + STRIDE * i, my_last); };   // past the last: the last again, never used
+  const int mine = n_local > wfirst ? (n_local - wfirst + STRIDE - 1) / STRIDE : 0;
+  const int my_last = c_lo + wfirst + STRIDE * (mine > 0 ? mine - 1 : 0);
+  auto nth = [&](int i) { return min(c_lo + wfirst + STRIDE * i, my_last); };   // past the last: the last again, never used
   Where wha = lookup(min(nth(0), last)), whb = lookup(min(nth(1), last));
 
   // ---- prologue: this row's q (GROUP heads), k and v (one kv head) from the projection
@@ -121,6 +138,7 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   const int off = slot >= 0 ? slot % B : 0;
   for (int item = threadIdx.x; item < (GROUP + 2) * HALF; item += kFusWaves * kWave) {
     const int h = item / HALF, j = item % HALF;   // 0..GROUP-1: q heads, GROUP: k, GROUP+1: v
+    if (h >= GROUP && !(stores && slot >= 0)) continue;
     const int col = (h < GROUP ? (kvh * GROUP + h) * HD : h == GROUP ? (nh + kvh) * HD : (nh + nkv + kvh) * HD) + j;
     float a = value(col), b = value(col + HALF);
     if (h <= GROUP && cos_sin) {
@@ -239,12 +257,12 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
       request(whb, chb);                 // this wave's chunk i + 1
       whb = lookup(nth(i + 3));
       __builtin_amdgcn_sched_barrier(0);
-      compute(wfirst + STRIDE * i, cha);
+      compute(c_lo + wfirst + STRIDE * i, cha);
       if (i + 1 >= mine) break;
       request(wha, cha);                 // chunk i + 2
       wha = lookup(nth(i + 4));
       __builtin_amdgcn_sched_barrier(0);
-      compute(wfirst + STRIDE * (i + 1), chb);
+      compute(c_lo + wfirst + STRIDE * (i + 1), chb);
     }
   }
 
@@ -269,7 +287,16 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
       num = fmaf(e, red[w][g][d], num);
       den = fmaf(e, w_sum[w][g], den);
     }
-    out[size_t(row) * out_stride + size_t(kvh * GROUP + g) * HD + d] = float_to_bf16_bits(num / den);
+    if (num_parts == 1) {
+      out[size_t(row) * out_stride + size_t(kvh * GROUP + g) * HD + d] = float_to_bf16_bits(num / den);
+    } else {   // (o / l, maximum in natural units, l) of this part, as the merge kernel reads them
+      float* dst = scratch + ((size_t(row) * nh + kvh * GROUP + g) * num_parts + blockIdx.z) * (HD + 2);
+      dst[d] = num / den;
+      if (d == 0) {
+        dst[HD] = m * 0.6931471805599453f;
+        dst[HD + 1] = den;
+      }
+    }
   }
 }
 
@@ -299,13 +326,13 @@ template <int HD>
 int dispatch_fused(int group, dim3 grid, hipStream_t s, const float* partials, int S, size_t pstride, const uint16_t* qkv,
                    int qkv_stride, const float2* cos_sin, const int* slots, uint16_t* kc, uint16_t* vc,
                    const int* tables, int table_stride, const int* row_seq, const int* ctx_lens, int nh, int nkv, int B,
-                   float scale, uint16_t* out, int out_stride) {
+                   float scale, uint16_t* out, int out_stride, int part_chunks, int num_parts, float* scratch) {
 #define KVCM_FUSED(G)                                                                                                   \
   case G:                                                                                                               \
     attention_decode_fused_kernel<HD, G><<<grid, FusWaves<HD>::N * kWave, 0, s>>>(partials, S, pstride, qkv, qkv_stride,      \
                                                                            cos_sin, slots, kc, vc, tables, table_stride, \
                                                                            row_seq, ctx_lens, nh, nkv, B, scale, out,   \
-                                                                           out_stride);                                 \
+                                                                           out_stride, part_chunks, num_parts, scratch); \
     return 0
   switch (group) {
     KVCM_FUSED(1); KVCM_FUSED(2); KVCM_FUSED(3); KVCM_FUSED(4); KVCM_FUSED(5); KVCM_FUSED(6); KVCM_FUSED(7); KVCM_FUSED(8);
@@ -336,16 +363,45 @@ int kvcm_attention_decode_fused_info(int nh, int nkv, int hd, int* out) {
   return 0;
 }
 
+// How a launch for T rows with contexts of at most max_context cuts them: one workgroup per
+// (kv head, row) while that fills the chip or contexts are short; else parts of whole chunks, about
+// one workgroup per CU in all.  Returns the number of parts, *part_chunks chunks of 256 tokens each.
+constexpr int kFusSingleMax = 1024;   // contexts up to this always run as one part
+constexpr int kFusTargetWorkgroups = 256;
+static int fused_parts(int T, int nkv, int max_context, int* part_chunks) {
+  const int nchunks = max_context > 0 ? (max_context + kFusChunk - 1) / kFusChunk : 1;
+  long long parts = 1;
+  if (max_context > kFusSingleMax) {
+    const long long wgs = static_cast<long long>(T) * nkv;
+    parts = (kFusTargetWorkgroups + wgs - 1) / wgs;
+    if (parts > nchunks) parts = nchunks;
+    if (parts < 1) parts = 1;
+  }
+  int pc = static_cast<int>((nchunks + parts - 1) / parts);
+  const int n = (nchunks + pc - 1) / pc;
+  *part_chunks = n == 1 ? (1 << 20) : pc;
+  return n;
+}
+
+// Floats of scratch a launch of these sizes needs (0: contexts are not cut).
+long long kvcm_attention_decode_fused_scratch(int T, int nh, int nkv, int hd, int max_context) {
+  int pc;
+  const int parts = fused_parts(T, nkv, max_context, &pc);
+  return parts <= 1 ? 0 : static_cast<long long>(T) * nh * parts * (hd + 2);
+}
+
 // Rows of T different sequences.  The projection's result is either `partials` (split-K sums
 // [S][T][width], width = (nh + 2 nkv) * hd, added in split order) or, when partials is null, the
 // bfloat16 rows `qkv`.  cos_sin [T][hd/2] (cos, sin) rotates q and k by pairs (j, j + hd/2); null:
 // no rotation.  slots [T]: where the row's key and value go (page * B + offset; negative or a
 // null array: nothing is stored and the context is read as it is).  ctx_lens[t] includes the
-// row's own token.
+// row's own token.  max_context: an upper bound of every row's context length (0: unknown, contexts
+// are never cut into parts); scratch: kvcm_attention_decode_fused_scratch floats when that is not 0.
 int kvcm_attention_decode_fused(const float* partials, int S, const void* qkv, int qkv_stride, const float* cos_sin,
                                 const int* slots, void* kcache, void* vcache, const int* tables, int table_stride,
                                 const int* row_seq, const int* ctx_lens, int T, int nh, int nkv, int hd, int B,
-                                float scale, void* out, int out_stride, hipStream_t s) {
+                                float scale, void* out, int out_stride, int max_context, float* scratch,
+                                long long scratch_floats, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(kvcm_attention_decode_fused_supported(nh, nkv, hd, B),
                "attention_decode_fused: unsupported shape heads=%d kv_heads=%d head_dim=%d page=%d", nh, nkv, hd, B);
@@ -357,19 +413,26 @@ int kvcm_attention_decode_fused(const float* partials, int S, const void* qkv, i
                    reinterpret_cast<uintptr_t>(cos_sin) % 8 == 0,
                "attention_decode_fused: operands must be 16-byte aligned");
   const size_t pstride = size_t(T) * (nh + 2 * nkv) * hd;
-  const dim3 grid(nkv, T);
+  int part_chunks;
+  const int parts = fused_parts(T, nkv, max_context, &part_chunks);
+  KVCM_REQUIRE(parts <= 65535, "attention_decode_fused: context too long");
+  const long long need = kvcm_attention_decode_fused_scratch(T, nh, nkv, hd, max_context);
+  KVCM_REQUIRE(need == 0 || (scratch != nullptr && scratch_floats >= need),
+               "attention_decode_fused: scratch too small (%lld floats needed)", need);
+  const dim3 grid(nkv, T, parts);
   int rc;
   if (hd == 64)
     rc = dispatch_fused<64>(nh / nkv, grid, s, partials, S, pstride, static_cast<const uint16_t*>(qkv), qkv_stride,
                             reinterpret_cast<const float2*>(cos_sin), slots, static_cast<uint16_t*>(kcache),
                             static_cast<uint16_t*>(vcache), tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale,
-                            static_cast<uint16_t*>(out), out_stride);
+                            static_cast<uint16_t*>(out), out_stride, part_chunks, parts, scratch);
   else
     rc = dispatch_fused<128>(nh / nkv, grid, s, partials, S, pstride, static_cast<const uint16_t*>(qkv), qkv_stride,
                              reinterpret_cast<const float2*>(cos_sin), slots, static_cast<uint16_t*>(kcache),
                              static_cast<uint16_t*>(vcache), tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale,
-                             static_cast<uint16_t*>(out), out_stride);
+                             static_cast<uint16_t*>(out), out_stride, part_chunks, parts, scratch);
   KVCM_REQUIRE(rc == 0, "attention_decode_fused: no kernel for group size %d", nh / nkv);
+  if (parts > 1) launch_decode_merge(scratch, ctx_lens, out, out_stride, nh, T, hd, parts, part_chunks * kFusChunk, s);
   return launch_status("attention_decode_fused");
 }
 

@@ -22,7 +22,7 @@ import torch
 from .runner import StepContext
 
 _BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256, 384, 512)
-_CONTEXT_CLASSES = (2048, 8192, 32768)       # and the longest context the engine allows
+_CONTEXT_CLASSES = (1024, 2048, 8192, 32768)       # and the longest context the engine allows
 
 
 class DecodeGraphs:

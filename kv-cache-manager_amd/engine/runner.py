@@ -193,14 +193,23 @@ class ModelRunner:
     # The one-launch decode kernel walks a row's context chunk by chunk inside one workgroup:
     # right when contexts are moderate or there are enough rows to fill the chip; a few rows with
     # very long contexts are better cut into partitions that run in parallel.
-    FUSED_DECODE_MAX_CONTEXT = 2048
-    FUSED_DECODE_FULL_CHIP = 192
+    def _decode_parts_scratch(self, rows, nh, nkv, hd, bound):
+        """Scratch for the decode kernel when it cuts long contexts of few rows into parts; sized at
+        once for the worst case (rows x parts <= 256 / kv heads + rows), so that a captured graph's
+        pointer stays good."""
+        need = self.ops.attention_decode_fused_scratch(rows, nh, nkv, hd, bound)
+        if need == 0:
+            return None
+        most_rows = min(self.DECODE_ATTENTION_MAX_ROWS, self.limits.max_tokens)
+        worst = nh * (256 // nkv + 1 + most_rows) * (hd + 2)
+        return self.workspace.flat("decode_parts", max(need, worst))
 
     def decode_attention_fused(self, step, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):
-        """From the QKV projection to the attention output.  Decode-shaped steps: one launch.  Mixed
-        steps (the scheduler puts decoding requests first): the leading single-token runs take that
-        launch too, the rows after them are rotated and stored, then attended by the tiled kernel;
-        a single-token run there would otherwise cost a whole tile of its own."""
+        """From the QKV projection to the attention output.  Decode-shaped steps: one launch (and a
+        small merge when few rows have long contexts).  Mixed steps (the scheduler puts decoding
+        requests first): the leading single-token runs take that launch too, the rows after them
+        are rotated and stored, then attended by the tiled kernel; a single-token run there would
+        otherwise cost a whole tile of its own."""
         ops = self.ops
         if (self.attn != "auto" or window != 0 or out.dtype != torch.bfloat16
                 or not ops.attention_decode_fused_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
@@ -208,10 +217,10 @@ class ModelRunner:
         if step.max_run == 1:
             if step.rows > self.DECODE_ATTENTION_MAX_ROWS:
                 return False
-            if step.max_context_bound > self.FUSED_DECODE_MAX_CONTEXT and step.rows * nkv < self.FUSED_DECODE_FULL_CHIP:
-                return False
+            bound = step.max_context_bound
             ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
-                                       step.ctx_lens, nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=step.rows)
+                                       step.ctx_lens, nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=step.rows,
+                                       max_context=bound, scratch=self._decode_parts_scratch(step.rows, nh, nkv, hd, bound))
             return True
         D, T, S = step.leading_single_runs(), step.real_rows, step.real_seqs
         if (D == 0 or D > self.DECODE_ATTENTION_MAX_ROWS or isinstance(projection, ops.PartialSums)
@@ -219,7 +228,8 @@ class ModelRunner:
             return False
         stride = step.table_stride(g)
         ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), stride, step.row_seq, step.ctx_lens,
-                                   nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=D)
+                                   nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=D, max_context=step.max_context,
+                                   scratch=self._decode_parts_scratch(D, nh, nkv, hd, step.max_context))
         if (cos_sin is not None or slots is not None) and T > D:
             ops.rope_cache(projection[D:T], nh, nkv, hd, cos_sin=cos_sin[D:T] if cos_sin is not None else None,
                            slots=slots[D:T] if slots is not None else None, kcache=kcache, vcache=vcache,

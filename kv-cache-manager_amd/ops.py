@@ -35,7 +35,10 @@ def _declare(lib):
     fn("kvcm_rope_table", vp, vp, vp, i, i, vp)
     fn("kvcm_attention_decode_info", i, i, i, vp)
     fn("kvcm_attention_decode_fused_supported", i, i, i, i)
-    fn("kvcm_attention_decode_fused", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, vp, i, vp)
+    fn("kvcm_attention_decode_fused", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, vp, i, i, vp,
+       C.c_longlong, vp)
+    lib.kvcm_attention_decode_fused_scratch.restype = C.c_longlong
+    lib.kvcm_attention_decode_fused_scratch.argtypes = [i, i, i, i, i]
     fn("kvcm_attention_generic_info", i, vp)
     fn("kvcm_attention_decode_fused_info", i, i, i, vp)
     fn("kvcm_gemm_skinny_swiglu_supported", i, i, i)
@@ -385,12 +388,21 @@ def attention_decode_fused_supported(nh, nkv, hd, dtype, block_size=16):
     return dtype == torch.bfloat16 and bool(lib().kvcm_attention_decode_fused_supported(nh, nkv, hd, block_size))
 
 
+def attention_decode_fused_scratch(rows, nh, nkv, hd, max_context):
+    """Floats of scratch ``attention_decode_fused`` needs for these sizes (0: contexts are not cut
+    into parts: short ones, or rows x kv heads fill the chip)."""
+    return int(lib().kvcm_attention_decode_fused_scratch(rows, nh, nkv, hd, max_context))
+
+
 def attention_decode_fused(projection, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, nh, nkv, hd, scale,
-                           cos_sin=None, slots=None, rows=None):
-    """One launch from the QKV projection to the attention output for rows of different sequences
-    (bfloat16): ``projection`` is the fused [q | k | v] rows or their un-added split-K sums
-    (PartialSums); q and k are rotated by ``cos_sin`` [rows, hd/2, 2] (None: not rotated), k and v
-    stored at ``slots`` (None: nothing stored), and every row attends over its whole context."""
+                           cos_sin=None, slots=None, rows=None, max_context=0, scratch=None):
+    """From the QKV projection to the attention output for rows of different sequences (bfloat16):
+    ``projection`` is the fused [q | k | v] rows or their un-added split-K sums (PartialSums); q and
+    k are rotated by ``cos_sin`` [rows, hd/2, 2] (None: not rotated), k and v stored at ``slots``
+    (None: nothing stored), and every row attends over its whole context.  One launch; with
+    ``max_context`` (a bound of every row's context length) beyond 1,024 and few rows, contexts are
+    cut into parts that a second small launch merges, which needs ``scratch``
+    (attention_decode_fused_scratch floats; allocated here when not given)."""
     partial = isinstance(projection, PartialSums)
     rows_t = projection.out if partial else projection
     T = rows_t.shape[0] if rows is None else rows
@@ -412,11 +424,18 @@ def attention_decode_fused(projection, out, kcache, vcache, tables, table_stride
     _i32(ctx_lens, "ctx_lens", T)
     _i32(tables, "tables")
     _need(out.shape[0] >= T and out.shape[1] >= nh * hd, "out must be [rows, nh * hd]")
+    need = attention_decode_fused_scratch(T, nh, nkv, hd, int(max_context))
+    if need and scratch is None:
+        scratch = torch.empty(need, dtype=torch.float32, device=out.device)
+    if scratch is not None:
+        _dev(scratch)
+        _need(scratch.dtype == torch.float32 and scratch.is_contiguous(), "scratch must be contiguous float32")
     _check(lib().kvcm_attention_decode_fused(
         _ptr(projection.data) if partial else 0, projection.splits if partial else 0,
         0 if partial else _ptr(rows_t), 0 if partial else rows_t.stride(0), _ptr(cos_sin), _ptr(slots), _ptr(kcache),
         _ptr(vcache), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh, nkv, hd, kcache.shape[2],
-        float(scale), _ptr(out), out.stride(0), _stream()))
+        float(scale), _ptr(out), out.stride(0), int(max_context), _ptr(scratch),
+        scratch.numel() if scratch is not None else 0, _stream()))
 
 
 def attention_prefill_supported(nh, nkv, hd, dtype, block_size=16):

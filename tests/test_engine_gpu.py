@@ -246,9 +246,9 @@ def test_graph_replays_at_matrix_core_sizes(tmp_path):
 
 
 def test_graphs_follow_the_context_across_classes(tmp_path):
-    """An engine that allows 4,096 tokens captures decode graphs per context class: steps whose
-    longest context is at most 2,048 replay the one-launch attention, longer ones the partitioned
-    kernel sized for 4,096.  A request that crosses 2,048 while decoding changes class on the way."""
+    """An engine that allows 4,096 tokens captures decode graphs per context class (1,024, 2,048,
+    4,096): each replays the decode attention with the parts that suit its bound.  A request that
+    crosses 2,048 while decoding changes class on the way."""
     d = str(tmp_path / "m")
     H.make_model_dir(d, H.TINY_D, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=H.SHARPEN["D"])
     pm = plain.load_model_dir(d, plain.round_bf16)

@@ -765,6 +765,68 @@ def test_fused_decode_attention_equals_rope_write_attend(ops, nh, nkv, hd, B, so
     np.testing.assert_allclose(_np(got), _np(want), atol=2 ** -6, rtol=0)        # two kernels, a rounding apart
 
 
+@pytest.mark.parametrize("nh,nkv,hd,B", [(8, 2, 64, 16), (6, 2, 128, 32), (32, 4, 64, 16)])
+def test_fused_decode_attention_in_parts(ops, nh, nkv, hd, B):
+    """Few rows with long contexts: the launch cuts them into parts of whole chunks and a second
+    launch merges them.  The part that holds a row's newest token stores it; a padding row and a
+    row of one token ride along; one key in a middle part outweighs all others."""
+    rng = np.random.default_rng(nh * 7 + hd + B)
+    lens = [5000, 2300, 257, 1, 1025]
+    P = _paged_problem(rng, lens, nh, nkv, hd, B, all_rows=False)
+    R, W = P["R"], (nh + 2 * nkv) * hd
+    far, head = 2600, nh - 1
+    kvh = head // (nh // nkv)
+    pos = (P["ctx"] - 1).astype(np.int32)
+    k_new = _bf16_grid(rng.normal(size=(R, nkv, hd)))
+    v_new = _bf16_grid(rng.normal(size=(R, nkv, hd)))
+    rows = np.concatenate([P["Q"].reshape(R, -1), k_new.reshape(R, -1), v_new.reshape(R, -1)], axis=1)
+    rows = np.concatenate([rows, np.ones((1, W))])                              # + a padding row without context
+    slots = np.array([P["tables"][s, p // B] * B + p % B for s, p in zip(P["row_seq"], pos)] + [-1], dtype=np.int32)
+    row_seq = np.concatenate([P["row_seq"], [0]]).astype(np.int32)
+    ctx = np.concatenate([P["ctx"], [0]]).astype(np.int32)
+    inv = _t(_inv_freq(hd, 1e4), torch.float32)
+    table = torch.empty(R + 1, hd // 2, 2, device=DEV)
+    ops.rope_table(_t(np.concatenate([pos, [0]]), torch.int32), inv, table)
+    tables = _t(P["tables"], torch.int32)
+
+    def caches():
+        return _t(P["Kc"], torch.bfloat16), _vt(P["Vc"], torch.bfloat16)
+
+    kc1, vc1 = caches()
+    q1 = _t(rows, torch.bfloat16)
+    ops.rope_cache(q1, nh, nkv, hd, positions=_t(np.concatenate([pos, [0]]), torch.int32), inv_freq=inv,
+                   slots=_t(slots, torch.int32), kcache=kc1, vcache=vc1, block_size=B, cos_sin=table)
+    want = torch.zeros(R + 1, nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention(q1, want, kc1, vc1, tables, P["max_blocks"], _t(row_seq, torch.int32), _t(ctx, torch.int32), nh, nkv, hd,
+                  1.0 / math.sqrt(hd))
+    for bound in (5000, 8192):
+        need = ops.attention_decode_fused_scratch(R + 1, nh, nkv, hd, bound)
+        assert need > 0 and ops.attention_decode_fused_scratch(R + 1, nh, nkv, hd, 1024) == 0
+        kc2, vc2 = caches()
+        got = torch.full((R + 1, nh * hd), 5.0, dtype=torch.bfloat16, device=DEV)
+        scratch = torch.full((need,), float("nan"), dtype=torch.float32, device=DEV)
+        ops.attention_decode_fused(_t(rows, torch.bfloat16), got, kc2, vc2, tables, P["max_blocks"], _t(row_seq, torch.int32),
+                                   _t(ctx, torch.int32), nh, nkv, hd, 1.0 / math.sqrt(hd), cos_sin=table,
+                                   slots=_t(slots, torch.int32), max_context=bound, scratch=scratch)
+        assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)                  # the new tokens reached their pages, once
+        np.testing.assert_allclose(_np(got), _np(want), atol=2 ** -6, rtol=0)
+        assert not _np(got)[R].any()
+    with pytest.raises(ops.KernelError, match="scratch too small"):
+        ops.attention_decode_fused(_t(rows, torch.bfloat16), got, kc2, vc2, tables, P["max_blocks"], _t(row_seq, torch.int32),
+                                   _t(ctx, torch.int32), nh, nkv, hd, 1.0, max_context=5000, scratch=scratch[:100])
+    # an outstanding key in a middle part, no rotation, nothing stored
+    P["Q"][0, head] = 0.0
+    P["Q"][0, head, 5] = 40.0
+    kvec = np.zeros(hd)
+    kvec[5] = 40.0
+    P["Kc"][P["tables"][0, far // B], kvh, far % B] = kvec
+    rows[:R, :nh * hd] = P["Q"].reshape(R, -1)
+    kc3, vc3 = caches()
+    ops.attention_decode_fused(_t(rows, torch.bfloat16), got, kc3, vc3, tables, P["max_blocks"], _t(row_seq, torch.int32),
+                               _t(ctx, torch.int32), nh, nkv, hd, 1.0, max_context=5000)
+    np.testing.assert_allclose(_np(got)[0].reshape(nh, hd)[head], P["Vl"][0][far, kvh], atol=1e-2)
+
+
 def test_fused_decode_attention_against_plain_far_key_padding_and_no_store(ops):
     rng = np.random.default_rng(91)
     nh, nkv, hd, B = 8, 2, 64, 16

@@ -131,30 +131,32 @@ def test_long_decoding(setups, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoding_beyond_2048_tokens_of_context(setups, dtype):
-    """A few rows with a long context: in bfloat16 such decode steps take the kernel that cuts the
-    context into partitions (nine of them here) instead of the one-launch kernel."""
+    """A few rows with a long context: in bfloat16 the decode kernel cuts such contexts into parts
+    (nine chunks here) that a second launch merges."""
     from kvcm_amd.engine.replay import TraceReplayer
     d, _, ref_all, _ = setups[("D", dtype)]
-    toks = np.random.default_rng(77).integers(0, H.TINY_D["vocab_size"], size=2150).tolist()
+    raw = H.TINY_D
+    toks = np.random.default_rng(77).integers(0, raw["vocab_size"], size=2150).tolist()
     ref, _ = H.plain_logits(d, {"long": toks}, bf16=dtype == "bfloat16")
     rp = TraceReplayer(d, dtype, max_tokens=2176, block_size=H.BLOCK_SIZE["D"])
-    calls = []
+    ops, bounds = rp.runner.ops, []
+    inner = ops.attention_decode_fused
     if dtype == "bfloat16":
-        inner = rp.runner.ops.attention_decode
-        rp.runner.ops.attention_decode = lambda *a, **k: (calls.append(1), inner(*a, **k))[1]
+        ops.attention_decode_fused = lambda *a, **k: (bounds.append(k.get("max_context", 0)), inner(*a, **k))[1]
     try:
         steps = [{"step": 0, "entries": [{"id": "long", "tokens": toks[:2100], "want": [2099]}], "end": []}]
         steps += [{"step": i - 2099, "entries": [{"id": "long", "tokens": [toks[i]], "want": [0]}],
                    "end": ["long"] if i == 2149 else []} for i in range(2100, 2150)]
         got = H.replay(rp, steps, {"long": toks})
     finally:
-        if dtype == "bfloat16":
-            rp.runner.ops.attention_decode = inner
+        ops.attention_decode_fused = inner
     tol = tolerance(dtype, ref)
     err = np.abs(got["long"][2099:] - ref["long"][2099:]).max(axis=1)
     assert (err <= tol).all(), f"first wrong logits at position {2099 + int(np.nonzero(err > tol)[0][0])}: {err.max():.3g}"
     if dtype == "bfloat16":
-        assert len(calls) == 50 * H.TINY_D["num_hidden_layers"]
+        assert len(bounds) == 50 * raw["num_hidden_layers"] and min(bounds) > 2048
+        nh, nkv, hd = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
+        assert ops.attention_decode_fused_scratch(1, nh, nkv, hd, min(bounds)) > 0       # in parts
 
 
 def test_stale_pages_do_not_leak_into_a_new_request(setups):
