@@ -161,7 +161,8 @@ class HostCore:
         self.prefill_chunk = prefill_chunk
         self.prefix_caching = bool(prefix_caching) and policy == "paged"
         self._desc = np.zeros(self._lib.kvcm_batch_desc_len(self._h), dtype=np.int32)
-        self._summary = np.zeros(5, dtype=np.int64)
+        self._summary = np.zeros(6, dtype=np.int64)
+        self.plan_max_context = 0      # of the last schedule_summary: the longest context a row of the plan sees
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -281,6 +282,7 @@ class HostCore:
         decode_shaped) without building the plan's entries in Python (``plan()`` still gives them)."""
         check(self._lib.kvcm_sched_schedule_summary(self._h, float(now), self._summary.ctypes.data_as(i64p)))
         s = self._summary
+        self.plan_max_context = int(s[5])
         return int(s[0]), int(s[1]), int(s[2]), int(s[3]), bool(s[4])
 
     def update_sampled(self, ids, now=0.0):

@@ -342,18 +342,20 @@ int kvcm_sched_plan(void* c, int64_t* ids, int32_t* start, int32_t* count, int32
 }
 // Runs the scheduler and says what it planned without handing the entries over:
 // out = {entries, prompt tokens, decoding sequences, entries that sample, 1 if every entry is a
-// single token that samples (a decode-shaped step)}.
+// single token that samples (a decode-shaped step), the longest context a row of the step sees}.
 int kvcm_sched_schedule_summary(void* c, double now, int64_t* out) {
   return static_cast<int>(guarded([&]() -> int64_t {
     const auto& plan = static_cast<Core*>(c)->sched->schedule(now);
-    int64_t prefill = 0, decode = 0, sampling = 0, single = 1;
+    int64_t prefill = 0, decode = 0, sampling = 0, single = 1, longest = 0;
     for (const auto& p : plan) {
       if (p.is_prefill) prefill += p.num_tokens; else ++decode;
       if (p.samples) ++sampling;
       if (p.num_tokens != 1 || !p.samples) single = 0;
+      if (p.start + p.num_tokens > longest) longest = p.start + p.num_tokens;
     }
     out[0] = static_cast<int64_t>(plan.size()); out[1] = prefill; out[2] = decode; out[3] = sampling;
     out[4] = plan.empty() ? 0 : single;
+    out[5] = longest;   // the longest context any row of the step sees
     return static_cast<int64_t>(plan.size());
   }));
 }

@@ -34,6 +34,7 @@ class DecodeGraphs:
         lim = self.runner.limits
         self.buckets = [b for b in _BUCKETS if b <= min(lim.max_seqs, lim.max_logit_rows, lim.max_tokens)]
         self.table_stride = lim.max_blocks_per_seq
+        self.block_size = engine.config.block_size
         self.context_classes = [c for c in _CONTEXT_CLASSES if c < lim.max_context_len] + [lim.max_context_len]
         self.graphs: Dict[tuple, torch.cuda.CUDAGraph] = {}      # (bucket, context class) -> graph
         self._views = {}      # bucket -> (device view, pinned view, ints) of the metadata a replay uploads
@@ -80,8 +81,12 @@ class DecodeGraphs:
         """Runs the scheduler's current plan (n decode-shaped entries); returns the n sampled ids."""
         bucket = self._bucket(n)
         runner, s = self.runner, self.sampler
+        # the class also fixes how many page ids per sequence a replay uploads and reads
+        bound = self._context_class(max(self.core.plan_max_context, 1))
+        stride = min(self.table_stride, -(-bound // self.block_size))
         layout = self.core.build_batch_from_plan(runner.host_buffer(), pad_rows=bucket, pad_seqs=bucket,
-                                                 pad_logit_rows=bucket, table_stride=self.table_stride)
+                                                 pad_logit_rows=bucket, table_stride=stride)
+        assert layout.max_context <= bound
         runner._check(layout)
         views = self._views.get(bucket)
         if views is None or views[2] != layout.total:
@@ -90,7 +95,6 @@ class DecodeGraphs:
         # no event: the synchronous download below ends after this upload, so the pinned buffer
         # is free again when the next step fills it
         runner._upload_pending = False
-        bound = self._context_class(layout.max_context)
         graph = self.graphs.get((bucket, bound))
         if graph is None:
             self._forward(layout, bucket, bound)          # eager once: creates every work buffer

@@ -224,6 +224,7 @@ def test_schedule_summary_and_update_by_sampled_ids():
     core.sched_add(2, list(range(10, 19)), 3)    # 9 tokens: three portions, samples in the third
     n, prefill, decode, sampling, shaped = core.schedule_summary()
     assert (n, prefill, decode, sampling, shaped) == (2, 7, 0, 1, False)
+    assert core.plan_max_context == 4            # the longest context a row of this plan sees: tokens 0..3 of request 2
     assert [(p.id, p.count, p.samples) for p in core.plan()] == [(1, 3, True), (2, 4, False)]
     with pytest.raises(Exception):
         core.update_sampled([42, 43])            # one sampling entry, two ids
@@ -233,6 +234,7 @@ def test_schedule_summary_and_update_by_sampled_ids():
     core.update_sampled([43])
     n, prefill, decode, sampling, shaped = core.schedule_summary()
     assert (n, prefill, decode, sampling, shaped) == (2, 0, 2, 2, True)        # a prompt's last single token runs like a decode
+    assert core.plan_max_context == 9            # request 2's ninth token
     core.update_sampled([44, 50])
     n, prefill, decode, sampling, shaped = core.schedule_summary()
     assert (n, prefill, decode, sampling, shaped) == (1, 0, 1, 1, True)        # request 1 is done, request 2 decodes
