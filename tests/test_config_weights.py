@@ -286,3 +286,29 @@ def test_plain_model_cuts_agree_with_itself():
     full = pm.logits(toks)
     np.testing.assert_allclose(pm.logits(toks[:11]), full[:11], atol=1e-12)
     assert full.shape == (20, 256)
+
+
+def test_kvmodel_writes_a_folder_that_loads(tmp_path):
+    """bin/kvmodel as a program: a configuration and a seed give config.json + model.safetensors
+    whose tensors are the ones the architecture declares; the same seed gives the same bytes."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    tool = os.path.join(root, "bin", "kvmodel")
+    outs = []
+    for k in range(2):
+        d = tmp_path / f"m{k}"
+        p = subprocess.run([sys.executable, tool, "--out", str(d), "--sizes", "tiny-b", "--weights-seed", "3", "--dtype", "fp32"],
+                           capture_output=True, text=True, timeout=120)
+        assert p.returncode == 0, p.stderr
+        outs.append(open(d / "model.safetensors", "rb").read())
+    assert outs[0] == outs[1]
+    raw = json.load(open(tmp_path / "m0" / "config.json"))
+    assert raw["architectures"] == ["LlamaForCausalLM"] and raw["num_key_value_heads"] == 1 and raw["torch_dtype"] == "float32"
+    from kvcm_amd.config.model_config import LlamaConfig
+    from kvcm_amd.weights.random_init import expected_tensors
+    t = plain.read_safetensors(str(tmp_path / "m0" / "model.safetensors"))
+    want = expected_tensors("LlamaForCausalLM", LlamaConfig.from_dict(raw))
+    assert set(t) == set(want) and all(tuple(t[n].shape) == want[n][0] for n in t)
+    bad = subprocess.run([sys.executable, tool, "--out", str(tmp_path / "x"), "--sizes", "nope"], capture_output=True, text=True)
+    assert bad.returncode == 1 and "unknown --sizes" in bad.stderr
