@@ -223,9 +223,13 @@ class ModelRunner:
                                        max_context=bound, scratch=self._decode_parts_scratch(step.rows, nh, nkv, hd, bound))
             return True
         D, T, S = step.leading_single_runs(), step.real_rows, step.real_seqs
-        if (D == 0 or D > self.DECODE_ATTENTION_MAX_ROWS or isinstance(projection, ops.PartialSums)
+        if (D == 0 or D > self.DECODE_ATTENTION_MAX_ROWS
                 or not ops.attention_prefill_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
             return False
+        if isinstance(projection, ops.PartialSums):
+            # three consumers here (decode rows, rotation of the others, tiled attention): add the
+            # split sums up once instead of handing every single-token run to the tiled kernel
+            projection = projection.materialize()
         stride = step.table_stride(g)
         ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), stride, step.row_seq, step.ctx_lens,
                                    nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=D, max_context=step.max_context,

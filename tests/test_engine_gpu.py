@@ -90,16 +90,27 @@ def test_temperature_generation_config_b_chunked(models, dtype):
         assert again == done
 
 
-def test_mixed_steps_at_matrix_core_sizes(tmp_path):
+# wide enough (K = 1024) that the QKV product of a step of about a hundred rows splits K: the mixed
+# step then starts from partial sums
+TINY_WIDE = dict(architectures=["LlamaForCausalLM"], vocab_size=300, hidden_size=1024, intermediate_size=1408,
+                 num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2, head_dim=64,
+                 max_position_embeddings=2048, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+
+
+@pytest.mark.parametrize("raw,chunk,budget,sharpen", [(H.TINY_D, 160, 200, H.SHARPEN["D"]), (TINY_WIDE, 100, 110, 3.0)],
+                         ids=["narrow", "wide_split_k"])
+def test_mixed_steps_at_matrix_core_sizes(tmp_path, raw, chunk, budget, sharpen):
     """head_dim 64, bfloat16: decoding requests (the scheduler puts them first) take the one-launch
     decode kernel inside steps that also carry long prompt portions for the tiled kernel; graphs
     replay the pure decode steps.  Greedy tokens must be those of the plain implementation."""
     d = str(tmp_path / "m")
-    H.make_model_dir(d, H.TINY_D, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=H.SHARPEN["D"])
+    H.make_model_dir(d, raw, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=sharpen)
     pm = plain.load_model_dir(d, plain.round_bf16)
-    prompts = _prompts(H.TINY_D, [40, 12, 700, 90, 1200, 25], seed=9)
-    eng = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, prefill_chunk=160, max_batched_tokens=200)
+    prompts = _prompts(raw, [40, 12, 700, 90, 1200, 25], seed=9)
+    eng = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, prefill_chunk=chunk, max_batched_tokens=budget)
     ids = [eng.add_request(p, 10) for p in prompts]
+    qkv_width = (raw["num_attention_heads"] + 2 * raw["num_key_value_heads"]) * raw["head_dim"]
+    split_seen = False
     # which attention kernels the steps take (a silent fall back to the general kernel would pass the comparison)
     ops, calls = eng.runner.ops, {"fused": 0, "fused_in_mixed": 0, "tiled": 0, "general": 0}
     real = (ops.attention_decode_fused, ops.attention_prefill, ops.attention)
@@ -122,8 +133,11 @@ def test_mixed_steps_at_matrix_core_sizes(tmp_path):
         while not eng.idle():
             before = dict(calls)
             info = eng.step()
-            if info.decode_seqs > 0 and info.prefill_tokens >= 100:
+            # (a plan is in admission order: where an older request still runs its prompt while a
+            # younger one decodes, no decode row leads and the tiled kernel takes them all)
+            if info.decode_seqs > 0 and info.prefill_tokens >= chunk - 60 and eng.runner.last_step.leading_single_runs() > 0:
                 mixed_big += 1
+                split_seen |= ops.skinny_splits(info.rows, qkv_width, raw["hidden_size"]) > 1
                 calls["fused_in_mixed"] += calls["fused"] > before["fused"] and calls["tiled"] > before["tiled"]
             for f in eng.take_finished():
                 done[f.id] = f.generated
@@ -131,6 +145,7 @@ def test_mixed_steps_at_matrix_core_sizes(tmp_path):
         ops.attention_decode_fused, ops.attention_prefill, ops.attention = real
     assert mixed_big > 3, "no step mixed decoding requests with a long prompt portion"
     assert calls["fused_in_mixed"] == mixed_big and calls["general"] == 0, calls
+    assert split_seen == (raw is TINY_WIDE)
     for rid, p in zip(ids, prompts):
         want, margins = pm.generate(p, 10)
         assert _same_up_to_near_ties(done[rid], want, margins, 5e-2), (rid, done[rid], want, margins)
