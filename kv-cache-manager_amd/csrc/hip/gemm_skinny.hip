@@ -326,13 +326,16 @@ extern "C" {
 int kvcm_gemm_skinny_splits(int M, int N, int K) {
   if (M <= 0 || N % 16 != 0 || K % kUnit != 0 || N <= 0 || K <= 0) return 0;
   if (shares_rows(M, N)) {
-    const int groups = (N / 64) * row_blocks(M), units = K / kUnit;
-    if (groups >= 256) return 1;
-    int S = (512 + groups - 1) / groups;       // aim at two workgroups per CU ...
-    if (S > units / 4) S = units / 4;          // ... of at least four units each ...
-    if (S > K / (4 * M)) S = K / (4 * M);      // ... and partial sums (S*M*N floats) that stay below the weights' bytes
-    if (S > 8) S = 8;
-    return S < 1 ? 1 : S;
+    // Measured over the projections of three model sizes at 32, 64 and 128 rows: powers of two
+    // only (a slice then is a whole number of trips), four slices, eight where there are few
+    // column groups; each slice at least one trip of four units, and partial sums (S*M*N floats)
+    // that stay below the weights' bytes.
+    const int cols = N / 64, units = K / kUnit;
+    if (cols * row_blocks(M) >= 256) return 1;
+    int S = cols <= 32 ? 8 : 4;
+    const int cap = units / 4 < K / (4 * M) ? units / 4 : K / (4 * M);
+    while (S > 1 && S > cap) S >>= 1;
+    return S;
   }
   if (M > 64) return 0;
   const int tiles = N / 16, units = K / kUnit;
