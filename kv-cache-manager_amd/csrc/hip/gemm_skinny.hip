@@ -339,10 +339,9 @@ int kvcm_gemm_skinny_splits(int M, int N, int K) {
   }
   if (M > 64) return 0;
   const int tiles = N / 16, units = K / kUnit;
-  int S = (640 + tiles - 1) / tiles;           // aim at >= 640 workgroups (2.5 per CU)
-  if (S > units / 2) S = units / 2;            // at least two units per split ...
-  if (S < 1) S = 1;
-  if (S > 16) S = 16;
+  int S = (640 + tiles - 1) / tiles;           // aim at >= 640 workgroups (2.5 per CU) ...
+  if (S >= 5) S = 8;                           // ... five to seven slices lose to eight in whole decode steps (measured)
+  while (S > 1 && S > units / 2) --S;          // at least two units per slice
   return S;
 }
 
