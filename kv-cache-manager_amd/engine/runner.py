@@ -54,12 +54,10 @@ class Workspace:
         when that shape is not split.  Sized once for the most rows the split kernel takes."""
         key = ("scratch", name, n, k)
         if key not in self.buffers:
-            # the number of splits changes with the rows: room for the worst of the row counts at
-            # which it can change
+            # the number of splits changes with the rows: room for the worst row count
             need = 0
             if self.ops is not None:
-                for m in (1, 16, 17, 32, 64, 65, 128, 129, 256, 257, 512):
-                    m = min(m, self.limits.max_tokens)
+                for m in range(1, min(512, self.limits.max_tokens) + 1):
                     splits = self.ops.skinny_splits(m, n, k)
                     if splits > 1:
                         need = max(need, splits * m * n)
