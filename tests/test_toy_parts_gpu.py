@@ -402,3 +402,112 @@ def test_full_and_windowed_layers_routed_ffn_and_another_position_encoding(tmp_p
             srt = np.sort(row)
             assert g[k] == int(np.argmax(row)) or srt[-1] - srt[-2] < 1e-4, (k, g[k], int(np.argmax(row)))
             toks.append(g[k])
+
+
+# ------------------------------------------- another norm and another arrangement of a block
+def test_toy_norm_and_parallel_block_arrangement(tmp_path):
+    """A norm with mean removal and a bias, and a block that feeds one normed input to mixer and
+    feed-forward side by side (x += mixer(n(x)) + ffn(n(x))), both defined here: the norm keeps the
+    contract of ``Norm.forward`` (pending addition, row gather), the block that of ``Block.forward``."""
+    from kvcm_amd.engine.replay import TraceReplayer
+    from kvcm_amd.parts.base import Block, LayerSpec, ModelSpec, Norm, ParamSpec, PartSpec
+    from kvcm_amd.registry import ARCHITECTURES, BLOCKS, NORMS, Architecture
+    from kvcm_amd.weights.random_init import write_model_dir
+
+    if "toy_layernorm" not in NORMS:
+        @NORMS.register("toy_layernorm")
+        class ToyLayerNorm(Norm):
+            def param_specs(self):
+                n = self.params["size"]
+                return [ParamSpec("weight", ((self.prefix + "weight", (n,)),), role="vector"),
+                        ParamSpec("bias", ((self.prefix + "bias", (n,)),), role="vector")]
+
+            def forward(self, x, out, add=None, rows=None):
+                if add is not None:
+                    add = add.materialize() if hasattr(add, "materialize") else add
+                    if rows is None:
+                        x += add.float()
+                        v = x
+                    else:
+                        v = x[rows.long()] + add[rows.long()].float()
+                else:
+                    v = x if rows is None else x[rows.long()]
+                mu = v.mean(-1, keepdim=True)
+                var = ((v - mu) ** 2).mean(-1, keepdim=True)
+                y = (v - mu) / torch.sqrt(var + self.params["eps"]) * self.w["weight"].float() + self.w["bias"].float()
+                out[:v.shape[0]] = y.to(out.dtype)
+                return out
+
+        @BLOCKS.register("toy_parallel_residual")
+        class ParallelResidual(Block):
+            def forward(self, step, x, pending):
+                h = step.ws("normed", (step.rows, x.shape[1]))
+                self.parts["norm"].forward(x, h, add=pending)                 # adds what the block before left
+                a = self.parts["mixer"].forward(step, h)
+                a = a.materialize() if hasattr(a, "materialize") else a
+                f = self.parts["ffn"].forward(step, h)
+                f = f.materialize() if hasattr(f, "materialize") else f
+                both = step.ws("both", (step.rows, x.shape[1]), torch.float32)
+                both.copy_(a.float() + f.float())
+                return both
+
+    @dataclass(frozen=True)
+    class Cfg:
+        vocab_size: int
+        width: int
+        heads: int
+        head_dim: int
+        inner: int
+        depth: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("vocab_size", "width", "heads", "head_dim", "inner", "depth", "eps")})
+
+        def to_dict(self):
+            return asdict(self)
+
+    def spec(cfg):
+        def norm(prefix):
+            return PartSpec("toy_layernorm", {"size": cfg.width, "eps": cfg.eps}, prefix)
+        attn = {"num_heads": cfg.heads, "num_kv_heads": cfg.heads, "head_dim": cfg.head_dim, "scale": cfg.head_dim ** -0.5,
+                "window": 0, "position": PartSpec("rotary", {"theta": 1000.0, "dim": cfg.head_dim})}
+        layers = tuple(LayerSpec(f"p{l}", "toy_parallel_residual",
+                                 {"norm": norm(f"h.{l}.ln."), "mixer": PartSpec("gqa_attention", attn, f"h.{l}.attn."),
+                                  "ffn": PartSpec("swiglu", {"intermediate_size": cfg.inner}, f"h.{l}.mlp.")})
+                       for l in range(cfg.depth))
+        return ModelSpec("ToyParallelForCausalLM", cfg.width, cfg.vocab_size,
+                         PartSpec("token_embedding", {"vocab_size": cfg.vocab_size}, "wte."), layers, tuple(range(cfg.depth)),
+                         norm("ln_f."), PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "tied": True}, "head."))
+
+    ARCHITECTURES.register("ToyParallelForCausalLM", Architecture("ToyParallelForCausalLM", Cfg, spec))
+    raw = dict(architectures=["ToyParallelForCausalLM"], vocab_size=77, width=40, heads=2, head_dim=16, inner=72, depth=2, eps=2e-5)
+    cfg = Cfg.from_dict(raw)
+    d = write_model_dir(str(tmp_path / "par"), "ToyParallelForCausalLM", cfg, seed=13, dtype=torch.float32, std=0.2, norm_jitter=0.2)
+    t = plain.read_safetensors(os.path.join(d, "model.safetensors"))
+    toks = np.random.default_rng(2).integers(0, 77, size=41).tolist()
+
+    def ln(v, pre):
+        mu = v.mean(-1, keepdims=True)
+        var = ((v - mu) ** 2).mean(-1, keepdims=True)
+        return (v - mu) / np.sqrt(var + raw["eps"]) * t[pre + "weight"] + t[pre + "bias"]
+
+    n, pos = len(toks), np.arange(len(toks))
+    x = plain.embedding(t["wte.weight"], toks)
+    for l in range(2):
+        p = f"h.{l}."
+        h = ln(x, p + "ln.")
+        q = plain.rotary(plain.linear(h, t[p + "attn.q_proj.weight"]).reshape(n, 2, 16), pos, 1000.0)
+        k = plain.rotary(plain.linear(h, t[p + "attn.k_proj.weight"]).reshape(n, 2, 16), pos, 1000.0)
+        v = plain.linear(h, t[p + "attn.v_proj.weight"]).reshape(n, 2, 16)
+        a = plain.linear(plain.attention(q, k, v, pos, pos, 0.25).reshape(n, 32), t[p + "attn.o_proj.weight"])
+        gu = np.concatenate([plain.linear(h, t[p + "mlp.gate_proj.weight"]), plain.linear(h, t[p + "mlp.up_proj.weight"])], -1)
+        x = x + a + plain.linear(plain.swiglu(gu), t[p + "mlp.down_proj.weight"])
+    ref = ln(x, "ln_f.") @ t["wte.weight"].T
+
+    rp = TraceReplayer(d, "float32", max_tokens=64)
+    a = rp.step({"step": 0, "entries": [{"id": "s", "tokens": toks[:17], "want": list(range(17))}], "end": []})
+    b = rp.step({"step": 1, "entries": [{"id": "s", "tokens": toks[17:19], "want": [0, 1]}], "end": []})
+    c = rp.step({"step": 2, "entries": [{"id": "s", "tokens": toks[19:], "want": list(range(22))}], "end": ["s"]})
+    np.testing.assert_allclose(np.concatenate([a, b, c]), ref, atol=2e-4)
