@@ -107,12 +107,19 @@ def main(argv=None):
     print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
     rp = TraceReplayer(args.model, args.dtype, args.max_tokens, args.block_size, attn=args.attn)
     print("[trace_run] ready", file=sys.stderr, flush=True)
-    for line in sys.stdin:
+    for number, line in enumerate(sys.stdin, 1):
         line = line.strip()
         if not line:
             continue
-        record = json.loads(line)
-        logits = rp.step(record)
+        try:
+            record = json.loads(line)
+            if not isinstance(record, dict) or "step" not in record:
+                raise ReplayError('a step is a JSON object {"step": .., "entries": [..], "end": [..]}')
+            logits = rp.step(record)
+        except (ReplayError, ValueError, KeyError, TypeError) as e:      # what the input can get wrong: one line, exit 1
+            what = f"missing key {e}" if isinstance(e, KeyError) else str(e)
+            print(f"trace_run: input line {number}: {what}", file=sys.stderr, flush=True)
+            return 1
         if logits is not None:
             np.ascontiguousarray(logits, dtype="<f4").tofile(os.path.join(args.out, f"{record['step']}.f32"))
         print(f"done {record['step']}", flush=True)

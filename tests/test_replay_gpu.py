@@ -214,3 +214,20 @@ def test_trace_run_program(setups, dtype, tmp_path):
             pos[e["id"]] += len(e["tokens"])
     bad = H.first_difference(got, {rid: ref[rid] for rid in sub}, tolerance(dtype, ref))
     assert bad is None, f"first wrong logits at request {bad[0]} position {bad[1]}: error {bad[2]:.3g}"
+
+
+def test_trace_run_reports_bad_input_and_stops(setups, tmp_path):
+    """A step the program cannot run ends it with one line on stderr and exit code 1; the steps
+    before it are done."""
+    d, reqs, ref, _ = setups[("A", "float32")]
+    good = {"step": 0, "entries": [{"id": "a", "tokens": reqs["r0"], "want": [0]}], "end": []}
+    for bad, message in (({"step": 1, "entries": [{"id": "a", "tokens": [10 ** 6], "want": []}], "end": []}, "outside the vocabulary"),
+                         ({"step": 1, "entries": [], "end": ["nobody"]}, "not live"),
+                         ({"step": 1, "entries": [{"id": "a", "tokens": [1, 2], "want": [5]}], "end": []}, "wanted place"),
+                         ("not json", "line 2"), ({"entries": []}, "JSON object")):
+        lines = [json.dumps(good), bad if isinstance(bad, str) else json.dumps(bad)]
+        p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", "float32",
+                            "--out", str(tmp_path / "o"), "--max-tokens", "128"], input="\n".join(lines) + "\n",
+                           capture_output=True, text=True, env=dict(os.environ, HOME=str(tmp_path)), timeout=300)
+        assert p.returncode == 1 and p.stdout.strip() == "done 0", (p.returncode, p.stdout, p.stderr[-500:])
+        assert "trace_run: input line 2" in p.stderr and message in p.stderr, p.stderr[-500:]
