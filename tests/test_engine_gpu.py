@@ -460,3 +460,39 @@ def test_block_arrangement_alone():
     # x = 1 + 0.5 = 1.5; mixer(2x) = 4; x = 5.5; ffn(2x) = -11 pending
     assert torch.equal(x, torch.full((2, 4), 5.5, device="cuda:0"))
     assert torch.equal(pending, torch.full((2, 4), -11.0, device="cuda:0"))
+
+
+@pytest.mark.parametrize("which", ["D", "E"])
+def test_random_workloads_over_engine_options(tmp_path, which):
+    """Requests of random lengths arriving while others run, at the matrix-core sizes, over chunked and
+    whole prompts, small and large budgets, prefix cache, graphs and a pool small enough to preempt:
+    every request ends with the number of tokens it asked for and every page comes back."""
+    import itertools
+    raw, B = H.CONFIGS[which], H.BLOCK_SIZE[which]
+    d = str(tmp_path / "m")
+    H.make_model_dir(d, raw, H.WEIGHT_SEED[which], torch.bfloat16, sharpen=H.SHARPEN[which])
+    preempted = 0
+    for combo, (chunk, budget, prefix, graphs) in enumerate(itertools.product((0, 37), (96, 512), (False, True), (True, False))):
+        rng = np.random.default_rng(combo)
+        eng = _engine(d, dtype="bfloat16", block_size=B, num_blocks=70 * 16 // B, max_seq_len=1024, max_num_seqs=8,
+                      max_batched_tokens=budget, prefill_chunk=chunk, prefix_caching=prefix, use_graphs=graphs)
+        shared = rng.integers(0, raw["vocab_size"], size=100).tolist()
+        pending = []
+        for i in range(16):
+            toks = rng.integers(0, raw["vocab_size"], size=int(rng.choice([1, 2, 16, 17, 60, 130, 257, 400, 700]))).tolist()
+            if prefix and i % 2:
+                toks = (shared + toks)[:900]
+            pending.append((toks, int(rng.integers(1, 30)), float(rng.choice([0.0, 0.8]))))
+        want, done, steps = {}, {}, 0
+        while pending or not eng.idle():
+            if pending and steps % 3 == 0:
+                toks, gen, temp = pending.pop()
+                want[eng.add_request(toks, gen, temperature=temp, seed=7)] = gen
+            eng.step()
+            steps += 1
+            done.update({f.id: f.generated for f in eng.take_finished()})
+            assert steps < 5000
+        assert {r: len(g) for r, g in done.items()} == want, (combo, chunk, budget, prefix, graphs)
+        assert eng.core.blocks_in_use() == 0
+        preempted += eng.core.counters()["preemptions"]
+    assert preempted > 0, "the pool was meant to be small enough to preempt"
