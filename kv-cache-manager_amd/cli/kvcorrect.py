@@ -12,6 +12,7 @@ implementation.  With --refs FILE the reference's KVPR file format is read inste
   3. paged and contiguous policies give identical tokens (scattered physical pages);
   4. all prompts in one batch give the tokens of the solo runs;
   5. prefix caching on: hits happen and outputs stay identical.
+--write-refs FILE keeps the 32-bit yardstick of a run in that container.
 Exit code 0 all pass, 2 some fail, 1 error.
 """
 import struct
@@ -37,6 +38,19 @@ def load_refs(path):
             top_logits = np.frombuffer(f.read(4 * steps * topk), dtype="<f4").reshape(steps, topk)
             out.append(dict(prompt=prompt, greedy=greedy, top_ids=top_ids, top_logits=top_logits))
     return out, steps, topk
+
+
+def write_refs(path, refs, steps, topk):
+    """The same container (src/main_correct.cpp:30-58): "KVPR", prompts, steps, topk; per prompt its
+    length, ids, greedy ids [steps], top ids and top logits [steps][topk]."""
+    with open(path, "wb") as f:
+        f.write(struct.pack("<4s3i", b"KVPR", len(refs), steps, topk))
+        for r in refs:
+            f.write(struct.pack("<i", len(r["prompt"])))
+            f.write(np.asarray(r["prompt"], dtype="<i4").tobytes())
+            f.write(np.asarray(r["greedy"][:steps], dtype="<i4").tobytes())
+            f.write(np.ascontiguousarray(np.asarray(r["top_ids"])[:steps, :topk], dtype="<i4").tobytes())
+            f.write(np.ascontiguousarray(np.asarray(r["top_logits"])[:steps, :topk], dtype="<f4").tobytes())
 
 
 def synthetic_prompts(vocab, n=8, shared=48, seed=11):
@@ -116,6 +130,8 @@ def main(argv=None):
             steps = steps if steps > 0 else 32
             topk = 5
             refs = yardstick(a, base, synthetic_prompts(vocab), steps, topk)
+            if a.has("write-refs"):          # keep the 32-bit yardstick, in the reference's container
+                write_refs(a.str("write-refs", ""), refs, steps, topk)
         a.warn_unused()
         N = len(refs)
         print(f"{N} reference prompts, {steps} steps, top-{topk}")

@@ -50,3 +50,11 @@ def test_kvcorrect_passes_on_a_tiny_model(tmp_path):
     H.make_model_dir(d, H.CONFIGS["A"], H.WEIGHT_SEED["A"], torch.bfloat16)
     p = _run("kvcorrect", "--model", d, "--dtype", "bf16", "--max-seq-len", "128", "--num-blocks", "64", "--steps", "8")
     assert p.returncode == 0, p.stdout + p.stderr
+    assert "ALL CHECKS PASSED" in p.stdout
+    # the yardstick of that kind of run, kept in the reference's container, serves a later run as --refs
+    refs = str(tmp_path / "refs.bin")
+    p = _run("kvcorrect", "--model", d, "--dtype", "bf16", "--max-seq-len", "128", "--num-blocks", "64", "--steps", "8",
+             "--write-refs", refs)
+    assert p.returncode == 0 and os.path.getsize(refs) > 16, p.stdout + p.stderr
+    p = _run("kvcorrect", "--model", d, "--dtype", "bf16", "--max-seq-len", "128", "--num-blocks", "64", "--refs", refs)
+    assert p.returncode == 0 and "8 reference prompts, 8 steps" in p.stdout, p.stdout + p.stderr

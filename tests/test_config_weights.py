@@ -312,3 +312,30 @@ def test_kvmodel_writes_a_folder_that_loads(tmp_path):
     assert set(t) == set(want) and all(tuple(t[n].shape) == want[n][0] for n in t)
     bad = subprocess.run([sys.executable, tool, "--out", str(tmp_path / "x"), "--sizes", "nope"], capture_output=True, text=True)
     assert bad.returncode == 1 and "unknown --sizes" in bad.stderr
+
+
+def test_kvcorrect_refs_container_round_trips(tmp_path):
+    """The reference's KVPR file (src/main_correct.cpp:30-58): written and read back field by field;
+    a wrong magic and a truncated file are refused."""
+    from kvcm_amd.cli.kvcorrect import load_refs, write_refs
+    rng = np.random.default_rng(3)
+    steps, topk = 6, 5
+    refs = [dict(prompt=rng.integers(0, 100, size=n).tolist(), greedy=rng.integers(0, 100, size=steps).tolist(),
+                 top_ids=rng.integers(0, 100, size=(steps, topk)), top_logits=rng.normal(size=(steps, topk)).astype(np.float32))
+            for n in (3, 11, 1)]
+    path = str(tmp_path / "refs.bin")
+    write_refs(path, refs, steps, topk)
+    assert os.path.getsize(path) == 16 + sum(4 + 4 * len(r["prompt"]) + 4 * steps + 8 * steps * topk for r in refs)
+    got, s, k = load_refs(path)
+    assert (s, k, len(got)) == (steps, topk, 3)
+    for a, b in zip(refs, got):
+        assert a["prompt"] == b["prompt"] and a["greedy"] == b["greedy"]
+        np.testing.assert_array_equal(a["top_ids"], b["top_ids"])
+        np.testing.assert_array_equal(a["top_logits"], b["top_logits"])
+    raw = open(path, "rb").read()
+    open(path, "wb").write(b"XXXX" + raw[4:])
+    with pytest.raises(ValueError, match="magic"):
+        load_refs(path)
+    open(path, "wb").write(raw[:-10])
+    with pytest.raises(Exception):
+        load_refs(path)
