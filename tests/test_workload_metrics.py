@@ -81,3 +81,15 @@ def test_metrics_of_finished_requests_and_the_csv_columns(tmp_path):
     assert lines[0].split(",")[:13] == ["policy", "block_size", "num_blocks", "pool_gb", "rate", "shared_frac", "requests",
                                         "completed", "rejected", "wall_s", "output_tokens", "prompt_tokens", "out_tok_s"]
     assert lines[0].split(",")[-3:] == ["peak_blocks", "peak_kv_gb", "gpu_used_gb"] and len(lines[0].split(",")) == 35
+
+
+def test_command_line_parsing_follows_the_reference(capsys):
+    """--key=value, --key value and bare --flag, typed getters with defaults, and a warning for a flag
+    that nobody read (src/common/args.h:12-58)."""
+    a = Args(["--requests=12", "--rate", "2.5", "--prefix", "--policy", "paged", "--typo", "1"])
+    assert a.i32("requests", 0) == 12 and a.f64("rate", 0.0) == 2.5 and a.flag("prefix") and a.str("policy", "x") == "paged"
+    assert a.i32("block-size", 16) == 16 and not a.flag("no-graphs") and a.has("rate") and not a.has("seed")
+    a.warn_unused()
+    assert "unused flag --typo" in capsys.readouterr().err
+    with pytest.raises(ValueError, match="bad argument"):
+        Args(["requests", "3"])
