@@ -56,6 +56,17 @@ __global__ void __launch_bounds__(256)
 
   int u = w_lo;
   if constexpr (MT == 1) {
+    for (; u + 8 <= w_hi; u += 8) {  // long slices: eight units per trip
+      Frag b[16], a[16];
+      const uint16_t* p = wrow + size_t(u) * kUnit;
+      const uint16_t* q = xrow[0] + size_t(u) * kUnit;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) b[i].u = *reinterpret_cast<const uint4*>(p + (i / 2) * kUnit + (i % 2) * 8);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) a[i].u = *reinterpret_cast<const uint4*>(q + (i / 2) * kUnit + (i % 2) * 8);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[i].v, acc[0], 0, 0, 0);
+    }
     for (; u + 4 <= w_hi; u += 4) {  // few rows leave registers for four units per trip: eight weight loads in flight per lane
       Frag b[8], a[8];
       const uint16_t* p = wrow + size_t(u) * kUnit;
