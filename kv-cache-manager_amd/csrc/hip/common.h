@@ -14,11 +14,11 @@ struct bf16_t { uint16_t bits; };
 enum DType : int { kF32 = 0, kBF16 = 1 };
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
+// Round to nearest, ties to even; a NaN stays a quiet NaN.  gfx950 converts in one instruction
+// (v_cvt_pk_bf16_f32); written out in integer operations it costs six and a branch, which epilogues
+// that round a dozen values per lane pay in microseconds.
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest, ties to even
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 template <class T> __device__ __forceinline__ float load_f(const T* p);
@@ -33,6 +33,17 @@ template <> __device__ __forceinline__ void store_f<bf16_t>(bf16_t* p, float v) 
 template <class T> __device__ __forceinline__ float round_to(float v);
 template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }
 template <> __device__ __forceinline__ float round_to<bf16_t>(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+
+// silu(x) = x / (1 + exp(-x)) for a result stored as T.  A bfloat16 result keeps 8 bits of it: the
+// hardware's exp2 and reciprocal (about 1 ulp of float each) take a tenth of the instructions of the
+// exact functions, which in a product's epilogue is microseconds (a 64-lane wave spends 4 cycles
+// per instruction).  A float result takes the exact functions.  One definition for every kernel
+// that applies it, so that all of them give the same bits.
+template <class T> __device__ __forceinline__ float silu(float x);
+template <> __device__ __forceinline__ float silu<float>(float x) { return x / (1.0f + expf(-x)); }
+template <> __device__ __forceinline__ float silu<bf16_t>(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * x));
+}
 
 // (a, b) rotated by the angle whose cosine and sine are given.  One explicit sequence of
 // operations, shared by every kernel that rotates, so that all of them give the same bits.

@@ -361,8 +361,7 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < I) {
     const float x = load_f(g + i);
-    const float s = x / (1.0f + expf(-x));
-    store_f(o + i, round_to<T>(s) * load_f(u + i));
+    store_f(o + i, round_to<T>(silu<T>(x)) * load_f(u + i));
   }
 }
 
@@ -376,7 +375,7 @@ __global__ void __launch_bounds__(256) swiglu_vec_kernel(const T* __restrict__ g
   load4<T>(g, x); load4<T>(g + 4, x + 4);
   load4<T>(g + I, u); load4<T>(g + I + 4, u + 4);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) y[e] = round_to<T>(x[e] / (1.0f + expf(-x[e]))) * u[e];
+  for (int e = 0; e < 8; ++e) y[e] = round_to<T>(silu<T>(x[e])) * u[e];
   T* o = out + size_t(t) * I + i;
   store4<T>(o, y); store4<T>(o + 4, y + 4);
 }

@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(256)
         const int m = t * 16 + (l / 16) * 4 + i;
         if (m >= M) continue;
         const float x = round_to<TO>(g[i]);
-        const float act = x / (1.0f + expf(-x));
+        const float act = silu<TO>(x);
         store_f(out + size_t(m) * ldo + n0 + l % 16, round_to<TO>(act) * round_to<TO>(up[i]));
       }
     }
@@ -288,7 +288,7 @@ __global__ void __launch_bounds__(256)
         const int m = row_base + t * 16 + kq * 4 + i;
         if (m >= M) continue;
         const float x = round_to<TO>(acc[t][i]);
-        const float act = x / (1.0f + expf(-x));
+        const float act = silu<TO>(x);
         store_f(out + size_t(m) * ldo + c0 + r, round_to<TO>(act) * round_to<TO>(up[i]));
       }
     }
