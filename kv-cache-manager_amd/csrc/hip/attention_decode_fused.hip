@@ -70,7 +70,6 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   constexpr int kFusWaves = FusWaves<HD>::N;
   constexpr int STRIDE = kFusWaves / 4;   // a wave takes every STRIDE-th chunk
   const int kvh = blockIdx.x, row = blockIdx.y;
-  const int ctx = ctx_lens[row];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int wq = wave % 4, wfirst = wave / 4;   // which quarter of a chunk, and the first chunk, are this wave's
 
@@ -78,9 +77,43 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   __shared__ __attribute__((aligned(16))) float red[kFusWaves][16][HD + 4];
   __shared__ float w_max[kFusWaves][16], w_sum[kFusWaves][16];
 
+  // ---- prologue, part one: this row's q (GROUP heads), k and v (one kv head) come from the
+  // projection, a pair (j, j + HD/2) of one head per item.  The loads of every thread's first item
+  // go out before anything else is waited for (they need the row's number only, and every row of
+  // the launch, a padding row too, has its row in these arrays); the pages' numbers and the first
+  // keys and values are requested behind them, and only then are the items finished, so that the
+  // three trips to memory overlap instead of following one another.
+  constexpr int kItems = (GROUP + 2) * HALF, kThreads = kFusWaves * kWave;
+  const int width = (nh + 2 * nkv) * HD;
+  const float* prow = partials ? partials + size_t(row) * width : nullptr;
+  const uint16_t* rrow = qkv + size_t(row) * qkv_stride;
+  struct Item { float a[4], b[4]; float2 rot; };
+  auto item_col = [&](int item) {
+    const int h = item / HALF, j = item % HALF;   // 0..GROUP-1: q heads, GROUP: k, GROUP+1: v
+    return (h < GROUP ? (kvh * GROUP + h) * HD : h == GROUP ? (nh + kvh) * HD : (nh + nkv + kvh) * HD) + j;
+  };
+  auto item_request = [&](int item, Item& it) {
+    const int col = item_col(item);
+    if (prow) {   // the first four split-K sums (a split beyond S repeats the last and adds nothing)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const size_t o = size_t(j < S ? j : S - 1) * pstride + col;
+        it.a[j] = prow[o];
+        it.b[j] = prow[o + HALF];
+      }
+    } else {
+      it.a[0] = bf16_bits_to_float(rrow[col]);
+      it.b[0] = bf16_bits_to_float(rrow[col + HALF]);
+    }
+    it.rot = cos_sin && item / HALF <= GROUP ? cos_sin[size_t(row) * HALF + item % HALF] : float2{1.0f, 0.0f};
+  };
+  Item first;
+  item_request(threadIdx.x < kItems ? threadIdx.x : 0, first);
+
+  const int ctx = ctx_lens[row];
   if (ctx <= 0) {   // a padding row: zeros (from the merge when there are parts), nothing read or stored
     if (num_parts == 1)
-      for (int i = threadIdx.x; i < GROUP * HD; i += kFusWaves * kWave)
+      for (int i = threadIdx.x; i < GROUP * HD; i += kThreads)
         out[size_t(row) * out_stride + size_t(kvh) * GROUP * HD + i] = 0;
     return;
   }
@@ -117,61 +150,7 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   auto nth = [&](int i) { return min(c_lo + wfirst + STRIDE * i, my_last); };   // past the last: the last again, never used
   Where wha = lookup(min(nth(0), last)), whb = lookup(min(nth(1), last));
 
-  // ---- prologue: this row's q (GROUP heads), k and v (one kv head) from the projection
-  const int width = (nh + 2 * nkv) * HD;
-  const float* prow = partials ? partials + size_t(row) * width : nullptr;
-  const uint16_t* rrow = qkv + size_t(row) * qkv_stride;
-  auto value = [&](int col) {
-    if (!prow) return bf16_bits_to_float(rrow[col]);
-    float a = 0.f;
-    for (int s0 = 0; s0 < S; s0 += 4) {   // four loads requested together; a split beyond S adds nothing
-      float p[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) p[j] = prow[(s0 + j < S ? s0 + j : S - 1) * pstride + col];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) a += s0 + j < S ? p[j] : 0.f;
-    }
-    return bf16_bits_to_float(float_to_bf16_bits(a));   // the projection's result is a bfloat16 value
-  };
-  const int slot = slots ? slots[row] : -1;
-  const size_t page = slot >= 0 ? slot / B : 0;
-  const int off = slot >= 0 ? slot % B : 0;
-  for (int item = threadIdx.x; item < (GROUP + 2) * HALF; item += kFusWaves * kWave) {
-    const int h = item / HALF, j = item % HALF;   // 0..GROUP-1: q heads, GROUP: k, GROUP+1: v
-    if (h >= GROUP && !(stores && slot >= 0)) continue;
-    const int col = (h < GROUP ? (kvh * GROUP + h) * HD : h == GROUP ? (nh + kvh) * HD : (nh + nkv + kvh) * HD) + j;
-    float a = value(col), b = value(col + HALF);
-    if (h <= GROUP && cos_sin) {
-      const float2 t2 = cos_sin[size_t(row) * HALF + j];
-      rotate_pair(a, b, t2.x, t2.y);
-    }
-    const uint16_t ab = float_to_bf16_bits(a), bb = float_to_bf16_bits(b);
-    if (h < GROUP) {
-      q_lds[h][j] = ab;
-      q_lds[h][j + HALF] = bb;
-    } else if (slot >= 0) {
-      if (h == GROUP) {
-        uint16_t* kr = kcache + ((page * nkv + kvh) * B + off) * HD;
-        kr[j] = ab;
-        kr[j + HALF] = bb;
-      } else {   // values lie transposed inside the page: [dim][slot]
-        uint16_t* vr = vcache + (page * nkv + kvh) * size_t(HD) * B + off;
-        vr[size_t(j) * B] = ab;
-        vr[size_t(j + HALF) * B] = bb;
-      }
-    }
-  }
-  __syncthreads();   // q in LDS; the new key and value are stored before any wave of this workgroup loads them
-
   const int n16 = lane % 16, kq = lane / 16;
-  // B operand of S^T = K Q^T: lane = (query head n16, dims 8 kq .. + 7 of every 32); heads beyond the group are zero
-  FragF qf[KSTEPS];
-#pragma unroll
-  for (int c = 0; c < KSTEPS; ++c) {
-    qf[c].u = *reinterpret_cast<const uint4*>(&q_lds[n16 < GROUP ? n16 : 0][c * 32 + kq * 8]);
-    if (n16 >= GROUP) qf[c].u = uint4{0u, 0u, 0u, 0u};
-  }
-
   // A chunk's operands for this wave: two groups of 32 tokens; a group's keys as two 16-row tiles
   // whose row r holds token 8 (r / 4) + 4 tile + r % 4 of the group, its values as [dim][8 tokens].
   struct Chunk {
@@ -193,6 +172,81 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
       for (int d = 0; d < DT; ++d) ch.v[g][d].u = *reinterpret_cast<const uint4*>(vp + size_t(d) * 16 * B);
     }
   };
+  // The wave's first chunk is requested now unless it holds the token that this workgroup is about
+  // to store (then after the barrier below).  No load sits behind a branch: a wave that must wait
+  // requests the cache's first bytes instead, every lane the same, and drops them.
+  const int slot = slots ? slots[row] : -1;
+  const bool ahead = mine > 0 && !(stores && slot >= 0 && nth(0) == last);
+  Chunk cha, chb;
+  {
+    Where early = wha;
+    if (!ahead) early.k = early.v = 0u;
+    request(early, cha);
+  }
+
+  // ---- prologue, part two: sum, rotate, round; q to LDS, the new key and value to their page
+  const size_t page = slot >= 0 ? slot / B : 0;
+  const int off = slot >= 0 ? slot % B : 0;
+  auto item_finish = [&](int item, const Item& it) {
+    const int h = item / HALF, j = item % HALF;
+    if (h >= GROUP && !(stores && slot >= 0)) return;
+    float a = it.a[0], b = it.b[0];
+    if (prow) {
+      const int col = item_col(item);
+      a = 0.f;
+      b = 0.f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        a += k < S ? it.a[k] : 0.f;
+        b += k < S ? it.b[k] : 0.f;
+      }
+      for (int s0 = 4; s0 < S; s0 += 4) {   // four loads requested together
+        float pa[4], pb[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const size_t o = size_t(s0 + k < S ? s0 + k : S - 1) * pstride + col;
+          pa[k] = prow[o];
+          pb[k] = prow[o + HALF];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          a += s0 + k < S ? pa[k] : 0.f;
+          b += s0 + k < S ? pb[k] : 0.f;
+        }
+      }
+      a = bf16_bits_to_float(float_to_bf16_bits(a));   // the projection's result is a bfloat16 value
+      b = bf16_bits_to_float(float_to_bf16_bits(b));
+    }
+    if (h <= GROUP && cos_sin) rotate_pair(a, b, it.rot.x, it.rot.y);
+    const uint16_t ab = float_to_bf16_bits(a), bb = float_to_bf16_bits(b);
+    if (h < GROUP) {
+      q_lds[h][j] = ab;
+      q_lds[h][j + HALF] = bb;
+    } else if (h == GROUP) {
+      uint16_t* kr = kcache + ((page * nkv + kvh) * B + off) * HD;
+      kr[j] = ab;
+      kr[j + HALF] = bb;
+    } else {   // values lie transposed inside the page: [dim][slot]
+      uint16_t* vr = vcache + (page * nkv + kvh) * size_t(HD) * B + off;
+      vr[size_t(j) * B] = ab;
+      vr[size_t(j + HALF) * B] = bb;
+    }
+  };
+  if (threadIdx.x < kItems) item_finish(threadIdx.x, first);
+  for (int item = threadIdx.x + kThreads; item < kItems; item += kThreads) {
+    Item it;
+    item_request(item, it);
+    item_finish(item, it);
+  }
+  __syncthreads();   // q in LDS; the new key and value are stored before any wave of this workgroup loads them
+
+  // B operand of S^T = K Q^T: lane = (query head n16, dims 8 kq .. + 7 of every 32); heads beyond the group are zero
+  FragF qf[KSTEPS];
+#pragma unroll
+  for (int c = 0; c < KSTEPS; ++c) {
+    qf[c].u = *reinterpret_cast<const uint4*>(&q_lds[n16 < GROUP ? n16 : 0][c * 32 + kq * 8]);
+    if (n16 >= GROUP) qf[c].u = uint4{0u, 0u, 0u, 0u};
+  }
 
   // running state of this lane's head (n16): maximum (log2 domain), this lane's share of the sum,
   // and O^T (column = head, rows = dims 16 d + 4 kq + i)
@@ -250,8 +304,7 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   // The chunk after the last repeats the last one, so that no load sits behind a branch; what it
   // brings is never used.
   if (mine > 0) {
-    Chunk cha, chb;
-    request(wha, cha);
+    if (!ahead) request(wha, cha);
     wha = lookup(nth(2));
     for (int i = 0; i < mine; i += 2) {
       request(whb, chb);                 // this wave's chunk i + 1
