@@ -21,9 +21,9 @@
 // The only mask is causal: a row at position p sees tokens t <= p.  Rows of different sequences
 // never share a workgroup.  Head sizes 64 and 128; pages of 8, 16, 32, ... tokens (a power of two).
 //
-// Long contexts are cut into segments of 1,024 keys (at absolute multiples of 1,024) that run as
-// workgroups of their own: without that the launch lasts as long as its last rows need to walk
-// all their keys, while the workgroups of early rows have long finished.  A tile whose rows see
+// While tiles x heads x sequences give fewer than two workgroups per CU, contexts are cut into
+// segments of keys (multiples of 512, at absolute multiples of their length) that run as workgroups
+// of their own: without that a short portion behind a long context leaves most of the chip idle.  A tile whose rows see
 // one segment stores its result; otherwise every segment leaves (o / l, m, l) per row in scratch
 // and a second kernel merges them in segment order.
 #include <cfloat>
@@ -36,6 +36,10 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
+// 16 bytes on their way from the cache to LDS.  A native vector, not HIP's uint4: arrays of that
+// struct type are not split into registers by the compiler, they went through scratch memory, and
+// every load was waited for at once instead of two chunks later.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 union PFrag {
   uint4 u;
   uint2 h[2];
@@ -49,9 +53,9 @@ constexpr int kPfWaveRows = 16 * kPfRT;
 constexpr int kPfRows = kPfWaveRows * kPfWaves;  // query rows per workgroup
 constexpr int kPfChunk = 64;                     // keys per trip
 constexpr int kPfPad = 8;                        // bfloat16 of padding per LDS row (keeps 16-byte alignment)
-constexpr int kPfSeg = 1024;                     // keys per segment: a multiple of this, chosen per launch
+constexpr int kPfSeg = 512;                      // keys per segment: a multiple of this, chosen per launch
 constexpr int kPfSegMax = 16384;                 // at most (its page ids lie in LDS)
-constexpr long long kPfFill = 4096;              // workgroups a launch should have before segments grow
+constexpr long long kPfFill = 512;               // workgroups a launch should have before segments grow (two per CU)
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   union { bf16x2_t v; uint32_t u; } r;
@@ -60,16 +64,22 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 }
 // all-reduce over the four lanes that share lane % 16 (lanes l, l^16, l^32, l^48)
 __device__ __forceinline__ float quad_rows_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16, kWave));
-  return fmaxf(v, __shfl_xor(v, 32, kWave));
+  // v_permlane16_swap / v_permlane32_swap with both operands the same register leave one half of
+  // each lane pair in the first result and the other half in the second
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float quad_rows_sum(float v) {
   v += __shfl_xor(v, 16, kWave);
   return v + __shfl_xor(v, 32, kWave);
 }
 
+// Two waves per SIMD at least: with that bound the compiler keeps the accumulators of the matrix
+// instructions in ordinary registers (no copies to and from the accumulation registers around the softmax).
 template <int HD>
-__global__ void __launch_bounds__(kPfThreads)
+__global__ void __launch_bounds__(kPfThreads, 2)
     attention_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                              const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                              const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
@@ -143,17 +153,17 @@ __global__ void __launch_bounds__(kPfThreads)
   // pieces of keys (8 dims of one token) and as many of values (8 tokens of one dim).  Tokens past
   // the workgroup's last position are read from that position's place instead (always valid
   // memory); the mask keeps them out.
-  struct Pieces { uint4 k[PIECES], v[PIECES]; };
+  struct Pieces { u32x4 k[PIECES], v[PIECES]; };
   auto request = [&](int c0, Pieces& pc) {
     c0 = min(c0, block_last_pos & ~(kPfChunk - 1));   // past the last chunk: the last chunk again (no load behind a branch)
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
       const int e = threadIdx.x + i * kPfThreads;
       const int t = min(c0 + e / (HD / 8), block_last_pos);
-      pc.k[i] = *reinterpret_cast<const uint4*>(kbase + size_t(page_lds[(t >> b_shift) - page_lo]) * page_elems +
+      pc.k[i] = *reinterpret_cast<const u32x4*>(kbase + size_t(page_lds[(t >> b_shift) - page_lo]) * page_elems +
                                                 size_t(t & b_mask) * HD + (e % (HD / 8)) * 8);
       const int tv = min(c0 + (e % 8) * 8, block_last_pos & ~7);
-      pc.v[i] = *reinterpret_cast<const uint4*>(vbase + size_t(page_lds[(tv >> b_shift) - page_lo]) * page_elems +
+      pc.v[i] = *reinterpret_cast<const u32x4*>(vbase + size_t(page_lds[(tv >> b_shift) - page_lo]) * page_elems +
                                                 size_t(e / 8) * B + (tv & b_mask));
     }
   };
@@ -161,8 +171,8 @@ __global__ void __launch_bounds__(kPfThreads)
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
       const int e = threadIdx.x + i * kPfThreads;
-      *reinterpret_cast<uint4*>(&k_lds[buf][e / (HD / 8)][(e % (HD / 8)) * 8]) = pc.k[i];
-      *reinterpret_cast<uint4*>(&v_lds[buf][e / 8][(e % 8) * 8]) = pc.v[i];
+      *reinterpret_cast<u32x4*>(&k_lds[buf][e / (HD / 8)][(e % (HD / 8)) * 8]) = pc.k[i];
+      *reinterpret_cast<u32x4*>(&v_lds[buf][e / 8][(e % 8) * 8]) = pc.v[i];
     }
   };
 
@@ -224,7 +234,7 @@ __global__ void __launch_bounds__(kPfThreads)
             s[rt][j][i] = __builtin_amdgcn_exp2f(fmaf(s[rt][j][i], scale_log2, shift));
             sum += s[rt][j][i];
           }
-        l[rt] = l[rt] * alpha + quad_rows_sum(sum);
+        l[rt] = l[rt] * alpha + sum;   // this lane's share; the four lanes of a row are added up at the end
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // the maximum moves in few chunks
 #pragma unroll
           for (int d = 0; d < DT; ++d)
@@ -280,8 +290,9 @@ __global__ void __launch_bounds__(kPfThreads)
 #pragma unroll
   for (int rt = 0; rt < kPfRT; ++rt) {
     const int r = first + rt * 16 + n16;
+    const float l_row = quad_rows_sum(l[rt]);
     if (r >= n_rows) continue;
-    const float inv = l[rt] > 0.f ? 1.0f / l[rt] : 0.f;
+    const float inv = l_row > 0.f ? 1.0f / l_row : 0.f;
     if (n_segs == 1) {
       uint16_t* orow = out + size_t(row0 + r) * out_stride + size_t(head) * HD + 4 * kq;
 #pragma unroll
@@ -297,7 +308,7 @@ __global__ void __launch_bounds__(kPfThreads)
       for (int d = 0; d < DT; ++d)
         *reinterpret_cast<float4*>(dst + d * 16 + 4 * kq) =
             float4{o[rt][d][0] * inv, o[rt][d][1] * inv, o[rt][d][2] * inv, o[rt][d][3] * inv};
-      if (kq == 0) { dst[HD] = m[rt] > -0.5f * FLT_MAX ? m[rt] * scale_log2 : -FLT_MAX; dst[HD + 1] = l[rt]; }
+      if (kq == 0) { dst[HD] = m[rt] > -0.5f * FLT_MAX ? m[rt] * scale_log2 : -FLT_MAX; dst[HD + 1] = l_row; }
     }
   }
 }
@@ -348,8 +359,8 @@ int kvcm_attention_prefill_supported(int nh, int nkv, int hd, int B) {
   return nkv > 0 && nh % nkv == 0 && (hd == 64 || hd == 128) && B >= 8 && (B & (B - 1)) == 0;
 }
 
-// Keys per segment of a launch: 1,024 while that gives the chip fewer than kPfFill workgroups,
-// longer (in multiples of 1,024) when tiles x heads x sequences already fill it, since every segment
+// Keys per segment of a launch: 512 while that gives the chip fewer than kPfFill workgroups,
+// longer (in multiples of 512) when tiles x heads x sequences already fill it, since every segment
 // beyond the first costs a partial result per row and head in scratch.
 int kvcm_attention_prefill_segment(int max_run, int S, int nh, int max_context) {
   if (max_run <= 0 || S <= 0 || nh <= 0 || max_context <= 0) return kPfSeg;

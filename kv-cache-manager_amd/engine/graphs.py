@@ -14,12 +14,29 @@ context are captured for a bound on it.  There is one graph per (bucket, context
 replays the graph of the smallest class that holds its longest context, so that an engine that
 allows long sequences still runs short ones with the launches made for short ones.
 """
+import contextlib
+import gc
 from typing import Dict, List
 
 import numpy as np
 import torch
 
 from .runner import StepContext
+
+
+@contextlib.contextmanager
+def _no_collection():
+    """No garbage collection while a stream is being captured: a collection that happens to start
+    there may destroy device objects of an engine that is no longer used (its graphs, their memory
+    pools), and releasing device memory during a capture ends the process."""
+    was_enabled = gc.isenabled()
+    gc.collect()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if was_enabled:
+            gc.enable()
 
 _BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256, 384, 512)
 _CONTEXT_CLASSES = (1024, 2048, 8192, 32768)       # and the longest context the engine allows
@@ -100,7 +117,7 @@ class DecodeGraphs:
             self._forward(layout, bucket, bound)          # eager once: creates every work buffer
             torch.cuda.current_stream().synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            with _no_collection(), torch.cuda.graph(graph):
                 self._forward(layout, bucket, bound)
             self.graphs[(bucket, bound)] = graph
         graph.replay()

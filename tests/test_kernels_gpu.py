@@ -925,9 +925,10 @@ def test_prefill_attention_long_prompt(ops):
     runs = [(0, 1500), (1000, 300)]
     P = _runs_problem(rng, runs, nh, nkv, hd, B)
     got = _run_prefill(ops, P, runs, nh, nkv, hd)
-    # contexts beyond 1,024 keys are cut into segments that are merged afterwards: rows around the
-    # cut, a tile that the cut goes through (the second run starts at 1000), tile edges
-    rows = [0, 1, 63, 64, 700, 1023, 1024, 1025, 1151, 1152, 1499, 1500, 1523, 1524, 1627, 1628, 1799]
+    # a launch this narrow cuts contexts into segments of 512 keys that are merged afterwards: rows
+    # around the cuts, a tile that a cut goes through (the second run starts at 1000), tile edges
+    assert ops.attention_prefill_segment(1500, 2, nh, 1500) == 512
+    rows = [0, 1, 63, 64, 511, 512, 513, 700, 1023, 1024, 1025, 1151, 1152, 1499, 1500, 1523, 1524, 1535, 1536, 1627, 1628, 1799]
     ref = np.zeros((len(rows), nh, hd))
     for k, r in enumerate(rows):
         s, c = P["row_seq"][r], P["ctx"][r]
@@ -936,7 +937,7 @@ def test_prefill_attention_long_prompt(ops):
 
 
 def test_prefill_attention_three_segments_far_key(ops):
-    """A row deep in the third segment of keys must still find one outstanding key of the first."""
+    """A row deep in the fifth segment of keys must still find one outstanding key of the first."""
     rng = np.random.default_rng(52)
     nh, nkv, hd, B = 4, 1, 128, 16
     runs = [(0, 2300)]
@@ -959,17 +960,19 @@ def test_prefill_attention_three_segments_far_key(ops):
 
 
 def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops):
-    """Many heads and sequences fill the chip without short segments: the launch then cuts contexts
-    into segments of 2,048 keys.  Rows on both sides of that cut, and a far key of the first segment."""
+    """The wider a launch (tiles x heads x sequences), the longer its segments of keys; one that fills
+    the chip by itself is not cut at all.  Here three runs give segments of 1,024 keys: rows on both
+    sides of that cut, and a far key of the first segment."""
     rng = np.random.default_rng(53)
     nh, nkv, hd, B = 32, 4, 64, 16
-    runs = [(2000 + 13 * i, 300) for i in range(22)]
-    assert ops.attention_prefill_segment(300, len(runs), nh, max(s + n for s, n in runs)) == 2048
-    assert ops.attention_prefill_segment(300, 2, nh, 2600) == 1024 and ops.attention_prefill_segment(4096, 1, 32, 32768) == 8192
+    runs = [(900 + 13 * i, 384) for i in range(3)]
+    assert ops.attention_prefill_segment(384, len(runs), nh, max(s + n for s, n in runs)) == 1024
+    assert ops.attention_prefill_segment(300, 2, nh, 2600) == 1024 and ops.attention_prefill_segment(2048, 1, 32, 2048) == 2048
+    assert ops.attention_prefill_segment(4096, 1, 32, 32768) == 16384 and ops.attention_prefill_segment(128, 1, 4, 32768) == 512
     P = _paged_problem(rng, [s + n for s, n in runs], nh, nkv, hd, B, all_rows=False)
     R = sum(n for _, n in runs)
     Q = _bf16_grid(rng.normal(size=(R, nh, hd)))
-    far, seq, head = 40, 3, 9                                   # kv head 1
+    far, seq, head = 40, 1, 9                                   # kv head 1
     row_lo = sum(n for _, n in runs[:seq])
     Q[row_lo + 100:row_lo + 300, head] = 0.0
     Q[row_lo + 100:row_lo + 300, head, 3] = 30.0
@@ -981,8 +984,8 @@ def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops):
     got = _run_prefill(ops, P, runs, nh, nkv, hd, scale=1.0)
     np.testing.assert_allclose(got[row_lo + 100:row_lo + 300, head],
                                np.broadcast_to(P["Vl"][seq][far, 1], (200, hd)), atol=2e-2)
-    for s, r in ((0, 0), (0, 47), (0, 48), (0, 299), (3, 5), (3, 6), (21, 0), (21, 299), (10, 128)):
-        pos = runs[s][0] + r                                   # the cut lies between positions 2047 and 2048
+    for s, r in ((0, 0), (0, 123), (0, 124), (0, 383), (1, 110), (1, 111), (2, 97), (2, 98), (2, 383), (1, 128)):
+        pos = runs[s][0] + r                                   # the cut lies between positions 1023 and 1024
         row = sum(n for _, n in runs[:s]) + r
         ref = plain.attention(Q[row:row + 1], P["Kl"][s][:pos + 1], P["Vl"][s][:pos + 1], [pos], np.arange(pos + 1), 1.0)[0]
         np.testing.assert_allclose(got[row], ref, atol=1e-2, rtol=0, err_msg=f"sequence {s} row {r}")
