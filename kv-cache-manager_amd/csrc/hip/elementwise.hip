@@ -279,33 +279,67 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int
   for (int d = threadIdx.x; d < hd; d += blockDim.x) store_f(cache_head + size_t(d) * B, value(h * hd + d));
 }
 
+// Values of whole fused rows to their transposed pages ([page][kv_head][dim][slot]): a thread takes
+// one dim of one kv head for a group of 8 rows.  Lanes are neighbours in dim, so a wave reads
+// contiguous pieces of each row; where the group's slots are 8 consecutive ones that start at a
+// multiple of 8 (the rows of a prompt portion) the thread stores them as one vector, which makes the
+// page rows whole again, otherwise slot by slot.  Groups are counted from the first row whose slot
+// is a multiple of 8, so that a portion which starts anywhere in its sequence is still stored in
+// vectors (rows before it form a short group of their own).
+constexpr int kVGroup = 8;
+template <class T>
+__device__ __forceinline__ void v_page_item(const T* __restrict__ qkv, int row_stride, const int* __restrict__ slots,
+                                            T* __restrict__ vcache, int nh, int nkv, int hd, int B, int rows, long long item) {
+  const int d = int(item % hd), kvh = int((item / hd) % nkv), g = int(item / (static_cast<long long>(hd) * nkv));
+  const int s_first = slots[0];
+  const int shift = s_first >= 0 ? (kVGroup - s_first % kVGroup) % kVGroup : 0;
+  const int lo = shift - kVGroup + g * kVGroup;
+  const T* src = qkv + size_t(nh + nkv + kvh) * hd + d;
+  bool whole = lo >= 0 && lo + kVGroup <= rows && B % kVGroup == 0;
+  int s0 = -1;
+  if (whole) {
+    s0 = slots[lo];
+    whole = s0 >= 0 && s0 % kVGroup == 0;
+#pragma unroll
+    for (int k = 1; k < kVGroup; ++k) whole = whole && slots[lo + k] == s0 + k;
+  }
+  if (whole) {
+    float v[kVGroup];
+#pragma unroll
+    for (int k = 0; k < kVGroup; ++k) v[k] = load_f(src + size_t(lo + k) * row_stride);
+    T* dst = vcache + ((size_t(s0 / B) * nkv + kvh) * hd + d) * B + s0 % B;
+    store4<T>(dst, v);
+    store4<T>(dst + 4, v + 4);
+    return;
+  }
+  for (int t = lo < 0 ? 0 : lo; t < lo + kVGroup && t < rows; ++t) {
+    const int slot = slots[t];
+    if (slot >= 0) store_f(vcache + ((size_t(slot / B) * nkv + kvh) * hd + d) * B + slot % B, load_f(src + size_t(t) * row_stride));
+  }
+}
+
 // The same for whole fused rows (no partial sums) whose head size is a multiple of 16: a thread
-// takes 8 pairs of a q or k head (or 16 values of a v head) with vector loads and stores, so a
-// prompt's rows move at memory speed.  Same formulas, same values as the kernel above.
+// takes 8 pairs of a q or k head with vector loads and stores (items below qk_items), or one dim of
+// a v head for 8 rows (the items after them), so a prompt's rows move at memory speed.  Same
+// formulas, same values as the kernel above.
 template <class T>
 __global__ void __launch_bounds__(256)
     rope_cache_vec_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                           const float* __restrict__ inv_freq, const int* __restrict__ slots, T* __restrict__ kcache,
                           T* __restrict__ vcache, int nh, int nkv, int hd, int B, const float2* __restrict__ cos_sin,
-                          long long items) {
+                          int rows, long long qk_items, long long items) {
   const long long item = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x;
   if (item >= items) return;
-  const int cph = hd / 16, heads = nh + 2 * nkv, half = hd / 2;
+  if (item >= qk_items) {
+    v_page_item<T>(qkv, row_stride, slots, vcache, nh, nkv, hd, B, rows, item - qk_items);
+    return;
+  }
+  const int cph = hd / 16, heads = nh + nkv, half = hd / 2;
   const int c = int(item % cph), h = int((item / cph) % heads), t = int(item / (static_cast<long long>(cph) * heads));
   T* row = qkv + size_t(t) * row_stride + size_t(h) * hd;
   const int slot = slots ? slots[t] : -1;
   const size_t page = slot >= 0 ? slot / B : 0;
   const int off = slot >= 0 ? slot % B : 0;
-  if (h >= nh + nkv) {   // a v head: 16 values to the transposed page
-    if (slot < 0) return;
-    float v[16];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) load4<T>(row + c * 16 + 4 * k, v + 4 * k);
-    T* cache_head = vcache + (page * nkv + (h - nh - nkv)) * size_t(hd) * B + off;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) store_f(cache_head + size_t(c * 16 + e) * B, v[e]);
-    return;
-  }
   const bool is_k = h >= nh;
   T* cache_row = (is_k && slot >= 0) ? kcache + ((page * nkv + (h - nh)) * B + off) * hd : nullptr;
   const int j0 = c * 8;
@@ -455,19 +489,26 @@ int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, 
   KVCM_REQUIRE(!partials || S >= 1, "rope: partial sums need their split count");
   KVCM_REQUIRE(nh + 2 * nkv <= 65535 && nh + 2 * nkv > 0, "rope: too many heads");
   const bool aligned = reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
-                       reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0 && row_stride % 4 == 0;
+                       reinterpret_cast<uintptr_t>(vcache) % 16 == 0 && reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0 &&
+                       row_stride % 4 == 0;
   if (!partials && hd % 16 == 0 && aligned) {
-    const long long items = static_cast<long long>(T) * (nh + 2 * nkv) * (hd / 16);
+    // q and k heads: 8 pairs per item; v heads (only when there is a cache to store them to): one
+    // dim of 8 rows per item, one group more than the rows fill because groups start at a slot
+    // that is a multiple of 8
+    const long long qk_items = static_cast<long long>(T) * (nh + nkv) * (hd / 16);
+    const long long v_items = slots ? static_cast<long long>((T + kVGroup - 1) / kVGroup + 1) * nkv * hd : 0;
+    const long long items = qk_items + v_items;
     const long long blocks = (items + 255) / 256;
     KVCM_REQUIRE(blocks < (1ll << 31), "rope: too many rows");
+    if (blocks == 0) return 0;
     if (dtype == kF32)
       rope_cache_vec_kernel<float><<<static_cast<unsigned>(blocks), 256, 0, s>>>(
           static_cast<float*>(qkv), row_stride, positions, inv_freq, slots, static_cast<float*>(kcache),
-          static_cast<float*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), items);
+          static_cast<float*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), T, qk_items, items);
     else if (dtype == kBF16)
       rope_cache_vec_kernel<bf16_t><<<static_cast<unsigned>(blocks), 256, 0, s>>>(
           static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots, static_cast<bf16_t*>(kcache),
-          static_cast<bf16_t*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), items);
+          static_cast<bf16_t*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), T, qk_items, items);
     else KVCM_REQUIRE(false, "rope: unknown dtype %d", dtype);
     return launch_status("rope_cache");
   }

@@ -195,6 +195,37 @@ def test_reshape_and_cache_scatters_to_slots(ops, dtype):
     assert np.count_nonzero(K.any(axis=(1, 3))) == T - 1            # nothing else was touched
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,first_slots", [(16, [0]), (16, [37]), (8, [5, 64]), (32, [100, 3]), (16, [7, 72, 16 * 9 + 15])])
+def test_values_of_runs_of_consecutive_slots_reach_their_transposed_pages(ops, dtype, B, first_slots):
+    """Rows whose slots are consecutive (a prompt portion) are stored to the value pages eight at a
+    time: portions that start at a multiple of eight and elsewhere, several portions in one call (the
+    second is then out of step with the first), a row in the middle that is not stored, and rows
+    that cross pages.  Every other slot of the cache stays zero."""
+    rng = np.random.default_rng(61)
+    NH, KVH, HD, NB = 3, 2, 32, 24
+    lengths = [45, 23, 9][:len(first_slots)]
+    slots = np.concatenate([np.arange(f, f + n) for f, n in zip(first_slots, lengths)]).astype(np.int32)
+    assert slots.max() < NB * B and len(set(slots.tolist())) == len(slots)
+    T = len(slots)
+    skipped = 19
+    natural = slots[skipped]
+    slots[skipped] = -1
+    rows = _bf16_grid(rng.normal(size=(T, (NH + 2 * KVH) * HD)))
+    kc = torch.zeros(NB, KVH, B, HD, dtype=dtype, device=DEV)
+    vc = torch.zeros(NB, KVH, HD, B, dtype=dtype, device=DEV)
+    ops.rope_cache(_t(rows, dtype), NH, KVH, HD, slots=_t(slots, torch.int32), kcache=kc, vcache=vc, block_size=B)
+    K, V = _np(kc), _np(vc).transpose(0, 1, 3, 2)
+    want_k, want_v = np.zeros_like(K), np.zeros_like(V)
+    for t in range(T):
+        if slots[t] >= 0:
+            want_k[slots[t] // B, :, slots[t] % B] = rows[t, NH * HD:(NH + KVH) * HD].reshape(KVH, HD)
+            want_v[slots[t] // B, :, slots[t] % B] = rows[t, (NH + KVH) * HD:].reshape(KVH, HD)
+    np.testing.assert_array_equal(K, want_k)
+    np.testing.assert_array_equal(V, want_v)
+    assert not V[natural // B, :, natural % B].any()
+
+
 def test_fused_rope_and_cache_write_stores_rotated_keys(ops):
     rng = np.random.default_rng(6)
     T, NH, KVH, HD, B = 5, 6, 2, 32, 8
