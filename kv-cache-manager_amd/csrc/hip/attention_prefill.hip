@@ -15,8 +15,9 @@
 // 16-token tile; after exp those registers, rounded to bfloat16 and packed, ARE the B operand of
 // the second product (the order of the reduction index inside a matrix instruction is free as long
 // as both operands agree, so the values are read from LDS in that same token order).  The
-// probabilities never touch LDS, a row's maximum and sum live in one lane each, and the output is
-// stored four dims at a time.
+// probabilities never touch LDS, a row's maximum lives in one lane, its sum comes from a third
+// product (ones * P^T: the sum of the probabilities as the second product sees them), and the
+// output is stored four dims at a time.
 //
 // The only mask is causal: a row at position p sees tokens t <= p.  Rows of different sequences
 // never share a workgroup.  Head sizes 64 and 128; pages of 8, 16, 32, ... tokens (a power of two).
@@ -71,10 +72,6 @@ __device__ __forceinline__ float quad_rows_max(float v) {
   auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
-__device__ __forceinline__ float quad_rows_sum(float v) {
-  v += __shfl_xor(v, 16, kWave);
-  return v + __shfl_xor(v, 32, kWave);
-}
 
 // Two waves per SIMD at least: with that bound the compiler keeps the accumulators of the matrix
 // instructions in ordinary registers (no copies to and from the accumulation registers around the softmax).
@@ -91,9 +88,13 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   constexpr int KPITCH = HD + kPfPad, VPITCH = kPfChunk + kPfPad;
   // Workgroups are handed out in the order of blockIdx.x, round-robin over the chip's eight parts:
   // neighbours in that order are the heads of one (tile, segment), so that every part gets the
-  // same mix of long and short walks, and the long ones (late rows) start first.
+  // same mix of long and short walks.
   const int head = blockIdx.x % nh, seq = blockIdx.y;
-  const int unit = gridDim.x / nh - 1 - blockIdx.x / nh;
+  // The first half of the launch takes the longest walks, longest first, the second half the
+  // shortest, shortest first: when two workgroups at a time fit a CU, a long walk shares it with a
+  // short one and every CU gets about the same number of chunks (32 + 2, 30 + 4, ... for one prompt).
+  const int n_units = gridDim.x / nh, turn = blockIdx.x / nh, top = (n_units + 1) / 2;
+  const int unit = turn < top ? n_units - 1 - turn : turn - top;
   const int tile = unit / max_segs, seg = unit % max_segs;
   const int row0 = run_start[seq], n_rows = run_start[seq + 1] - row0;
   const int block_first = tile * kPfRows;
@@ -138,12 +139,15 @@ __global__ void __launch_bounds__(kPfThreads, 2)
     for (int c = 0; c < KSTEPS; ++c)
       qf[rt][c].u = *reinterpret_cast<const uint4*>(q + size_t(row0 + r) * q_stride + size_t(head) * HD + c * 32 + kq * 8);
   }
-  float m[kPfRT], l[kPfRT];
+  float m[kPfRT];
+  f32x4 l[kPfRT];   // every element: the sum of the lane's query row (a product with a matrix of ones)
+  PFrag ones;
+  ones.u = uint4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   f32x4 o[kPfRT][DT];   // O^T: column = query row n16, rows = dims 16 d + 4 kq + i
 #pragma unroll
   for (int rt = 0; rt < kPfRT; ++rt) {
     m[rt] = -FLT_MAX;
-    l[rt] = 0.f;
+    l[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int d = 0; d < DT; ++d) o[rt][d] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -153,26 +157,31 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   // pieces of keys (8 dims of one token) and as many of values (8 tokens of one dim).  Tokens past
   // the workgroup's last position are read from that position's place instead (always valid
   // memory); the mask keeps them out.
+  // A thread's key pieces are the same 8 dims of PIECES consecutive tokens (an aligned group, so one
+  // page), its value pieces the same 8 tokens of dims 32 apart: one page lookup each per chunk, the
+  // other pieces lie a constant away.
   struct Pieces { u32x4 k[PIECES], v[PIECES]; };
+  constexpr int KTPR = HD / 8;   // threads per key row
+  const int k_p = threadIdx.x / KTPR, k_col = threadIdx.x % KTPR;
+  const int v_g = threadIdx.x % 8, v_d = threadIdx.x / 8;
+  const int last_chunk = block_last_pos & ~(kPfChunk - 1), last_kgroup = block_last_pos & ~(PIECES - 1),
+            last_vgroup = block_last_pos & ~7;
   auto request = [&](int c0, Pieces& pc) {
-    c0 = min(c0, block_last_pos & ~(kPfChunk - 1));   // past the last chunk: the last chunk again (no load behind a branch)
+    c0 = min(c0, last_chunk);   // past the last chunk: the last chunk again (no load behind a branch)
+    const int t0 = min(c0 + k_p * PIECES, last_kgroup);
+    const uint16_t* kp = kbase + size_t(page_lds[(t0 >> b_shift) - page_lo]) * page_elems + size_t(t0 & b_mask) * HD + k_col * 8;
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-      const int e = threadIdx.x + i * kPfThreads;
-      const int t = min(c0 + e / (HD / 8), block_last_pos);
-      pc.k[i] = *reinterpret_cast<const u32x4*>(kbase + size_t(page_lds[(t >> b_shift) - page_lo]) * page_elems +
-                                                size_t(t & b_mask) * HD + (e % (HD / 8)) * 8);
-      const int tv = min(c0 + (e % 8) * 8, block_last_pos & ~7);
-      pc.v[i] = *reinterpret_cast<const u32x4*>(vbase + size_t(page_lds[(tv >> b_shift) - page_lo]) * page_elems +
-                                                size_t(e / 8) * B + (tv & b_mask));
-    }
+    for (int i = 0; i < PIECES; ++i) pc.k[i] = *reinterpret_cast<const u32x4*>(kp + i * HD);
+    const int tv = min(c0 + v_g * 8, last_vgroup);
+    const uint16_t* vp = vbase + size_t(page_lds[(tv >> b_shift) - page_lo]) * page_elems + size_t(v_d) * B + (tv & b_mask);
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) pc.v[i] = *reinterpret_cast<const u32x4*>(vp + size_t(i) * 32 * B);
   };
   auto stage = [&](int buf, const Pieces& pc) {
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
-      const int e = threadIdx.x + i * kPfThreads;
-      *reinterpret_cast<u32x4*>(&k_lds[buf][e / (HD / 8)][(e % (HD / 8)) * 8]) = pc.k[i];
-      *reinterpret_cast<u32x4*>(&v_lds[buf][e / 8][(e % 8) * 8]) = pc.v[i];
+      *reinterpret_cast<u32x4*>(&k_lds[buf][k_p * PIECES + i][k_col * 8]) = pc.k[i];
+      *reinterpret_cast<u32x4*>(&v_lds[buf][v_d + 32 * i][v_g * 8]) = pc.v[i];
     }
   };
 
@@ -225,17 +234,14 @@ __global__ void __launch_bounds__(kPfThreads, 2)
         const float shift = seen ? -m_new * scale_log2 : -FLT_MAX;       // exp2(s * scale + shift)
         const float alpha = seen ? __builtin_amdgcn_exp2f((m[rt] - m_new) * scale_log2) : 1.0f;
         m[rt] = m_new;
-        float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            // masked scores are -FLT_MAX: the product overflows to -inf, exp2 gives 0
+          for (int i = 0; i < 4; ++i)   // masked scores are -FLT_MAX: the product overflows to -inf, exp2 gives 0
             s[rt][j][i] = __builtin_amdgcn_exp2f(fmaf(s[rt][j][i], scale_log2, shift));
-            sum += s[rt][j][i];
-          }
-        l[rt] = l[rt] * alpha + sum;   // this lane's share; the four lanes of a row are added up at the end
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // the maximum moves in few chunks
+#pragma unroll
+          for (int i = 0; i < 4; ++i) l[rt][i] *= alpha;
 #pragma unroll
           for (int d = 0; d < DT; ++d)
 #pragma unroll
@@ -250,6 +256,11 @@ __global__ void __launch_bounds__(kPfThreads, 2)
           pf[rt][c].u.w = pack_bf16(s[rt][2 * c + 1][2], s[rt][2 * c + 1][3]);
         }
       }
+      // ---- the rows' sums, of the probabilities as the product below sees them: ones * P^T
+#pragma unroll
+      for (int rt = 0; rt < kPfRT; ++rt)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) l[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pf[rt][c].v, l[rt], 0, 0, 0);
       // ---- O^T += V^T * P^T, values read in the same token order
 #pragma unroll
       for (int c = 0; c < 2; ++c)
@@ -290,7 +301,7 @@ __global__ void __launch_bounds__(kPfThreads, 2)
 #pragma unroll
   for (int rt = 0; rt < kPfRT; ++rt) {
     const int r = first + rt * 16 + n16;
-    const float l_row = quad_rows_sum(l[rt]);
+    const float l_row = l[rt][0];
     if (r >= n_rows) continue;
     const float inv = l_row > 0.f ? 1.0f / l_row : 0.f;
     if (n_segs == 1) {
