@@ -7,11 +7,11 @@
 // One workgroup per (kv head, row) serves the row's whole query group.  After a common prologue
 // (q to LDS, new key and value to their page) its waves work on their own: the context is walked
 // in chunks of 256 tokens; with head_dim 64 there are eight waves, wave w takes tokens
-// 64 (w % 4) .. + 63 of every second chunk (starting at chunk w / 4), with head_dim 128 four waves
-// take every chunk (registers).  A wave keeps its own running maximum, sum and output, and asks
-// for the keys and values of its next chunk before it computes the current one.  No barrier
-// inside the loop; the waves' partial results are merged through LDS at the end, always in wave
-// order.
+// 64 (w % 4) .. + 63 of every second chunk (starting at chunk w / 4), with head_dim 128 (registers)
+// and in launches of many workgroups four waves take every chunk.  A wave keeps its own running
+// maximum, sum and output, and asks for the keys and values of its next chunk before it computes
+// the current one.  No barrier inside the loop; the waves' partial results are merged through LDS
+// at the end, always in wave order.
 //
 // Both products run on the matrix cores, transposed: S^T = K Q^T puts one query head in each
 // accumulator column, so a lane's softmax concerns one head only and its eight probabilities of a
@@ -54,8 +54,8 @@ __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
   return r.u;
 }
 
-template <int HD, int GROUP>
-__global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
+template <int HD, int GROUP, int WAVES>
+__global__ void __launch_bounds__(WAVES* kWave, HD == 64 ? 8 / WAVES : 1)
     attention_decode_fused_kernel(const float* __restrict__ partials, int S, size_t pstride,
                                   const uint16_t* __restrict__ qkv, int qkv_stride,
                                   const float2* __restrict__ cos_sin, const int* __restrict__ slots,
@@ -67,7 +67,7 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
   constexpr int KSTEPS = HD / 32;   // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;       // 16-dim tiles of the output
   constexpr int HALF = HD / 2;
-  constexpr int kFusWaves = FusWaves<HD>::N;
+  constexpr int kFusWaves = WAVES;
   constexpr int STRIDE = kFusWaves / 4;   // a wave takes every STRIDE-th chunk
   const int kvh = blockIdx.x, row = blockIdx.y;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -107,8 +107,13 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
     }
     it.rot = cos_sin && item / HALF <= GROUP ? cos_sin[size_t(row) * HALF + item % HALF] : float2{1.0f, 0.0f};
   };
-  Item first;
-  item_request(threadIdx.x < kItems ? threadIdx.x : 0, first);
+  constexpr int kPer = (kItems + kThreads - 1) / kThreads;   // items per thread (past the last: item 0 again, dropped)
+  Item mine_items[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int item = threadIdx.x + i * kThreads;
+    item_request(item < kItems ? item : 0, mine_items[i]);
+  }
 
   const int ctx = ctx_lens[row];
   if (ctx <= 0) {   // a padding row: zeros (from the merge when there are parts), nothing read or stored
@@ -232,11 +237,10 @@ __global__ void __launch_bounds__(FusWaves<HD>::N* kWave)
       vr[size_t(j + HALF) * B] = bb;
     }
   };
-  if (threadIdx.x < kItems) item_finish(threadIdx.x, first);
-  for (int item = threadIdx.x + kThreads; item < kItems; item += kThreads) {
-    Item it;
-    item_request(item, it);
-    item_finish(item, it);
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int item = threadIdx.x + i * kThreads;
+    if (item < kItems) item_finish(item, mine_items[i]);
   }
   __syncthreads();   // q in LDS; the new key and value are stored before any wave of this workgroup loads them
 
@@ -357,8 +361,9 @@ template <int HD, int GROUP>
 int fused_kernel_info(int* out) {
   hipFuncAttributes a;
   int per_cu = 0;
-  if (hipFuncGetAttributes(&a, reinterpret_cast<const void*>(&attention_decode_fused_kernel<HD, GROUP>)) != hipSuccess ||
-      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attention_decode_fused_kernel<HD, GROUP>, FusWaves<HD>::N * kWave, 0) != hipSuccess)
+  constexpr int W = FusWaves<HD>::N;
+  if (hipFuncGetAttributes(&a, reinterpret_cast<const void*>(&attention_decode_fused_kernel<HD, GROUP, W>)) != hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attention_decode_fused_kernel<HD, GROUP, W>, W * kWave, 0) != hipSuccess)
     return -1;
   out[0] = a.numRegs; out[1] = static_cast<int>(a.sharedSizeBytes); out[2] = per_cu; out[3] = FusWaves<HD>::N * kWave;
   return 0;
@@ -375,14 +380,14 @@ int dispatch_fused_info(int group, int* out) {
   }
 }
 
-template <int HD>
+template <int HD, int WAVES>
 int dispatch_fused(int group, dim3 grid, hipStream_t s, const float* partials, int S, size_t pstride, const uint16_t* qkv,
                    int qkv_stride, const float2* cos_sin, const int* slots, uint16_t* kc, uint16_t* vc,
                    const int* tables, int table_stride, const int* row_seq, const int* ctx_lens, int nh, int nkv, int B,
                    float scale, uint16_t* out, int out_stride, int part_chunks, int num_parts, float* scratch) {
 #define KVCM_FUSED(G)                                                                                                   \
   case G:                                                                                                               \
-    attention_decode_fused_kernel<HD, G><<<grid, FusWaves<HD>::N * kWave, 0, s>>>(partials, S, pstride, qkv, qkv_stride,      \
+    attention_decode_fused_kernel<HD, G, WAVES><<<grid, WAVES * kWave, 0, s>>>(partials, S, pstride, qkv, qkv_stride,         \
                                                                            cos_sin, slots, kc, vc, tables, table_stride, \
                                                                            row_seq, ctx_lens, nh, nkv, B, scale, out,   \
                                                                            out_stride, part_chunks, num_parts, scratch); \
@@ -421,6 +426,12 @@ int kvcm_attention_decode_fused_info(int nh, int nkv, int hd, int* out) {
 // one workgroup per CU in all.  Returns the number of parts, *part_chunks chunks of 256 tokens each.
 constexpr int kFusSingleMax = 1024;   // contexts up to this always run as one part
 constexpr int kFusTargetWorkgroups = 256;
+// A workgroup of eight waves has a CU to itself (registers).  From two workgroups per CU on, a
+// launch at head_dim 64 takes workgroups of four waves, each of which walks every chunk: two of
+// them share a CU, and one's trips to memory in the prologue and its merge overlap the other's
+// walk.  Measured inside decode steps of 512-token prompts: 128 rows 2.26 -> 2.16 ms, 256 rows
+// 3.45 -> 3.22 ms, 64 rows (256 workgroups) 1.61 -> 1.63 ms, hence the limit.
+constexpr long long kFusHalfFrom = 512;
 static int fused_parts(int T, int nkv, int max_context, int* part_chunks) {
   const int nchunks = max_context > 0 ? (max_context + kFusChunk - 1) / kFusChunk : 1;
   long long parts = 1;
@@ -474,16 +485,18 @@ int kvcm_attention_decode_fused(const float* partials, int S, const void* qkv, i
                "attention_decode_fused: scratch too small (%lld floats needed)", need);
   const dim3 grid(nkv, T, parts);
   int rc;
-  if (hd == 64)
-    rc = dispatch_fused<64>(nh / nkv, grid, s, partials, S, pstride, static_cast<const uint16_t*>(qkv), qkv_stride,
-                            reinterpret_cast<const float2*>(cos_sin), slots, static_cast<uint16_t*>(kcache),
-                            static_cast<uint16_t*>(vcache), tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale,
-                            static_cast<uint16_t*>(out), out_stride, part_chunks, parts, scratch);
+#define KVCM_FUSED_ARGS                                                                                                  \
+  nh / nkv, grid, s, partials, S, pstride, static_cast<const uint16_t*>(qkv), qkv_stride,                                \
+      reinterpret_cast<const float2*>(cos_sin), slots, static_cast<uint16_t*>(kcache), static_cast<uint16_t*>(vcache),   \
+      tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale, static_cast<uint16_t*>(out), out_stride, part_chunks,  \
+      parts, scratch
+  if (hd == 128)
+    rc = dispatch_fused<128, 4>(KVCM_FUSED_ARGS);
+  else if (static_cast<long long>(nkv) * T * parts >= kFusHalfFrom)
+    rc = dispatch_fused<64, 4>(KVCM_FUSED_ARGS);
   else
-    rc = dispatch_fused<128>(nh / nkv, grid, s, partials, S, pstride, static_cast<const uint16_t*>(qkv), qkv_stride,
-                             reinterpret_cast<const float2*>(cos_sin), slots, static_cast<uint16_t*>(kcache),
-                             static_cast<uint16_t*>(vcache), tables, table_stride, row_seq, ctx_lens, nh, nkv, B, scale,
-                             static_cast<uint16_t*>(out), out_stride, part_chunks, parts, scratch);
+    rc = dispatch_fused<64, 8>(KVCM_FUSED_ARGS);
+#undef KVCM_FUSED_ARGS
   KVCM_REQUIRE(rc == 0, "attention_decode_fused: no kernel for group size %d", nh / nkv);
   if (parts > 1) launch_decode_merge(scratch, ctx_lens, out, out_stride, nh, T, hd, parts, part_chunks * kFusChunk, s);
   return launch_status("attention_decode_fused");

@@ -745,9 +745,9 @@ def test_partitioned_decode_attention_padding_rows_and_far_key(ops):
 # ------------------------------------------ rotation + page write + attention in one launch
 @pytest.mark.parametrize("nh,nkv,hd,B", [(32, 4, 64, 16), (8, 8, 64, 8), (16, 4, 128, 16), (6, 2, 64, 64), (5, 1, 128, 16)])
 @pytest.mark.parametrize("source", ["rows", "partial_sums"])
-def test_fused_decode_attention_equals_rope_write_attend(ops, nh, nkv, hd, B, source):
+def test_fused_decode_attention_equals_rope_write_attend(ops, nh, nkv, hd, B, source, copies=1):
     rng = np.random.default_rng(nh + hd + B)
-    lens = [700, 256, 257, 1, 255, 33, 513, 1024]       # 1..4 chunks, chunk edges, the first token of a sequence
+    lens = [700, 256, 257, 1, 255, 33, 513, 1024] * copies    # 1..4 chunks, chunk edges, the first token of a sequence
     P = _paged_problem(rng, lens, nh, nkv, hd, B, all_rows=False)
     R, W = P["R"], (nh + 2 * nkv) * hd
     pos = (P["ctx"] - 1).astype(np.int32)
@@ -794,6 +794,13 @@ def test_fused_decode_attention_equals_rope_write_attend(ops, nh, nkv, hd, B, so
                                1.0 / math.sqrt(hd), cos_sin=table, slots=_t(slots, torch.int32))
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)                      # the same keys and values reached the pages
     np.testing.assert_allclose(_np(got), _np(want), atol=2 ** -6, rtol=0)        # two kernels, a rounding apart
+
+
+@pytest.mark.parametrize("source", ["rows", "partial_sums"])
+def test_fused_decode_attention_of_many_rows(ops, source):
+    """From 512 workgroups on (rows x kv heads) a launch at head_dim 64 takes workgroups of four waves
+    instead of eight: 64 rows of 8 kv heads, the same contexts as above."""
+    test_fused_decode_attention_equals_rope_write_attend(ops, 16, 8, 64, 16, source, copies=8)
 
 
 @pytest.mark.parametrize("nh,nkv,hd,B", [(8, 2, 64, 16), (6, 2, 128, 32), (32, 4, 64, 16)])
