@@ -14,7 +14,9 @@
 // In the accumulator of S^T a lane holds, for ONE query row (lane % 16), four tokens of each
 // 16-token tile; after exp those registers, rounded to bfloat16 and packed, ARE the B operand of
 // the second product (the order of the reduction index inside a matrix instruction is free as long
-// as both operands agree, so the values are read from LDS in that same token order).  The
+// as both operands agree, so the values are kept in LDS in that same token order: staging puts
+// token 16 a + 4 q + e of a group of 32 at place 8 q + 4 a + e, and a lane's 8 tokens of a step are one
+// 16-byte read; as two 8-byte reads of tokens as they lie they collided in the LDS banks).  The
 // probabilities never touch LDS, a row's maximum lives in one lane, its sum comes from a third
 // product (ones * P^T: the sum of the probabilities as the second product sees them), and the
 // output is stored four dims at a time.
@@ -43,7 +45,6 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 union PFrag {
   uint4 u;
-  uint2 h[2];
   bf16x8 v;
 };
 
@@ -181,7 +182,15 @@ __global__ void __launch_bounds__(kPfThreads, 2)
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
       *reinterpret_cast<u32x4*>(&k_lds[buf][k_p * PIECES + i][k_col * 8]) = pc.k[i];
-      *reinterpret_cast<u32x4*>(&v_lds[buf][v_d + 32 * i][v_g * 8]) = pc.v[i];
+      // tokens 8 g .. 8 g + 7 of the chunk: inside their group of 32 tokens, token 16 a + 4 q + e goes to
+      // place 8 q + 4 a + e, so that the 8 tokens a lane multiplies in one step lie together
+      {
+        const int r0 = (v_g * 8) % 32, grp = (v_g * 8) / 32;
+        const int a = r0 / 16, q0 = (r0 % 16) / 4;
+        uint16_t* dst = &v_lds[buf][v_d + 32 * i][grp * 32 + 4 * a];
+        *reinterpret_cast<uint2*>(dst + 8 * q0) = uint2{pc.v[i][0], pc.v[i][1]};
+        *reinterpret_cast<uint2*>(dst + 8 * (q0 + 1)) = uint2{pc.v[i][2], pc.v[i][3]};
+      }
     }
   };
 
@@ -267,8 +276,7 @@ __global__ void __launch_bounds__(kPfThreads, 2)
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
           PFrag vf;
-          vf.h[0] = *reinterpret_cast<const uint2*>(&v_lds[buf][d * 16 + n16][(2 * c) * 16 + 4 * kq]);
-          vf.h[1] = *reinterpret_cast<const uint2*>(&v_lds[buf][d * 16 + n16][(2 * c + 1) * 16 + 4 * kq]);
+          vf.u = *reinterpret_cast<const uint4*>(&v_lds[buf][d * 16 + n16][c * 32 + 8 * kq]);
 #pragma unroll
           for (int rt = 0; rt < kPfRT; ++rt) o[rt][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][c].v, o[rt][d], 0, 0, 0);
         }
