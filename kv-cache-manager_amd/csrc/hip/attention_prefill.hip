@@ -50,9 +50,12 @@ union PFrag {
 
 constexpr int kPfWaves = 4;
 constexpr int kPfThreads = kPfWaves * kWave;
-constexpr int kPfRT = 2;                         // 16-row tiles per wave
-constexpr int kPfWaveRows = 16 * kPfRT;
-constexpr int kPfRows = kPfWaveRows * kPfWaves;  // query rows per workgroup
+// A wave takes RT tiles of 16 query rows, a workgroup 64 RT rows: two tiles (128 rows) by default, one
+// (64 rows) for launches of little work at head_dim 64, where twice the workgroups, each with fewer
+// registers (four to a CU instead of two), hide one another's waits better than a workgroup's
+// larger share of every staged chunk saves.
+constexpr int kPfMaxRT = 2;
+constexpr int kPfSmallWork = 35 * 256;           // 128-row workgroup chunks (about 35 per CU) up to which hd 64 takes 64-row tiles
 constexpr int kPfChunk = 64;                     // keys per trip
 constexpr int kPfPad = 8;                        // bfloat16 of padding per LDS row (keeps 16-byte alignment)
 constexpr int kPfSeg = 512;                      // keys per segment: a multiple of this, chosen per launch
@@ -76,13 +79,14 @@ __device__ __forceinline__ float quad_rows_max(float v) {
 
 // Two waves per SIMD at least: with that bound the compiler keeps the accumulators of the matrix
 // instructions in ordinary registers (no copies to and from the accumulation registers around the softmax).
-template <int HD>
+template <int HD, int RT>
 __global__ void __launch_bounds__(kPfThreads, 2)
     attention_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                              const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                              const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
                              const int* __restrict__ seq_start, int nh, int nkv, int B, int b_shift, float scale,
                              int seg_len, int max_segs, float* __restrict__ scratch) {
+  constexpr int kPfRT = RT, kPfWaveRows = 16 * RT, kPfRows = kPfWaveRows * kPfWaves;   // tiles per wave, rows per wave and workgroup
   constexpr int KSTEPS = HD / 32;                          // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;                              // 16-dim tiles of the output
   constexpr int PIECES = kPfChunk * HD / 8 / kPfThreads;   // 16-byte pieces of a chunk per thread (keys; as many of values)
@@ -338,14 +342,14 @@ template <int HD>
 __global__ void __launch_bounds__(256)
     attention_prefill_merge_kernel(const float* __restrict__ scratch, uint16_t* __restrict__ out, int out_stride,
                                    const int* __restrict__ run_start, const int* __restrict__ seq_start, int nh,
-                                   int seg_len, int max_segs) {
+                                   int seg_len, int max_segs, int tile_rows) {
   const int seq = blockIdx.y, head = blockIdx.z;
   const int row0 = run_start[seq], n_rows = run_start[seq + 1] - row0;
   constexpr int PER_ROW = HD / 4;
   const int r = blockIdx.x * (256 / PER_ROW) + threadIdx.x / PER_ROW, piece = threadIdx.x % PER_ROW;
   if (r >= n_rows) return;
-  const int tile = r / kPfRows;
-  const int tile_last_pos = seq_start[seq] + min((tile + 1) * kPfRows, n_rows) - 1;
+  const int tile = r / tile_rows;
+  const int tile_last_pos = seq_start[seq] + min((tile + 1) * tile_rows, n_rows) - 1;
   const int n_segs = tile_last_pos / seg_len + 1;
   if (n_segs == 1) return;   // stored directly
   const float* base = scratch + (size_t(row0 + r) * nh + head) * max_segs * (HD + 4);
@@ -378,21 +382,40 @@ int kvcm_attention_prefill_supported(int nh, int nkv, int hd, int B) {
   return nkv > 0 && nh % nkv == 0 && (hd == 64 || hd == 128) && B >= 8 && (B & (B - 1)) == 0;
 }
 
-// Keys per segment of a launch: 512 while that gives the chip fewer than kPfFill workgroups,
-// longer (in multiples of 512) when tiles x heads x sequences already fill it, since every segment
-// beyond the first costs a partial result per row and head in scratch.
-int kvcm_attention_prefill_segment(int max_run, int S, int nh, int max_context) {
-  if (max_run <= 0 || S <= 0 || nh <= 0 || max_context <= 0) return kPfSeg;
-  const long long base = static_cast<long long>((max_run + kPfRows - 1) / kPfRows) * nh * S;
+// How a launch is cut: query rows per workgroup and keys per segment.  Rows: 128, or 64 at head_dim 64
+// when the launch is small (T rows that see about max_context - max_run / 2 keys each, counted in
+// chunks of 128-row workgroups).  Keys per segment: 512 while that gives the chip fewer than kPfFill
+// workgroups, longer (in multiples of 512) when tiles x heads x sequences already fill it, since
+// every segment beyond the first costs a partial result per row and head in scratch.
+struct PfPlan { int tile_rows, seg_len; };
+static PfPlan pf_plan(int T, int nh, int hd, int max_context, int max_run, int S) {
+  PfPlan p{64 * kPfMaxRT, kPfSeg};
+  if (max_run <= 0 || S <= 0 || nh <= 0 || max_context <= 0) return p;
+  if (T < max_run) T = max_run;
+  const double seen = max_context - 0.5 * max_run > 64.0 ? max_context - 0.5 * max_run : 64.0;
+  const double work = double(T) / 128.0 * (seen / kPfChunk) * nh;
+  if (hd == 64 && work <= kPfSmallWork) p.tile_rows = 64;
+  const long long base = static_cast<long long>((max_run + p.tile_rows - 1) / p.tile_rows) * nh * S;
   const long long want = (kPfFill + base - 1) / base;
   long long len = (max_context + want - 1) / want;
   len = (len + kPfSeg - 1) / kPfSeg * kPfSeg;
-  return static_cast<int>(len < kPfSeg ? kPfSeg : len > kPfSegMax ? kPfSegMax : len);
+  p.seg_len = static_cast<int>(len < kPfSeg ? kPfSeg : len > kPfSegMax ? kPfSegMax : len);
+  return p;
+}
+
+// Keys per segment that a launch of these sizes cuts contexts into (T: rows in all).
+int kvcm_attention_prefill_segment(int T, int nh, int hd, int max_context, int max_run, int S) {
+  return pf_plan(T, nh, hd, max_context, max_run, S).seg_len;
+}
+
+// Query rows per workgroup of such a launch.
+int kvcm_attention_prefill_tile_rows(int T, int nh, int hd, int max_context, int max_run, int S) {
+  return pf_plan(T, nh, hd, max_context, max_run, S).tile_rows;
 }
 
 // Floats of scratch a launch needs: none while no row's context exceeds one segment.
 long long kvcm_attention_prefill_scratch(int T, int nh, int hd, int max_context, int max_run, int S) {
-  const int seg_len = kvcm_attention_prefill_segment(max_run, S, nh, max_context);
+  const int seg_len = pf_plan(T, nh, hd, max_context, max_run, S).seg_len;
   const long long segs = (max_context + seg_len - 1) / seg_len;
   return segs <= 1 ? 0 : static_cast<long long>(T) * nh * segs * (hd + 4);
 }
@@ -415,14 +438,15 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(vcache) % 16 == 0, "attention_prefill: operands must be 16-byte aligned");
   KVCM_REQUIRE(out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0, "attention_prefill: output must be 8-byte aligned");
-  const int seg_len = kvcm_attention_prefill_segment(max_run, S, nh, max_context);
+  const PfPlan plan = pf_plan(T, nh, hd, max_context, max_run, S);
+  const int seg_len = plan.seg_len;
   const int max_segs = (max_context + seg_len - 1) / seg_len;
   const long long need = kvcm_attention_prefill_scratch(T, nh, hd, max_context, max_run, S);
   KVCM_REQUIRE(need == 0 || (scratch && scratch_floats >= need && reinterpret_cast<uintptr_t>(scratch) % 16 == 0),
                "attention_prefill: scratch too small (%lld floats needed)", need);
   int b_shift = 0;
   while ((1 << b_shift) < B) ++b_shift;
-  const long long units = static_cast<long long>((max_run + kPfRows - 1) / kPfRows) * max_segs * nh;
+  const long long units = static_cast<long long>((max_run + plan.tile_rows - 1) / plan.tile_rows) * max_segs * nh;
   KVCM_REQUIRE(units < (1ll << 31), "attention_prefill: too many workgroups");
   const dim3 grid(static_cast<unsigned>(units), S, 1);
   const size_t page_bytes = sizeof(int) * size_t(seg_len / B + 2);   // the pages of one segment
@@ -430,20 +454,21 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
                  *vc = static_cast<const uint16_t*>(vcache);
   const int merge_rows = 256 / (hd / 4);   // rows per workgroup of the merge
   const dim3 mgrid((max_run + merge_rows - 1) / merge_rows, S, nh);
-  if (hd == 64) {
-    attention_prefill_kernel<64><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
-                                                             tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale,
-                                                             seg_len, max_segs, scratch);
-    if (max_segs > 1)
+#define KVCM_PF(HD, RT)                                                                                                        \
+  attention_prefill_kernel<HD, RT><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, \
+                                                                        kc, vc, tables, table_stride, run_start, seq_start,  \
+                                                                        nh, nkv, B, b_shift, scale, seg_len, max_segs, scratch)
+  if (hd == 64 && plan.tile_rows == 64) KVCM_PF(64, 1);
+  else if (hd == 64) KVCM_PF(64, 2);
+  else KVCM_PF(128, 2);
+#undef KVCM_PF
+  if (max_segs > 1) {
+    if (hd == 64)
       attention_prefill_merge_kernel<64><<<mgrid, 256, 0, s>>>(scratch, static_cast<uint16_t*>(out), out_stride, run_start,
-                                                              seq_start, nh, seg_len, max_segs);
-  } else {
-    attention_prefill_kernel<128><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc,
-                                                              tables, table_stride, run_start, seq_start, nh, nkv, B, b_shift, scale,
-                                                              seg_len, max_segs, scratch);
-    if (max_segs > 1)
+                                                              seq_start, nh, seg_len, max_segs, plan.tile_rows);
+    else
       attention_prefill_merge_kernel<128><<<mgrid, 256, 0, s>>>(scratch, static_cast<uint16_t*>(out), out_stride, run_start,
-                                                               seq_start, nh, seg_len, max_segs);
+                                                               seq_start, nh, seg_len, max_segs, plan.tile_rows);
   }
   return launch_status("attention_prefill");
 }

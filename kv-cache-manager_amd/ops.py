@@ -58,7 +58,9 @@ def _declare(lib):
     lib.kvcm_attention_prefill_scratch.restype = C.c_longlong
     lib.kvcm_attention_prefill_scratch.argtypes = [i, i, i, i, i, i]
     lib.kvcm_attention_prefill_segment.restype = i
-    lib.kvcm_attention_prefill_segment.argtypes = [i, i, i, i]
+    lib.kvcm_attention_prefill_segment.argtypes = [i, i, i, i, i, i]
+    lib.kvcm_attention_prefill_tile_rows.restype = i
+    lib.kvcm_attention_prefill_tile_rows.argtypes = [i, i, i, i, i, i]
     lib.kvcm_attention_decode_scratch.restype = C.c_longlong
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
@@ -448,9 +450,14 @@ def attention_prefill_scratch(rows, nh, hd, max_context, max_run, num_seqs):
     return int(lib().kvcm_attention_prefill_scratch(rows, nh, hd, max_context, max_run, num_seqs))
 
 
-def attention_prefill_segment(max_run, num_seqs, nh, max_context):
+def attention_prefill_segment(rows, nh, hd, max_context, max_run, num_seqs):
     """Keys per segment that a launch of these sizes cuts contexts into."""
-    return int(lib().kvcm_attention_prefill_segment(max_run, num_seqs, nh, max_context))
+    return int(lib().kvcm_attention_prefill_segment(rows, nh, hd, max_context, max_run, num_seqs))
+
+
+def attention_prefill_tile_rows(rows, nh, hd, max_context, max_run, num_seqs):
+    """Query rows per workgroup of a launch of these sizes (128; 64 for small launches at head_dim 64)."""
+    return int(lib().kvcm_attention_prefill_tile_rows(rows, nh, hd, max_context, max_run, num_seqs))
 
 
 def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, seq_start, num_seqs, max_run, nh, nkv, hd,

@@ -963,9 +963,10 @@ def test_prefill_attention_long_prompt(ops):
     runs = [(0, 1500), (1000, 300)]
     P = _runs_problem(rng, runs, nh, nkv, hd, B)
     got = _run_prefill(ops, P, runs, nh, nkv, hd)
-    # a launch this narrow cuts contexts into segments of 512 keys that are merged afterwards: rows
-    # around the cuts, a tile that a cut goes through (the second run starts at 1000), tile edges
-    assert ops.attention_prefill_segment(1500, 2, nh, 1500) == 512
+    # a launch this narrow cuts contexts into segments of keys that are merged afterwards: rows
+    # around the cuts (and around multiples of 512, where cuts lie in other launches), a tile that a cut goes through (the second run starts at 1000), tile edges
+    # (little work at head_dim 64: workgroups of 64 rows, and with twice the workgroups segments of 1,024 keys)
+    assert ops.attention_prefill_tile_rows(1800, nh, hd, 1500, 1500, 2) == 64 and ops.attention_prefill_segment(1800, nh, hd, 1500, 1500, 2) == 1024
     rows = [0, 1, 63, 64, 511, 512, 513, 700, 1023, 1024, 1025, 1151, 1152, 1499, 1500, 1523, 1524, 1535, 1536, 1627, 1628, 1799]
     ref = np.zeros((len(rows), nh, hd))
     for k, r in enumerate(rows):
@@ -999,31 +1000,30 @@ def test_prefill_attention_three_segments_far_key(ops):
 
 def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops):
     """The wider a launch (tiles x heads x sequences), the longer its segments of keys; one that fills
-    the chip by itself is not cut at all.  Here three runs give segments of 1,024 keys: rows on both
-    sides of that cut, and a far key of the first segment."""
+    the chip by itself is not cut at all.  Here 64 heads over a long context give workgroups of 128
+    rows and segments of 2,048 keys: rows on both sides of the cut at 6,144, and a far key of the
+    first segment."""
     rng = np.random.default_rng(53)
-    nh, nkv, hd, B = 32, 4, 64, 16
-    runs = [(900 + 13 * i, 384) for i in range(3)]
-    assert ops.attention_prefill_segment(384, len(runs), nh, max(s + n for s, n in runs)) == 1024
-    assert ops.attention_prefill_segment(300, 2, nh, 2600) == 1024 and ops.attention_prefill_segment(2048, 1, 32, 2048) == 2048
-    assert ops.attention_prefill_segment(4096, 1, 32, 32768) == 16384 and ops.attention_prefill_segment(128, 1, 4, 32768) == 512
+    nh, nkv, hd, B = 64, 8, 64, 16
+    runs = [(6000, 256)]
+    assert ops.attention_prefill_tile_rows(256, nh, hd, 6256, 256, 1) == 128 and ops.attention_prefill_segment(256, nh, hd, 6256, 256, 1) == 2048
+    assert ops.attention_prefill_tile_rows(2048, 32, 64, 2048, 2048, 1) == 64 and ops.attention_prefill_segment(2048, 32, 64, 2048, 2048, 1) == 2048
+    assert ops.attention_prefill_tile_rows(3072, 32, 64, 3072, 3072, 1) == 128 and ops.attention_prefill_tile_rows(2048, 32, 128, 2048, 2048, 1) == 128
+    assert ops.attention_prefill_segment(4096, 32, 64, 32768, 4096, 1) == 16384 and ops.attention_prefill_segment(128, 4, 128, 32768, 128, 1) == 512
     P = _paged_problem(rng, [s + n for s, n in runs], nh, nkv, hd, B, all_rows=False)
     R = sum(n for _, n in runs)
     Q = _bf16_grid(rng.normal(size=(R, nh, hd)))
-    far, seq, head = 40, 1, 9                                   # kv head 1
-    row_lo = sum(n for _, n in runs[:seq])
-    Q[row_lo + 100:row_lo + 300, head] = 0.0
-    Q[row_lo + 100:row_lo + 300, head, 3] = 30.0
+    far, seq, head = 40, 0, 9                                   # kv head 1
+    Q[100:, head] = 0.0
+    Q[100:, head, 3] = 30.0
     kvec = np.zeros(hd)
     kvec[3] = 30.0
     P["Kl"][seq][far, 1] = kvec
     P["Kc"][P["tables"][seq, far // B], 1, far % B] = kvec
     P["Q"], P["R"] = Q, R
     got = _run_prefill(ops, P, runs, nh, nkv, hd, scale=1.0)
-    np.testing.assert_allclose(got[row_lo + 100:row_lo + 300, head],
-                               np.broadcast_to(P["Vl"][seq][far, 1], (200, hd)), atol=2e-2)
-    for s, r in ((0, 0), (0, 123), (0, 124), (0, 383), (1, 110), (1, 111), (2, 97), (2, 98), (2, 383), (1, 128)):
-        pos = runs[s][0] + r                                   # the cut lies between positions 1023 and 1024
-        row = sum(n for _, n in runs[:s]) + r
-        ref = plain.attention(Q[row:row + 1], P["Kl"][s][:pos + 1], P["Vl"][s][:pos + 1], [pos], np.arange(pos + 1), 1.0)[0]
-        np.testing.assert_allclose(got[row], ref, atol=1e-2, rtol=0, err_msg=f"sequence {s} row {r}")
+    np.testing.assert_allclose(got[100:, head], np.broadcast_to(P["Vl"][seq][far, 1], (R - 100, hd)), atol=2e-2)
+    for r in (0, 127, 128, 143, 144, 145, 255):                # the cut lies between positions 6143 and 6144
+        pos = runs[0][0] + r
+        ref = plain.attention(Q[r:r + 1], P["Kl"][0][:pos + 1], P["Vl"][0][:pos + 1], [pos], np.arange(pos + 1), 1.0)[0]
+        np.testing.assert_allclose(got[r], ref, atol=1e-2, rtol=0, err_msg=f"row {r}")
