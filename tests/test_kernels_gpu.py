@@ -924,7 +924,7 @@ def _runs_problem(rng, runs, nh, nkv, hd, B):
 
 
 @pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (4, 4, 128), (6, 1, 64), (32, 4, 64)])
-@pytest.mark.parametrize("B", [8, 16, 64])
+@pytest.mark.parametrize("B", [8, 16, 64, 128])
 def test_prefill_attention_runs_anywhere(ops, nh, nkv, hd, B):
     rng = np.random.default_rng(nh + hd + B)
     runs = [(0, 130), (0, 1), (77, 2), (200, 1), (15, 64), (63, 65), (0, 16), (31, 17)]
@@ -998,13 +998,14 @@ def test_prefill_attention_three_segments_far_key(ops):
     np.testing.assert_allclose(got[rows], ref, atol=1e-2, rtol=0)
 
 
-def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops):
+@pytest.mark.parametrize("B", [16, 8, 128])
+def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops, B):
     """The wider a launch (tiles x heads x sequences), the longer its segments of keys; one that fills
     the chip by itself is not cut at all.  Here 64 heads over a long context give workgroups of 128
     rows and segments of 2,048 keys: rows on both sides of the cut at 6,144, and a far key of the
     first segment."""
     rng = np.random.default_rng(53)
-    nh, nkv, hd, B = 64, 8, 64, 16
+    nh, nkv, hd = 64, 8, 64
     runs = [(6000, 256)]
     assert ops.attention_prefill_tile_rows(256, nh, hd, 6256, 256, 1) == 128 and ops.attention_prefill_segment(256, nh, hd, 6256, 256, 1) == 2048
     assert ops.attention_prefill_tile_rows(2048, 32, 64, 2048, 2048, 1) == 64 and ops.attention_prefill_segment(2048, 32, 64, 2048, 2048, 1) == 2048
