@@ -67,8 +67,11 @@ class LlamaConfig:
             problems.append(f"num_attention_heads {nh} must be a multiple of num_key_value_heads {nkv!r}")
         if not isinstance(hd, int) or hd <= 0 or hd % 2:
             problems.append(f"head_dim {hd!r} must be a positive even integer (rotary pairs)")
-        if raw.get("rope_scaling") not in (None, {}):
-            problems.append("rope_scaling is not supported (only plain rotary positions)")
+        scaling = raw.get("rope_scaling")
+        plain_rotary = scaling in (None, {}) or (isinstance(scaling, dict) and set(scaling) <= {"rope_type", "type"}
+                                                 and all(v == "default" for v in scaling.values()))
+        if not plain_rotary:
+            problems.append(f"rope_scaling {scaling!r} is not supported (only plain rotary positions)")
         for k in ("attention_bias", "mlp_bias"):
             if raw.get(k):
                 problems.append(f"{k}=true is not supported (projections have no bias)")

@@ -62,6 +62,13 @@ def test_config_refuses_what_the_engine_has_not(patch, fragment):
         LlamaConfig.from_dict({**H.TINY_A, **patch})
 
 
+def test_config_takes_rope_scaling_that_says_no_scaling():
+    for value in (None, {}, {"rope_type": "default"}, {"type": "default"}):
+        assert LlamaConfig.from_dict({**H.TINY_A, "rope_scaling": value}).rope_theta == H.TINY_A.get("rope_theta", 10000.0)
+    with pytest.raises(ConfigError, match="rope_scaling"):
+        LlamaConfig.from_dict({**H.TINY_A, "rope_scaling": {"rope_type": "llama3", "factor": 8.0}})
+
+
 def test_config_lists_every_problem_at_once():
     with pytest.raises(ConfigError) as e:
         LlamaConfig.from_dict({**H.TINY_A, "head_dim": 7, "attention_bias": True, "hidden_act": "relu"})
