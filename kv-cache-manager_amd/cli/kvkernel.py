@@ -15,6 +15,14 @@ With --graph (not in the reference) the timed calls are replays of one captured 
 holds ``--iters`` calls, which takes the host's launch cost out of the figure.
 Columns: registers per lane, LDS per workgroup, workgroups per CU, occupancy (resident waves as a
 percentage of a CU's 32 wave slots), workgroups launched and how many rounds of the chip they make.
+
+  --prefill 2048,1024,512@1536  [--seqs 1]        (not in the reference)
+
+times the tiled prompt attention instead: each item is a portion of TOKENS query rows that starts
+at position START of its sequence (default 0), ``--seqs`` such sequences in one call; random keys
+and values behind a shuffled block table.  TFLOP/s counts the causal work, 4 * head_dim * heads *
+(keys each row sees), against the bf16 matrix-core peak; the last columns say how the launch was
+cut (query rows per workgroup, keys per segment).
 """
 import sys
 
@@ -23,6 +31,7 @@ import numpy as np
 from .args import Args
 
 PEAK_GBS = 8000.0      # MI355X HBM3E
+PEAK_BF16_TFLOPS = 2500.0
 WAVE_SLOTS_PER_CU = 32
 
 
@@ -36,7 +45,10 @@ def main(argv=None):
     heads, kvh, hd = a.i32("heads", 32), a.i32("kv-heads", 4), a.i32("head-dim", 64)
     iters, out_csv = a.i32("iters", 100), a.str("out", "")
     use_graph = a.flag("graph")
+    prefill, seqs = a.str("prefill", ""), a.i32("seqs", 1)
     a.warn_unused()
+    if prefill:
+        return _prefill(prefill, seqs, blocks, heads, kvh, hd, iters, out_csv, use_graph)
 
     import torch
     from .. import ops
@@ -132,6 +144,77 @@ def main(argv=None):
                             f.write("%d,%d,%d,%s,%.3f,%.2f,%.2f,%d,%d,%d,%.1f,%d,%.3f\n" % (
                                 B, batch, ctx, name, us, gbs, 100 * gbs / PEAK_GBS, info["regs"], info["lds_bytes"],
                                 info["workgroups_per_cu"], occ, wgs, rounds))
+    if f:
+        f.close()
+    return 0
+
+
+def _prefill(spec, seqs, blocks, heads, kvh, hd, iters, out_csv, use_graph):
+    import torch
+    from .. import ops
+    ops.lib()
+    dev = torch.device("cuda:0")
+    bf16 = torch.bfloat16
+    items = []
+    for part in spec.split(","):
+        tokens, _, start = part.partition("@")
+        items.append((int(tokens), int(start or 0)))
+    f = open(out_csv, "w") if out_csv else None
+    if f:
+        f.write("block_size,seqs,tokens,start,us,tflops,pct_peak,tile_rows,segment\n")
+    print("%5s %5s %7s %7s %10s %9s %7s %5s %8s" % ("B", "seqs", "tokens", "start", "us/call", "TFLOP/s", "%peak", "rows", "segment"))
+    gen = torch.Generator(device=dev).manual_seed(0)
+    for B in blocks:
+        if not ops.attention_prefill_supported(heads, kvh, hd, bf16, B):
+            print("%5d %s" % (B, "unsupported"))
+            continue
+        for tokens, start in items:
+            ctx = start + tokens
+            mb = (ctx + B - 1) // B
+            K = torch.randn(seqs * mb, kvh, B, hd, device=dev, generator=gen).to(bf16)
+            V = torch.randn(seqs * mb, kvh, hd, B, device=dev, generator=gen).to(bf16)
+            Q = torch.randn(seqs * tokens, (heads + 2 * kvh) * hd, device=dev, generator=gen).to(bf16)
+            O = torch.zeros(seqs * tokens, heads * hd, dtype=bf16, device=dev)
+            tab = torch.randperm(seqs * mb, device=dev, generator=gen).to(torch.int32)
+            run_start = torch.arange(0, seqs * tokens + 1, tokens, dtype=torch.int32, device=dev)
+            seq_start = torch.full((seqs,), start, dtype=torch.int32, device=dev)
+            need = ops.attention_prefill_scratch(seqs * tokens, heads, hd, ctx, tokens, seqs)
+            scratch = torch.zeros(max(need, 4), dtype=torch.float32, device=dev)
+
+            def call():
+                ops.attention_prefill(Q, O, K, V, tab, mb, run_start, seq_start, seqs, tokens, heads, kvh, hd,
+                                      1.0 / hd ** 0.5, rows=seqs * tokens, max_context=ctx, scratch=scratch)
+
+            for _ in range(5):
+                call()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            if use_graph:
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(iters):
+                        call()
+                graph.replay()
+                torch.cuda.synchronize()
+                e0.record()
+                graph.replay()
+                e1.record()
+            else:
+                e0.record()
+                for _ in range(iters):
+                    call()
+                e1.record()
+            e1.synchronize()
+            us = 1e3 * e0.elapsed_time(e1) / iters
+            seen = seqs * (tokens * start + tokens * (tokens + 1) / 2.0)
+            tflops = 4.0 * hd * heads * seen / (us * 1e-6) / 1e12
+            rows = ops.attention_prefill_tile_rows(seqs * tokens, heads, hd, ctx, tokens, seqs)
+            seg = ops.attention_prefill_segment(seqs * tokens, heads, hd, ctx, tokens, seqs)
+            print("%5d %5d %7d %7d %10.2f %9.1f %6.1f%% %5d %8d" % (B, seqs, tokens, start, us, tflops,
+                                                                  100 * tflops / PEAK_BF16_TFLOPS, rows, seg))
+            if f:
+                f.write("%d,%d,%d,%d,%.3f,%.2f,%.2f,%d,%d\n" % (B, seqs, tokens, start, us, tflops,
+                                                               100 * tflops / PEAK_BF16_TFLOPS, rows, seg))
     if f:
         f.close()
     return 0
