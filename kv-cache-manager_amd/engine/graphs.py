@@ -30,8 +30,7 @@ def _no_collection():
     there may destroy device objects of an engine that is no longer used (its graphs, their memory
     pools), and releasing device memory during a capture ends the process."""
     was_enabled = gc.isenabled()
-    gc.collect()
-    gc.disable()
+    gc.disable()   # (torch.cuda.graph collects once itself before the capture begins)
     try:
         yield
     finally:
