@@ -4,7 +4,8 @@
 // (src/cuda/paged_attention.cu:50-183, docs/design.md:113-114): every row re-reads all its keys.
 //
 // Here a workgroup takes 128 query rows of one head, each of its four waves 32 of them (two
-// 16-row tiles), and walks the keys 64 at a time with a running maximum (no score buffer).  A
+// 16-row tiles; in small launches at head_dim 64: 64 rows, one tile per wave), and walks the keys
+// 64 at a time with a running maximum (no score buffer).  A
 // chunk of keys and values is staged in LDS once per workgroup, double-buffered: the next chunk's
 // global loads are in flight while the current one is multiplied.
 //
@@ -26,9 +27,9 @@
 //
 // While tiles x heads x sequences give fewer than two workgroups per CU, contexts are cut into
 // segments of keys (multiples of 512, at absolute multiples of their length) that run as workgroups
-// of their own: without that a short portion behind a long context leaves most of the chip idle.  A tile whose rows see
-// one segment stores its result; otherwise every segment leaves (o / l, m, l) per row in scratch
-// and a second kernel merges them in segment order.
+// of their own: without that a short portion behind a long context leaves most of the chip idle.
+// A tile whose rows see one segment stores its result; otherwise every segment leaves
+// (o / l, m, l) per row in scratch and a second kernel merges them in segment order.
 #include <cfloat>
 
 #include "common.h"
