@@ -113,11 +113,14 @@ class DecodeGraphs:
         runner._upload_pending = False
         graph = self.graphs.get((bucket, bound))
         if graph is None:
-            self._forward(layout, bucket, bound)          # eager once: creates every work buffer
+            # eager once: creates every work buffer, and its result is this step's result (a capture
+            # runs nothing, so the sampled ids stay where the eager pass left them)
+            self._forward(layout, bucket, bound)
             torch.cuda.current_stream().synchronize()
             graph = torch.cuda.CUDAGraph()
             with _no_collection(), torch.cuda.graph(graph):
                 self._forward(layout, bucket, bound)
             self.graphs[(bucket, bound)] = graph
+            return s.download(n)
         graph.replay()
         return s.download(n)
