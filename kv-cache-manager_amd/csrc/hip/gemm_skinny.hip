@@ -15,7 +15,10 @@
 // and the 8 up rows of the same columns, and stores act = round(round(silu(g)) * u) [M, I]
 // directly (g, u rounded to the storage type first, exactly what the separate SwiGLU kernel
 // computes from the stored product).  Unsplit only.
+#include <mutex>
+
 #include "common.h"
+#include "kvcm_hip.h"
 
 namespace kvcm {
 
@@ -449,6 +452,59 @@ int kvcm_reduce_store(const float* partials, void* out, int out_dtype, int M, in
   else if (out_dtype == kF32) reduce_store_kernel<float><<<blocks, 256, 0, st>>>(partials, static_cast<float*>(out), M, N, ldo, S);
   else KVCM_REQUIRE(false, "reduce_store: unknown output dtype %d", out_dtype);
   return launch_status("reduce_store");
+}
+
+// ---- the product for callers that cannot allocate -------------------------------------------
+// Partial sums of a split product, for kvcm_gemm_skinny_noalloc: part of the library's device
+// image, one copy per GPU at that GPU's own address.  Host code never passes the array's name to a
+// kernel (on the host it is a stand-in, not a device address): it passes the address that
+// hipGetSymbolAddress gave for the current device.
+constexpr long long kNoAllocFloats = 2ll << 20;
+static __device__ __align__(256) float scratch[kNoAllocFloats];
+
+constexpr int kMaxDevices = 64;
+static float* g_noalloc_ptr[kMaxDevices];
+static std::mutex g_noalloc_lock;
+
+// The current device's copy of the array; looked up once per device, with that device current.
+static int noalloc_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("gemm_skinny_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    return -2;
+  }
+  KVCM_REQUIRE(dev >= 0 && dev < kMaxDevices, "gemm_skinny_noalloc: device %d beyond the %d this library keeps track of", dev, kMaxDevices);
+  std::lock_guard<std::mutex> hold(g_noalloc_lock);
+  if (g_noalloc_ptr[dev] == nullptr) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("gemm_skinny_noalloc: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+      return -2;
+    }
+    g_noalloc_ptr[dev] = p;
+  }
+  *out = g_noalloc_ptr[dev];
+  return 0;
+}
+
+long long kvcm_gemm_skinny_noalloc_capacity() { return kNoAllocFloats; }
+
+int kvcm_gemm_skinny_noalloc(const void* X, const void* W, void* out, int out_dtype, int M, int N, int K, int ldx,
+                             int ldw, int ldo, hipStream_t st) {
+  const int S = kvcm_gemm_skinny_splits(M, N, K);
+  KVCM_REQUIRE(S > 0, "gemm_skinny_noalloc: unsupported shape M=%d N=%d K=%d", M, N, K);
+  KVCM_REQUIRE(out != nullptr && ldo >= N, "gemm_skinny_noalloc: missing output buffer or leading dimension below N");
+  if (S == 1) return kvcm_gemm_skinny(X, W, nullptr, out, out_dtype, M, N, K, ldx, ldw, ldo, 1, st);
+  const long long need = (long long)S * M * N;
+  KVCM_REQUIRE(need <= kNoAllocFloats,
+               "gemm_skinny_noalloc: M=%d N=%d K=%d needs %lld floats of partial sums (%d slices), the built-in array holds %lld",
+               M, N, K, need, S, kNoAllocFloats);
+  float* partials = nullptr;
+  if (int rc = noalloc_scratch(&partials)) return rc;
+  if (int rc = kvcm_gemm_skinny(X, W, partials, out, out_dtype, M, N, K, ldx, ldw, ldo, S, st)) return rc;
+  return kvcm_reduce_store(partials, out, out_dtype, M, N, ldo, S, st);
 }
 
 }  // extern "C"
