@@ -26,6 +26,7 @@ def main(argv=None):
         time_limit = a.f64("time-limit", 1e9)
         temperature, sampler_seed = a.f64("temperature", 0.0), a.i64("sampler-seed", 0)
         eng = make_engine(a, ec)
+        wl.max_seq_len = eng.config.max_seq_len      # as built: within the model's own range
         a.warn_unused()
         wl.vocab = eng.model.spec.vocab_size
         import torch

@@ -22,7 +22,9 @@ class EngineConfig:
     attn: str = "auto"               # "v1" | "v2" | "auto"
     max_logit_rows: int = 0          # 0: max(max_num_seqs, 512)
     dtype: str = "bfloat16"          # "bfloat16" | "float32"
-    use_graphs: bool = True          # replay decode-only steps from captured HIP graphs
+    use_graphs: bool = True          # replay decode-only steps from captured HIP graphs (models whose parts are all capturable)
+    use_programs: bool = True        # replay other step shapes from natively recorded launch lists (same condition)
+    beyond_max_position: bool = False  # False: max_seq_len is cut down to the model's max_position_embeddings (with a notice)
 
     def validate(self):
         if self.policy not in ("paged", "contiguous"):

@@ -1,7 +1,9 @@
 """From a model folder (or a configuration with tensors in memory) to a runner that can step:
 config.json -> architecture (registry) -> parts -> weights by name -> cache groups and pages ->
 work buffers.  Pool sizing and limits follow the reference (src/engine/engine.cpp:19-45)."""
+import dataclasses
 import os
+import sys
 from typing import Dict, Optional
 
 import torch
@@ -39,6 +41,19 @@ def read_model_config(model_dir):
     return arch, arch.config_class.from_dict(raw)
 
 
+def within_max_position(ec: EngineConfig, max_position: int) -> EngineConfig:
+    """The model's own length limit against the engine's.  The reference carries max_pos in its
+    weights header and never looks at it (src/model/weights.cpp:24-40): positions are rotated on the
+    fly, so any length computes.  Here the engine's max_seq_len is cut down to the model's
+    max_position (0: the architecture states none), with one line on stderr, unless the option
+    ``beyond_max_position`` says that running past it is meant (replay of given traces does)."""
+    if max_position <= 0 or ec.max_seq_len <= max_position or ec.beyond_max_position:
+        return ec
+    print(f"[kvcm] max_seq_len {ec.max_seq_len} exceeds the model's max_position_embeddings {max_position}: "
+          f"sequences end at {max_position} tokens (EngineConfig.beyond_max_position=True lifts this)", file=sys.stderr, flush=True)
+    return dataclasses.replace(ec, max_seq_len=max_position)
+
+
 def build_runner(model_dir: Optional[str] = None, engine_config: Optional[EngineConfig] = None, *,
                  architecture: Optional[str] = None, model_config=None, tensors: Optional[Dict[str, torch.Tensor]] = None,
                  device="cuda:0"):
@@ -57,6 +72,7 @@ def build_runner(model_dir: Optional[str] = None, engine_config: Optional[Engine
             raise ValueError("give a model folder, or architecture + model_config + tensors")
         arch, cfg, source = ARCHITECTURES.get(architecture), model_config, DictSource(tensors)
     spec = arch.build_spec(cfg)
+    ec = within_max_position(ec, spec.max_position)
     model = Model(spec, BuildContext(dtype, dev, spec.hidden_size, ec.block_size, ops))
     try:
         weight_bytes = load_weights(model, source, dtype, dev)

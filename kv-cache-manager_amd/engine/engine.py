@@ -36,8 +36,12 @@ class Engine:
         self._next_id = 0
         self._score_id = -1
         self._t0 = time.perf_counter()
+        self.config = self.runner.engine_config      # as built (max_seq_len within the model's range)
+        # Recorded steps (graphs) replay a fixed launch sequence: only for models whose parts all
+        # declare that their launches depend on the step's shape alone (Part.capturable).
         self.decode_graphs = None
-        if self.config.use_graphs:
+        self.programs = None
+        if self.config.use_graphs and self.model.capturable:
             from .graphs import DecodeGraphs
             self.decode_graphs = DecodeGraphs(self)
 

@@ -29,7 +29,8 @@ class TraceReplayer:
         span = max(pages * block_size, block_size)
         ec = EngineConfig(policy="paged", block_size=block_size, max_seq_len=span, num_blocks=max(pages, 1),
                           watermark_blocks=0, max_num_seqs=max_live, max_batched_tokens=span,
-                          max_logit_rows=min(span, 1024), dtype=dtype, attn=attn, use_graphs=False)
+                          max_logit_rows=min(span, 1024), dtype=dtype, attn=attn, use_graphs=False,
+                          beyond_max_position=True)     # a trace's lengths are given, not generated
         self.runner, self.core, self.model, self.model_config = build_runner(model_dir, ec, device=device)
         self.vocab_size = self.model.spec.vocab_size
         self._ids = {}          # external id -> integer id

@@ -14,7 +14,7 @@ import torch
 
 from ..cache.manager import BatchLayout, CacheGroupSpec, HostCore
 from ..cache.storage import KVStorage, StateStorage, bytes_per_block
-from ..parts.base import BuildContext, KVCacheNeed, StateNeed
+from ..parts.base import BuildContext, KVCacheNeed, StateNeed, StepView
 from ..parts.model import Model
 
 
@@ -35,6 +35,7 @@ class Workspace:
         self.device, self.default_dtype, self.limits, self.ops = device, default_dtype, limits, ops
         self.buffers: Dict[str, torch.Tensor] = {}
         self.row_caps = {"head_in": limits.max_logit_rows, "logits": limits.max_logit_rows}
+        self.retired: List[torch.Tensor] = []
 
     def get(self, name, shape, dtype=None):
         dtype = dtype or self.default_dtype
@@ -65,24 +66,31 @@ class Workspace:
         return self.buffers[key]
 
     def flat(self, name, numel, dtype=torch.float32):
-        """A flat buffer of at least ``numel`` elements (grows if a larger one is asked for)."""
+        """A flat buffer of at least ``numel`` elements.  Asked for more than it holds it is replaced
+        by one at least half as large again; the old one is kept, not freed: recorded steps (graphs,
+        launch lists) hold its address."""
         key = ("flat", name, dtype)
         buf = self.buffers.get(key)
         if buf is None or buf.numel() < numel:
+            if buf is not None:
+                self.retired.append(buf)
+                numel = max(numel, buf.numel() + buf.numel() // 2)
             buf = torch.empty(numel, dtype=dtype, device=self.device)
             self.buffers[key] = buf
         return buf
 
     def bytes(self):
-        return sum(b.numel() * b.element_size() for b in self.buffers.values() if b is not None)
+        return sum(b.numel() * b.element_size() for b in list(self.buffers.values()) + self.retired if b is not None)
 
 
-class StepContext:
-    """What the parts see of one step: where each array of the packed metadata lies on the device
-    and on the host, the work buffers, and the attention entry point."""
+class StepContext(StepView):
+    """What the parts see of one step (parts.base.StepView): where each array of the packed
+    metadata lies on the device and on the host, and the work buffers."""
 
     def __init__(self, runner, layout: BatchLayout):
         self.runner, self.layout = runner, layout
+        self.limits, self.attention_mode = runner.limits, runner.attn
+        self.recording = False
         L = layout
         self.rows, self.real_rows = L.rows_padded, L.rows
         self.seqs, self.real_seqs = L.seqs_padded, L.seqs
@@ -91,7 +99,6 @@ class StepContext:
         # what kernels that size their launch by the context may assume; a captured graph sets it
         # to the largest context the engine allows, so that the launch fits every replay
         self.max_context_bound = max(L.max_context, 1)
-        self.shared = {}    # what parts of one step compute once and share (keyed by the part kind)
         self._leading = None
         d, h = runner.meta_dev, runner.meta_host
         T, S, R = self.rows, self.seqs, self.logit_rows_padded
@@ -148,15 +155,8 @@ class StepContext:
             return None
         return self.runner.workspace.scratch(name, rows, n, k)
 
-    def attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window=0):
-        self.runner.attention(self, q, out, kcache, vcache, g, nh, nkv, hd, scale, window)
-
-    def decode_attention_fused(self, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):
-        """Rotation by ``cos_sin``, page write at ``slots`` and attention in one launch, straight
-        from the QKV projection's result; False when this step or shape has no such kernel (then
-        the caller runs them one after the other: the same values up to rounding)."""
-        return self.runner.decode_attention_fused(self, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window,
-                                                  cos_sin, slots)
+    def flat(self, name, numel, dtype=torch.float32):
+        return self.runner.workspace.flat(name, numel, dtype)
 
 
 class ModelRunner:
@@ -183,98 +183,6 @@ class ModelRunner:
             self._upload_done.synchronize()
             self._upload_pending = False
         return self.meta_host
-
-    # ------------------------------------------------------------------------- attention
-    # Rows up to which a step is treated as decode-shaped by the partitioned attention kernel.
-    DECODE_ATTENTION_MAX_ROWS = 512
-
-    # The one-launch decode kernel walks a row's context chunk by chunk inside one workgroup:
-    # right when contexts are moderate or there are enough rows to fill the chip; a few rows with
-    # very long contexts are better cut into partitions that run in parallel.
-    def _decode_parts_scratch(self, rows, nh, nkv, hd, bound):
-        """Scratch for the decode kernel when it cuts long contexts of few rows into parts; sized at
-        once for the worst case (rows x parts <= 256 / kv heads + rows), so that a captured graph's
-        pointer stays good."""
-        need = self.ops.attention_decode_fused_scratch(rows, nh, nkv, hd, bound)
-        if need == 0:
-            return None
-        most_rows = min(self.DECODE_ATTENTION_MAX_ROWS, self.limits.max_tokens)
-        worst = nh * (256 // nkv + 1 + most_rows) * (hd + 2)
-        return self.workspace.flat("decode_parts", max(need, worst))
-
-    def decode_attention_fused(self, step, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):
-        """From the QKV projection to the attention output.  Decode-shaped steps: one launch (and a
-        small merge when few rows have long contexts).  Mixed steps (the scheduler puts decoding
-        requests first): the leading single-token runs take that launch too, the rows after them
-        are rotated and stored, then attended by the tiled kernel; a single-token run there would
-        otherwise cost a whole tile of its own."""
-        ops = self.ops
-        if (self.attn != "auto" or window != 0 or out.dtype != torch.bfloat16
-                or not ops.attention_decode_fused_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
-            return False
-        if step.max_run == 1:
-            if step.rows > self.DECODE_ATTENTION_MAX_ROWS:
-                return False
-            bound = step.max_context_bound
-            ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
-                                       step.ctx_lens, nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=step.rows,
-                                       max_context=bound, scratch=self._decode_parts_scratch(step.rows, nh, nkv, hd, bound))
-            return True
-        D, T, S = step.leading_single_runs(), step.real_rows, step.real_seqs
-        if (D == 0 or D > self.DECODE_ATTENTION_MAX_ROWS
-                or not ops.attention_prefill_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
-            return False
-        if isinstance(projection, ops.PartialSums):
-            # three consumers here (decode rows, rotation of the others, tiled attention): add the
-            # split sums up once instead of handing every single-token run to the tiled kernel
-            projection = projection.materialize()
-        stride = step.table_stride(g)
-        ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), stride, step.row_seq, step.ctx_lens,
-                                   nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=D, max_context=step.max_context,
-                                   scratch=self._decode_parts_scratch(D, nh, nkv, hd, step.max_context))
-        if (cos_sin is not None or slots is not None) and T > D:
-            ops.rope_cache(projection[D:T], nh, nkv, hd, cos_sin=cos_sin[D:T] if cos_sin is not None else None,
-                           slots=slots[D:T] if slots is not None else None, kcache=kcache, vcache=vcache,
-                           block_size=kcache.shape[2], rows=T - D)
-        need = ops.attention_prefill_scratch(T, nh, hd, step.max_context, step.max_run, S - D)
-        scratch = self.workspace.flat("prefill_partials", need) if need else None
-        ops.attention_prefill(projection, out, kcache, vcache, step.tables(g)[D * stride:], stride, step.run_start[D:],
-                              step.seq_start[D:], S - D, step.max_run, nh, nkv, hd, scale, rows=T,
-                              max_context=step.max_context, scratch=scratch)
-        return True
-
-    def attention(self, step, q, out, kcache, vcache, g, nh, nkv, hd, scale, window):
-        """attn = "v1": the generic kernel, one pass over the whole context per (row, head); "v2" and
-        "auto": for bfloat16, decode-shaped steps take the kernel that cuts contexts into partitions
-        and merges them, steps with runs of positions take the tiled kernel; "v2" insists on the
-        partitioned kernel for decode steps, "auto" prefers the one-launch kernel above where it
-        applies.  The 32-bit path always takes v1, whose result does not depend on the batch."""
-        ops = self.ops
-        partitioned = (self.attn != "v1" and window == 0 and step.max_run == 1
-                       and step.rows <= self.DECODE_ATTENTION_MAX_ROWS
-                       and ops.attention_decode_supported(nh, nkv, hd, q.dtype, kcache.shape[2]))
-        if self.attn == "v2" and not partitioned and q.dtype == torch.bfloat16 and step.max_run == 1:
-            raise RuntimeError(f"attn=v2: the partitioned kernel does not take heads={nh} kv_heads={nkv} "
-                               f"head_dim={hd} window={window} rows={step.rows}")
-        if partitioned:
-            bound = step.max_context_bound
-            need = ops.attention_decode_scratch(step.rows, nh, hd, bound)
-            scratch = self.workspace.flat("attention_partials", max(need, ops.attention_decode_scratch(
-                min(self.DECODE_ATTENTION_MAX_ROWS, self.limits.max_tokens), nh, hd, self.limits.max_context_len)))
-            ops.attention_decode(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
-                                 step.ctx_lens, nh, nkv, hd, scale, bound, scratch, rows=step.rows)
-            return
-        if (self.attn != "v1" and window == 0 and step.max_run > 1
-                and ops.attention_prefill_supported(nh, nkv, hd, q.dtype, kcache.shape[2])):
-            # runs of consecutive positions: keys are read once per 64 query rows, on the matrix cores
-            need = ops.attention_prefill_scratch(step.real_rows, nh, hd, step.max_context, step.max_run, step.real_seqs)
-            scratch = self.workspace.flat("prefill_partials", need) if need else None
-            ops.attention_prefill(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.run_start,
-                                  step.seq_start, step.real_seqs, step.max_run, nh, nkv, hd, scale,
-                                  rows=step.real_rows, max_context=step.max_context, scratch=scratch)
-            return
-        ops.attention(q, out, kcache, vcache, step.tables(g), step.table_stride(g), step.row_seq,
-                      step.ctx_lens, nh, nkv, hd, scale, window, rows=step.rows)
 
     # ------------------------------------------------------------------------------ steps
     def _check(self, layout: BatchLayout, logits_in_portions=False):

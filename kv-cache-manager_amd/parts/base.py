@@ -1,6 +1,11 @@
 """What a part is: the interfaces the model assembly, the weight loader, the cache planner and
 the step function rely on.  A part gets its sizes and constants as parameters and never learns
 which model it is in.
+
+Everything a part may rely on, and everything the engine asks of a part, is declared in this file:
+``StepView`` (what ``step`` offers), the base classes with their optional capabilities as class
+attributes (``capturable``, ``accepts_partial_sums``, ``rotates``, ``rotation_table``), and the
+``Deferred`` convention for results that are not added up yet.  Nothing else is probed.
 """
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -87,15 +92,96 @@ class BuildContext:
     ops: object                 # the kernel module (kvcm_amd.ops)
 
 
+# ------------------------------------------------------------------------------------- step
+class StepView:
+    """What a part sees of one step.  The engine's step context implements exactly this; a part
+    uses nothing else of it.
+
+    Shape of the step (host integers, fixed for a recorded step):
+      rows, real_rows              rows the kernels run (padded) / rows that carry tokens
+      seqs, real_seqs              sequences in the step (padded / real)
+      logit_rows, logit_rows_padded
+      max_run                      longest run of rows of one sequence (1: a decode-shaped step)
+      max_context                  longest context among the rows
+      max_context_bound            what launches sized by the context may assume (>= max_context; a
+                                   recorded step sets it to the bound it was recorded for)
+      limits                       the engine's ModelLimits (largest step the buffers are made for)
+      attention_mode               "auto" | "v1" | "v2" (the engine option of that name)
+      recording                    True while the step is being recorded for replay: a part may then
+                                   call nothing but this package's kernels (ctx.ops) on device arrays
+
+    Device arrays (int32, this step's metadata; all a capturable part may read):
+      tokens[rows] positions[rows] ctx_lens[rows] row_seq[rows]
+      run_start[seqs + 1] seq_start[seqs] seq_end[seqs] state_slots[seqs] logit_row_index[R]
+      slots(g)[rows]               where each row's key and value go in group g (-1: nowhere)
+      tables(g), table_stride(g)   page tables of group g, [seqs, table_stride(g)]
+
+    The same on the host (NumPy views, for parts that loop over sequences in Python; reading them
+    makes a part not capturable):
+      host_positions host_run_start host_seq_start host_seq_end host_state_slots
+      leading_single_runs()        how many of the first sequences run exactly one row
+
+    Work memory (stable addresses, reused by every step):
+      ws(name, (rows, cols), dtype=None)   a named 2-d work buffer in the compute dtype (or dtype)
+      flat(name, numel, dtype=float32)     a named flat buffer of at least numel elements
+      scratch(name, rows, n, k)            32-bit scratch for the split-K sums of a [rows, k] x [n, k]
+                                           product, or None where that product is not split
+      shared                               a dict in which parts of one step leave what later parts of
+                                           the same step may reuse (keyed by the part; see Rotary)
+
+    The members below are the defaults of a step that offers the least (what a part run on its own
+    in a test needs to override is ``rows``, the arrays it reads and ``ws``)."""
+
+    recording = False
+    attention_mode = "auto"
+    max_run = 1
+    limits = None
+
+    @property
+    def shared(self):
+        return self.__dict__.setdefault("_shared", {})
+
+    def scratch(self, name, rows, n, k):
+        return None
+
+    def leading_single_runs(self):
+        return 0
+
+
+class Deferred:
+    """Convention for a result that is not a plain tensor yet (ops.PartialSums: the un-added split-K
+    sums of a product).  It has ``materialize() -> tensor``; ``as_tensor`` turns either into a
+    tensor.  A consumer that can take the deferred form itself says so (``accepts_partial_sums``)."""
+
+    def materialize(self):
+        raise NotImplementedError
+
+
+def as_tensor(value):
+    return value.materialize() if hasattr(value, "materialize") else value
+
+
 class Part:
     """Base of every part.  Subclasses read ``params``, declare tensors in ``param_specs`` and get
     them (already on the device, in the precision their role asks for) through ``bind``."""
+
+    # True when ``forward`` (``apply``) is a fixed sequence of this package's kernel launches for
+    # a fixed step shape: every per-step value is read from the step's device arrays inside
+    # kernels, never from the host copies (``step.host_*``), nothing is allocated and no library
+    # routine is called.  Steps of a model whose parts are all capturable are recorded once per
+    # shape and replayed (HIP graphs for decode steps, native launch lists for the others); one
+    # part that is not keeps the whole model on the direct path.  The default is the safe one.
+    capturable = False
 
     def __init__(self, params: dict, prefix: str, ctx: BuildContext):
         self.params = dict(params)
         self.prefix = prefix
         self.ctx = ctx
         self.w: Dict[str, torch.Tensor] = {}
+
+    def sub_parts(self) -> Sequence["Part"]:
+        """Parts this part builds and drives itself (an attention's position encoding)."""
+        return ()
 
     def param_specs(self) -> List[ParamSpec]:
         return []
@@ -109,6 +195,9 @@ class Part:
 
 
 class Norm(Part):
+    # True: ``add`` may be a Deferred (un-added split-K sums), which the norm adds up itself.
+    accepts_partial_sums = False
+
     def forward(self, x, out, add=None, rows=None):
         """out = norm(x (+ add)); when ``add`` is given and ``rows`` is not, x += add as well.
         x is the 32-bit residual stream; rows gathers source rows."""
@@ -116,6 +205,20 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    # True: ``apply`` takes ``source=`` (the projection's un-added split-K sums) instead of
+    # finished rows.
+    accepts_partial_sums = False
+    # False: q and k are left as they are (no encoding at this place), which lets an attention
+    # kernel that stores k and v itself run without one.
+    rotates = True
+
+    def rotation_table(self, step, head_dim):
+        """For encodings that rotate pairs (j, j + head_dim/2) by an angle that depends on the row
+        alone: (cos, sin) of every row's angles, float32 [rows, head_dim/2, 2] on the device, for
+        attention kernels that rotate inside.  None: this encoding is no such rotation (the
+        attention then calls ``apply``)."""
+        return None
+
     def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None):
         """Transforms the q and k heads of the fused rows in place, given step.positions.  When a
         cache (k, v tensors) and slots are passed, also stores k (transformed) and v there and
@@ -156,8 +259,16 @@ class Head(Part):
 class Block:
     """An arrangement of parts.  ``forward`` takes the residual stream x (32-bit, updated in
     place) and the output of the previous block that has not been added to x yet (``pending``,
-    may be None); it returns its own not-yet-added output, so that the addition fuses into the
-    next norm."""
+    a tensor, a Deferred or None); it returns its own not-yet-added output, so that the addition
+    fuses into the next norm.
+
+    ``part_registries`` maps the names a LayerSpec may give this arrangement's parts to the
+    registry each is looked up in (a registry object, or its name: "mixer", "feed_forward",
+    "norm", "position").  Names it does not list fall back to the common ones: ``mixer``, ``ffn``
+    and anything starting with ``norm``."""
+
+    part_registries: Dict[str, object] = {}
+    capturable = False      # as Part.capturable, for what the arrangement itself does between parts
 
     def __init__(self, parts: Dict[str, Part]):
         self.parts = parts

@@ -9,20 +9,16 @@ import math
 import torch
 
 from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS
-from .base import (Block, Embedding, FeedForward, Head, KVCacheNeed, Mixer, Norm, ParamSpec, PositionEncoding)
+from . import paged_attention
+from .base import (Block, Embedding, FeedForward, Head, KVCacheNeed, Mixer, Norm, ParamSpec, PositionEncoding, as_tensor)
 
 
 def _linear(ctx, step, x, w, name, keep_partial=False, dtype=None):
     """x @ w^T into the work buffer ``name``.  With ``keep_partial`` the result may come back as
     un-added split-K sums (ops.PartialSums) for a consumer that adds them up itself."""
     out = step.ws(name, (x.shape[0], w.shape[0]), dtype)
-    scratch = step.scratch(name, x.shape[0], w.shape[0], w.shape[1]) if hasattr(step, "scratch") else None
+    scratch = step.scratch(name, x.shape[0], w.shape[0], w.shape[1])
     return ctx.ops.gemm(x, w, out, scratch=scratch, keep_partial=keep_partial and scratch is not None)
-
-
-def _tensor(value):
-    """A product's result as a plain tensor (adds partial sums up if that is what it is)."""
-    return value.materialize() if hasattr(value, "materialize") else value
 
 
 @NORMS.register("rmsnorm")
@@ -30,10 +26,11 @@ class RMSNorm(Norm):
     """out = weight * round(x / sqrt(mean(x^2) + eps)); eps inside the root, no mean removed, the
     weight a plain multiplier (src/cuda/kernels.cu:34-49).  params: size, eps."""
 
+    capturable = True
+    accepts_partial_sums = True
+
     def param_specs(self):
         return [ParamSpec("weight", ((self.prefix + "weight", (self.params["size"],)),), role="vector")]
-
-    accepts_partial_sums = True
 
     def forward(self, x, out, add=None, rows=None):
         self.ctx.ops.rmsnorm(x, self.w["weight"], out, self.params["eps"], add=add, rows=rows)
@@ -46,6 +43,9 @@ class Rotary(PositionEncoding):
     head: pairs (j, j + dim/2), inv_freq_j = theta^(-2j/dim), angle = position * inv_freq_j in
     32-bit (src/cuda/kernels.cu:51-70).  params: theta, dim."""
 
+    capturable = True
+    accepts_partial_sums = True
+
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
         dim = params["dim"]
@@ -55,21 +55,21 @@ class Rotary(PositionEncoding):
     def ignorable_tensors(self):
         return (self.prefix + "rotary_emb.inv_freq",)
 
-    accepts_partial_sums = True
-
     def rotation_table(self, step, head_dim):
-        """(cos, sin) of every row's angles [rows, head_dim/2, 2], or None where the step cannot
-        share work between layers.  The angles depend on the row only: the first layer of a step
-        computes them, the others (same theta and dim) read them."""
-        shared = getattr(step, "shared", None)
-        if shared is None or head_dim != self.params["dim"]:
+        """(cos, sin) of every row's angles [rows, head_dim/2, 2].  The angles depend on the row
+        only: the first layer of a step computes them, the others with the same theta and dim read
+        them.  Each (theta, dim) has a table and a work buffer of its own, so layers that alternate
+        between two thetas do not overwrite each other's angles."""
+        if head_dim != self.params["dim"]:
             return None
-        key = ("rotary", float(self.params["theta"]), head_dim)
-        table = shared.get(key)
+        theta = float(self.params["theta"])
+        key = ("rotary", theta, head_dim)
+        table = step.shared.get(key)
         if table is None:
-            table = step.ws("rotary_cos_sin_%d" % head_dim, (step.rows, head_dim), torch.float32).view(step.rows, head_dim // 2, 2)
+            name = "rotary_cos_sin_%d_%s" % (head_dim, theta.hex())
+            table = step.ws(name, (step.rows, head_dim), torch.float32).view(step.rows, head_dim // 2, 2)
             self.ctx.ops.rope_table(step.positions, self.inv_freq, table, rows=step.rows)
-            shared[key] = table
+            step.shared[key] = table
         return table
 
     def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None, source=None):
@@ -85,6 +85,7 @@ class Rotary(PositionEncoding):
 
 @POSITIONS.register("none")
 class NoPosition(PositionEncoding):
+    capturable = True
     rotates = False
 
     def apply(self, step, qkv, num_heads, num_kv_heads, head_dim, cache=None, slots=None):
@@ -98,6 +99,11 @@ class GQAAttention(Mixer):
     step's rows before attention reads them (llama.cpp:111-115), so a portion of a prompt attends
     to itself through the cache; causality is context length = position + 1.
     params: num_heads, num_kv_heads, head_dim, scale, window (0 = all keys), position (PartSpec)."""
+
+    capturable = True
+
+    def sub_parts(self):
+        return (self.position,)
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
@@ -125,31 +131,24 @@ class GQAAttention(Mixer):
         ops = self.ctx.ops
         g = self.cache.group
         kc, vc = self.cache.k(self.cache_index), self.cache.v(self.cache_index)
-        fused = getattr(self.position, "accepts_partial_sums", False)
-        res = _linear(self.ctx, step, h, self.w["wqkv"], "qkv", keep_partial=fused)
+        pos = self.position
+        res = _linear(self.ctx, step, h, self.w["wqkv"], "qkv", keep_partial=pos.accepts_partial_sums)
         qkv = step.ws("qkv", (step.rows, self.q_dim + 2 * self.kv_dim))
         slots = step.slots(g) if self.cache_owner else None
         attn = step.ws("attn", (step.rows, self.q_dim))
         # decode-shaped steps: rotation, page write and attention in one launch, where the position
-        # encoding is a rotation by pairs (or none) and the step offers that kernel
-        fused_attention = getattr(step, "decode_attention_fused", None)
-        if fused_attention is not None:
-            pos, table, fusable = self.position, None, False
-            if getattr(pos, "rotates", True) is False:
-                fusable = True
-            elif hasattr(pos, "rotation_table"):
-                table = pos.rotation_table(step, self.hd)
-                fusable = table is not None
-            if fusable and fused_attention(res, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window,
-                                           table, slots):
-                return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
+        # encoding is a rotation by pairs (or none) and the step's shape has that kernel
+        table = pos.rotation_table(step, self.hd) if pos.rotates else None
+        if (table is not None or not pos.rotates) and paged_attention.attend_from_projection(
+                step, ops, res, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window, table, slots):
+            return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
         extra = {"source": res} if hasattr(res, "materialize") else {}
-        stored = self.position.apply(step, qkv, self.nh, self.nkv, self.hd,
-                                     cache=(kc, vc) if self.cache_owner else None, slots=slots, **extra)
+        stored = pos.apply(step, qkv, self.nh, self.nkv, self.hd,
+                           cache=(kc, vc) if self.cache_owner else None, slots=slots, **extra)
         if self.cache_owner and not stored:
             ops.rope_cache(qkv, self.nh, self.nkv, self.hd, slots=slots, kcache=kc, vcache=vc,
                            block_size=self.ctx.block_size, rows=step.rows)
-        step.attention(qkv, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window)
+        paged_attention.attend(step, ops, qkv, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window)
         return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
 
 
@@ -157,6 +156,8 @@ class GQAAttention(Mixer):
 class SwiGLU(FeedForward):
     """down( round(silu(gate(h))) * up(h) ) with gate and up as one fused projection
     (src/model/llama.cpp:119-122, src/cuda/kernels.cu:72-82).  params: intermediate_size."""
+
+    capturable = True
 
     def param_specs(self):
         H, I, pre = self.ctx.hidden_size, self.params["intermediate_size"], self.prefix
@@ -177,6 +178,8 @@ class TokenEmbedding(Embedding):
     """x = float(table[token]); nothing scaled or added (src/cuda/kernels.cu:27-32).
     params: vocab_size."""
 
+    capturable = True
+
     def param_specs(self):
         return [ParamSpec("table", ((self.prefix + "weight", (self.params["vocab_size"], self.ctx.hidden_size)),),
                           role="table")]
@@ -190,6 +193,8 @@ class TokenEmbedding(Embedding):
 class LinearHead(Head):
     """logits = h @ table^T in 32-bit, only for the rows that are asked for
     (src/model/llama.cpp:126-128).  params: vocab_size, tied (use the embedding's table)."""
+
+    capturable = True
 
     def param_specs(self):
         if self.params.get("tied"):
@@ -211,10 +216,12 @@ class PreNormResidual(Block):
     """x += mixer(norm_mixer(x)); x += ffn(norm_ffn(x))  (src/model/llama.cpp:104-124).  Each
     addition is done by the norm that follows it."""
 
+    capturable = True
+
     def forward(self, step, x, pending):
         h = step.ws("normed", (step.rows, x.shape[1]))
         n1, n2 = self.parts["norm_mixer"], self.parts["norm_ffn"]
-        n1.forward(x, h, add=pending if getattr(n1, "accepts_partial_sums", False) else _tensor(pending))
+        n1.forward(x, h, add=pending if n1.accepts_partial_sums else as_tensor(pending))
         a = self.parts["mixer"].forward(step, h)
-        n2.forward(x, h, add=a if getattr(n2, "accepts_partial_sums", False) else _tensor(a))
+        n2.forward(x, h, add=a if n2.accepts_partial_sums else as_tensor(a))
         return self.parts["ffn"].forward(step, h)

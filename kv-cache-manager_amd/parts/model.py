@@ -6,19 +6,34 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
-from .base import BuildContext, KVCacheNeed, Mixer, ModelSpec, Part, StateNeed
+from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, Registry
+from .base import BuildContext, KVCacheNeed, Mixer, ModelSpec, Part, StateNeed, as_tensor
 
-# which registry a named slot of a block is looked up in
-_SLOT_REGISTRY = {"mixer": MIXERS, "ffn": FEED_FORWARDS}
+# registries by the names a block arrangement may use in ``part_registries``
+_REGISTRY_NAMES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "ffn": FEED_FORWARDS, "norm": NORMS,
+                   "position": POSITIONS}
 
 
-def _registry_for(slot):
-    if slot in _SLOT_REGISTRY:
-        return _SLOT_REGISTRY[slot]
+def _registry_for(slot, block_class=None):
+    """The registry a part named ``slot`` of a layer is built from: what the layer's block
+    arrangement declares for that name (``Block.part_registries``), else the common names."""
+    declared = getattr(block_class, "part_registries", None) or {}
+    if slot in declared:
+        reg = declared[slot]
+        if isinstance(reg, Registry):
+            return reg
+        if reg in _REGISTRY_NAMES:
+            return _REGISTRY_NAMES[reg]
+        raise KeyError(f"{getattr(block_class, '__name__', block_class)}.part_registries[{slot!r}] names no registry: "
+                       f"{reg!r} (a Registry, or one of {sorted(_REGISTRY_NAMES)})")
+    if slot == "mixer":
+        return MIXERS
+    if slot == "ffn":
+        return FEED_FORWARDS
     if slot.startswith("norm"):
         return NORMS
-    raise KeyError(f"a block part named {slot!r} has no registry (mixer, ffn, norm*)")
+    raise KeyError(f"a block part named {slot!r} has no registry: the block arrangement must list it in "
+                   f"part_registries (common names: mixer, ffn, norm*)")
 
 
 @dataclass
@@ -40,9 +55,11 @@ class Model:
         self.blocks = []
         self.layer_parts: List[Dict[str, Part]] = []
         for layer in spec.layers:
-            parts = {slot: _registry_for(slot).get(ps.kind)(ps.params, ps.prefix, ctx) for slot, ps in layer.parts.items()}
+            block_class = BLOCKS.get(layer.block)
+            parts = {slot: _registry_for(slot, block_class).get(ps.kind)(ps.params, ps.prefix, ctx)
+                     for slot, ps in layer.parts.items()}
             self.layer_parts.append(parts)
-            self.blocks.append(BLOCKS.get(layer.block)(parts))
+            self.blocks.append(block_class(parts))
         for i in spec.schedule:
             if not 0 <= i < len(self.blocks):
                 raise ValueError(f"schedule names layer {i}, the model has {len(self.blocks)}")
@@ -55,6 +72,26 @@ class Model:
             out.extend(parts.values())
         out += [self.final_norm, self.head]
         return out
+
+    def every_part(self) -> List[Part]:
+        """All parts, with the parts that parts drive themselves."""
+        out, todo = [], list(self.all_parts())
+        while todo:
+            p = todo.pop()
+            out.append(p)
+            todo.extend(p.sub_parts())
+        return out
+
+    @property
+    def capturable(self) -> bool:
+        """May a step of this model be recorded once and replayed?  Only when every part and every
+        block arrangement says so of itself."""
+        return all(p.capturable for p in self.every_part()) and all(b.capturable for b in self.blocks)
+
+    def not_capturable(self) -> List[str]:
+        names = [type(p).__name__ for p in self.every_part() if not p.capturable]
+        names += [type(b).__name__ for b in self.blocks if not b.capturable]
+        return sorted(set(names))
 
     def finish_binding(self):
         """Called by the loader after every part got its tensors: shares tied tables."""
@@ -115,8 +152,8 @@ class Model:
         addition) and output head on those rows only (src/model/llama.cpp:126-128)."""
         R = row_index.numel()
         h_last = step.ws("head_in", (R, self.spec.hidden_size))
-        if hasattr(pending, "materialize") and not getattr(self.final_norm, "accepts_partial_sums", False):
-            pending = pending.materialize()
+        if not self.final_norm.accepts_partial_sums:
+            pending = as_tensor(pending)
         self.final_norm.forward(x, h_last, add=pending, rows=row_index)
         logits = out if out is not None else step.ws("logits", (R, self.spec.vocab_size), torch.float32)
         return self.head.forward(step, h_last, logits)

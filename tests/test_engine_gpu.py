@@ -268,7 +268,8 @@ def test_graphs_follow_the_context_across_classes(tmp_path):
     H.make_model_dir(d, H.TINY_D, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=H.SHARPEN["D"])
     pm = plain.load_model_dir(d, plain.round_bf16)
     prompts = _prompts(H.TINY_D, [2030, 100], seed=13)
-    kw = dict(dtype="bfloat16", num_blocks=300, max_seq_len=4096, max_batched_tokens=4096)
+    # (the tiny model states 2,048 positions; running past them is what this test is about)
+    kw = dict(dtype="bfloat16", num_blocks=300, max_seq_len=4096, max_batched_tokens=4096, beyond_max_position=True)
     eng = _engine(d, use_graphs=True, **kw)
     got = eng.generate(prompts, 40)
     assert sorted(eng.decode_graphs.graphs) == [(2, 2048), (2, 4096)]
@@ -317,11 +318,17 @@ def _ctx(dtype, hidden):
     return BuildContext(dtype, torch.device("cuda:0"), hidden, 8, ops)
 
 
-class _Step:
-    """The little of a step that a part needs when it is run on its own."""
+def _step_base():
+    from kvcm_amd.parts.base import StepView
+    return StepView
+
+
+class _Step(_step_base()):
+    """The little of a step that a part needs when it is run on its own: the declared view of a step
+    (parts.base.StepView) with the arrays this part reads."""
 
     def __init__(self, rows, positions=None):
-        self.rows = rows
+        self.rows = self.real_rows = rows
         self.positions = None if positions is None else torch.tensor(positions, dtype=torch.int32, device="cuda:0")
         self.tokens = None
         self._bufs = {}
@@ -410,12 +417,19 @@ def test_part_attention_mixer_alone_through_the_cache():
             super().__init__(hi - lo, list(range(lo, hi)))
             self.lo, self.hi = lo, hi
 
+            self.max_run, self.real_seqs, self.seqs = hi - lo, 1, 1
+            self.row_seq = _dev([0] * self.rows, torch.int32)
+            self.ctx_lens = _dev([p + 1 for p in range(lo, hi)], torch.int32)
+            self.max_context = self.max_context_bound = hi
+
         def slots(self, g):
             return _dev([table[p // B] * B + p % B for p in range(self.lo, self.hi)], torch.int32)
 
-        def attention(self, q, out, kc, vc, g, nh_, nkv_, hd_, scale, window=0):
-            ctx.ops.attention(q, out, kc, vc, _dev(table, torch.int32), 3, _dev([0] * self.rows, torch.int32),
-                              _dev([p + 1 for p in range(self.lo, self.hi)], torch.int32), nh_, nkv_, hd_, scale, window)
+        def tables(self, g):
+            return _dev(table, torch.int32)
+
+        def table_stride(self, g):
+            return 3
 
     outs = []
     for lo, hi in [(0, 13), (13, 14), (14, 19), (19, 20), (20, 21)]:
@@ -475,7 +489,8 @@ def test_random_workloads_over_engine_options(tmp_path, which):
     for combo, (chunk, budget, prefix, graphs) in enumerate(itertools.product((0, 37), (96, 512), (False, True), (True, False))):
         rng = np.random.default_rng(combo)
         eng = _engine(d, dtype="bfloat16", block_size=B, num_blocks=70 * 16 // B, max_seq_len=1024, max_num_seqs=8,
-                      max_batched_tokens=budget, prefill_chunk=chunk, prefix_caching=prefix, use_graphs=graphs)
+                      max_batched_tokens=budget, prefill_chunk=chunk, prefix_caching=prefix, use_graphs=graphs,
+                      beyond_max_position=True)      # (configuration E states 512 positions; lengths here go to 930)
         shared = rng.integers(0, raw["vocab_size"], size=100).tolist()
         pending = []
         for i in range(16):

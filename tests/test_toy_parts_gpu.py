@@ -138,9 +138,13 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         np.testing.assert_allclose(np.concatenate(got[rid]), ref[rid], atol=2e-4)
     assert rp.core.state_slots_free() == 8
 
-    # and through the scheduler: greedy generation equals the plain toy
+    # and through the scheduler, with the engine's default options for recorded steps (graphs, launch
+    # lists): this mixer reads the step's host arrays, says nothing about being capturable, and so
+    # every step of the model runs directly; greedy generation equals the plain toy
     eng = Engine(d, EngineConfig(dtype="float32", num_blocks=8, max_seq_len=64, max_num_seqs=4, max_batched_tokens=64,
-                                 prefill_chunk=6, use_graphs=False))
+                                 prefill_chunk=6))
+    assert eng.config.use_graphs and eng.config.use_programs
+    assert eng.decode_graphs is None and eng.programs is None and eng.model.not_capturable() == ["DecayState"]
     prompts = [reqs["y"], reqs["z"][:5]]
     outs = eng.generate(prompts, 6)
     for p, g in zip(prompts, outs):
@@ -312,6 +316,10 @@ _MIXED_LAYERS = [
          ffn=("swiglu", {"intermediate_size": 48})),
     dict(heads=4, kv_heads=2, head_dim=16, window=0, position=("none", {}),
          ffn=("toy_top1_experts", {"experts": 2, "inner": 40})),
+    # the first layer's theta and width again, after a layer with another theta of the same width: each
+    # (theta, width) keeps angles of its own within a step
+    dict(heads=4, kv_heads=2, head_dim=16, window=0, position=("rotary", {"theta": 10000.0, "dim": 16}),
+         ffn=("swiglu", {"intermediate_size": 64})),
 ]
 
 
@@ -366,7 +374,7 @@ def test_full_and_windowed_layers_routed_ffn_and_another_position_encoding(tmp_p
     rp = TraceReplayer(d, "float32", max_tokens=192)
     kinds = [(g.kind, g.window) for g in rp.core.groups]
     assert kinds == [("full", 0), ("window", 20), ("window", 9)]
-    assert [p.layers for p in rp.model.groups] == [["b0", "b3"], ["b1"], ["b2"]]
+    assert [p.layers for p in rp.model.groups] == [["b0", "b3", "b4"], ["b1"], ["b2"]]
     steps = [[("a", 0, 30), ("b", 0, 2)], [("a", 30, 33), ("b", 2, 41)], [("a", 33, 34), ("c", 0, 17)],
              [("a", 34, 70), ("c", 17, 18)], [("c", 18, 57)], [("a", 70, 72)]] + [[("a", k, k + 1)] for k in range(72, 90)]
     got = {k: [] for k in reqs}
@@ -392,7 +400,8 @@ def test_full_and_windowed_layers_routed_ffn_and_another_position_encoding(tmp_p
 
     # through the scheduler, with few pages and prompts cut into portions
     eng = Engine(d, EngineConfig(dtype="float32", block_size=16, num_blocks=9, max_seq_len=128, max_num_seqs=4,
-                                 max_batched_tokens=48, prefill_chunk=13, use_graphs=False))
+                                 max_batched_tokens=48, prefill_chunk=13))
+    assert eng.decode_graphs is None and eng.model.not_capturable() == ["Damped", "Top1Experts"]
     prompts = [reqs["b"], reqs["c"][:30]]
     outs = eng.generate(prompts, 24)
     for p, g in zip(prompts, outs):
