@@ -14,6 +14,9 @@ struct Sequence {
   int prompt_len = 0;
   int max_new_tokens = 0;
   int num_computed = 0;
+  // True from admission until a token has been sampled: the runs of that time cover tokens that
+  // were given (the prompt, or everything after a preemption), and are booked as prefill.
+  bool in_prompt = false;
 
   // One page table per cache group (empty for groups that hold fixed-size state).  Logical token
   // t of group g lives in page tables[g][t / B]; an entry of -1 is a page that a window has

@@ -233,7 +233,7 @@ def test_schedule_summary_and_update_by_sampled_ids():
     assert (n, prefill, decode, sampling, shaped) == (2, 4, 1, 1, False)       # request 1 decodes beside a portion of 2
     core.update_sampled([43])
     n, prefill, decode, sampling, shaped = core.schedule_summary()
-    assert (n, prefill, decode, sampling, shaped) == (2, 0, 2, 2, True)        # a prompt's last single token runs like a decode
+    assert (n, prefill, decode, sampling, shaped) == (2, 1, 1, 2, True)        # a prompt's last single token: shaped like a decode, booked as prompt
     assert core.plan_max_context == 9            # request 2's ninth token
     core.update_sampled([44, 50])
     n, prefill, decode, sampling, shaped = core.schedule_summary()
@@ -241,3 +241,29 @@ def test_schedule_summary_and_update_by_sampled_ids():
     core.update_sampled([51])
     done = {f.id: f.generated for f in core.take_finished()}
     assert done[1] == [42, 43, 44]
+
+
+def test_a_prompt_whose_last_portion_is_one_token_is_still_booked_as_prompt():
+    m = HostCore(num_blocks=100, block_size=4, max_seq_len=64, prefill_chunk=6)
+    m.sched_add(0, _prompt(0, 7), 3)
+    kinds = []
+    while not m.idle():
+        plan = m.schedule(0)
+        kinds.append([(p.start, p.count, p.is_prefill, p.samples) for p in plan])
+        m.update([42] * len(plan), 0)
+    assert kinds == [[(0, 6, True, False)], [(6, 1, True, True)], [(7, 1, False, True)], [(8, 1, False, True)]]
+    c = m.counters()
+    assert c["prefill_tokens"] == 7 and c["decode_tokens"] == 2      # the third sampled token is never run
+    f = m.take_finished()[0]
+    assert f.prefill_tokens_computed == 7 and len(f.generated) == 3
+
+
+def test_an_uncut_prompt_larger_than_the_budget_runs_whole_in_an_empty_step():
+    m = HostCore(num_blocks=1000, block_size=16, max_seq_len=4096, max_batched_tokens=100)
+    m.sched_add(0, _prompt(0, 300), 2)
+    m.sched_add(1, _prompt(1, 40), 2)
+    plan = m.schedule(0)
+    assert [(p.id, p.start, p.count, p.samples) for p in plan] == [(0, 0, 300, True)]       # not cut, and nothing beside it
+    m.update([42], 0)
+    plan = m.schedule(1)
+    assert [(p.id, p.start, p.count) for p in plan] == [(0, 300, 1), (1, 0, 40)]
