@@ -161,8 +161,10 @@ class HostCore:
         self.prefill_chunk = prefill_chunk
         self.prefix_caching = bool(prefix_caching) and policy == "paged"
         self._desc = np.zeros(self._lib.kvcm_batch_desc_len(self._h), dtype=np.int32)
-        self._summary = np.zeros(6, dtype=np.int64)
-        self.plan_max_context = 0      # of the last schedule_summary: the longest context a row of the plan sees
+        self._summary = np.zeros(10, dtype=np.int64)
+        # of the last schedule_summary: the longest context a row of the plan sees, its rows in all, how
+        # many of its first entries run one token, its longest run
+        self.plan_max_context = self.plan_rows = self.plan_leading = self.plan_max_run = 0
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -282,7 +284,7 @@ class HostCore:
         decode_shaped) without building the plan's entries in Python (``plan()`` still gives them)."""
         check(self._lib.kvcm_sched_schedule_summary(self._h, float(now), self._summary.ctypes.data_as(i64p)))
         s = self._summary
-        self.plan_max_context = int(s[5])
+        self.plan_max_context, self.plan_rows, self.plan_leading, self.plan_max_run = int(s[5]), int(s[6]), int(s[7]), int(s[8])
         return int(s[0]), int(s[1]), int(s[2]), int(s[3]), bool(s[4])
 
     def update_sampled(self, ids, now=0.0):
@@ -343,8 +345,19 @@ class HostCore:
         return BatchLayout(self._desc, self.num_groups)
 
     def build_batch_from_plan(self, out: np.ndarray, *, pad_rows=0, pad_seqs=0, pad_logit_rows=0,
-                              table_stride=0) -> BatchLayout:
-        check(self._lib.kvcm_build_batch_from_plan(
-            self._h, pad_rows, pad_seqs, pad_logit_rows, table_stride, out.ctypes.data, out.size,
+                              table_stride=0, pad_leading=0) -> BatchLayout:
+        """The scheduler's current plan as a batch.  ``pad_leading``: bring the leading single-token
+        runs up to that many with padding sequences of one padding row each (recorded step shapes)."""
+        check(self._lib.kvcm_build_batch_from_plan_shaped(
+            self._h, pad_rows, pad_seqs, pad_logit_rows, table_stride, pad_leading, out.ctypes.data, out.size,
             self._desc.ctypes.data_as(i32p)))
         return BatchLayout(self._desc, self.num_groups)
+
+    @property
+    def handle(self):
+        """The native core, for native callers (the step executor)."""
+        return self._h
+
+    def native_function(self, name) -> int:
+        """Address of one of the host core's C functions."""
+        return C.cast(getattr(self._lib, name), C.c_void_p).value

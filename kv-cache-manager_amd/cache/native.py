@@ -73,6 +73,7 @@ def _declare(lib):
     fn("kvcm_batch_desc_len", i, vp)
     fn("kvcm_build_batch", i, vp, i, i64p, i32p, i32p, i32p, i32p, i, i, i, i, C.c_void_p, i64, i32p)
     fn("kvcm_build_batch_from_plan", i, vp, i, i, i, i, C.c_void_p, i64, i32p)
+    fn("kvcm_build_batch_from_plan_shaped", i, vp, i, i, i, i, i, C.c_void_p, i64, i32p)
 
 
 def lib():

@@ -27,6 +27,10 @@ HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={GPU_ARCH}", "-Xclan
              "-Xclang", "-packed-fp32-ops", "-Wno-unused-result", "-ffp-contract=fast"]
 
 
+# the vendor library's matrix product (prompt steps), as the reference links cuBLAS
+HIP_LINK = ["-lhipblaslt"]
+
+
 def _say(msg):
     print(f"[kvcm build] {msg}", file=sys.stderr, flush=True)
 
@@ -137,7 +141,7 @@ def build_host(force=False):
 def build_hip(force=False, jobs=None):
     srcs = _sources(HIP_DIR, (".hip",))
     deps = _sources(HIP_DIR, (".hip", ".h"))
-    digest = _digest(deps, HIP_FLAGS)
+    digest = _digest(deps, HIP_FLAGS + HIP_LINK)
     name = "libkvcm_hip.so"
     if not force:
         lib = _find_built(name, digest)
@@ -186,7 +190,7 @@ def build_hip(force=False, jobs=None):
     if errors:
         raise errors[0]
     tmp = lib + f".tmp{os.getpid()}"
-    _run([hipcc, "-shared", "-fPIC", f"--offload-arch={GPU_ARCH}"] + sorted(objs) + ["-o", tmp], "link")
+    _run([hipcc, "-shared", "-fPIC", f"--offload-arch={GPU_ARCH}"] + sorted(objs) + HIP_LINK + ["-o", tmp], "link")
     os.replace(tmp, lib)
     with open(lib + ".stamp", "w") as f:
         f.write(digest)

@@ -1,8 +1,10 @@
-// C entry points of libkvcm_hip.so that programs other than this package's Python layer call.
-// Every entry returns 0 on success and a negative value on failure; kvcm_hip_last_error() then
-// holds the reason (per calling thread).  Pointers are device pointers unless said otherwise.
+// C entry points of libkvcm_hip.so.  Every entry that launches returns 0 on success and a negative
+// value on failure; kvcm_hip_last_error() then holds the reason (per calling thread).  Pointers are
+// device pointers unless said otherwise; `*_dtype` arguments are KVCM_F32 or KVCM_BF16.  An entry
+// checks on the host that sizes fit what its kernel assumes and launches nothing when they do not.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -42,6 +44,70 @@ int kvcm_reduce_store(const float* partials, void* out, int out_dtype, int M, in
 long long kvcm_gemm_skinny_noalloc_capacity();
 int kvcm_gemm_skinny_noalloc(const void* X, const void* W, void* out, int out_dtype, int M, int N, int K, int ldx,
                              int ldw, int ldo, hipStream_t stream);
+
+// ---- row-wise kernels (elementwise.hip) ------------------------------------------------------
+int kvcm_embed(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, hipStream_t s);
+int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const float* partials, int S, int T, const int* rows,
+                 const void* w, int w_dtype, void* out, int out_dtype, int R, int H, float eps, int write_back,
+                 hipStream_t s);
+int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, const float* inv_freq, const int* slots,
+                    void* kcache, void* vcache, int T, int nh, int nkv, int hd, int B, const float* partials, int S,
+                    const float* cos_sin, hipStream_t s);
+int kvcm_rope_table(const int* positions, const float* inv_freq, float* cos_sin, int T, int half, hipStream_t s);
+int kvcm_swiglu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t s);
+int kvcm_add_residual(float* x, const void* y, int dtype, long long n, hipStream_t s);
+
+// ---- products --------------------------------------------------------------------------------
+int kvcm_gemm_skinny_swiglu_supported(int M, int I, int K);
+int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dtype, int M, int I, int K, int ldx,
+                            int ldw, int ldo, hipStream_t stream);
+int kvcm_gemm_f32(const float* X, const float* W, float* Y, int M, int N, int K, int ldx, int ldw, int ldy, hipStream_t s);
+int kvcm_gemm_bf16(const void* X, const void* W, void* Y, int out_dtype, int M, int N, int K, int ldx, int ldw, int ldy,
+                   hipStream_t s);
+// The vendor library's product (hipBLASLt), bfloat16 operands and result, 32-bit accumulation, for
+// the many-row products of prompt steps, where the reference calls cuBLAS (src/model/llama.cpp:45-52).
+// `workspace` is device memory the caller owns (at least kvcm_gemm_library_workspace_bytes()).
+long long kvcm_gemm_library_workspace_bytes();
+int kvcm_gemm_library(const void* X, const void* W, void* out, int M, int N, int K, int ldx, int ldw, int ldo,
+                      void* workspace, long long workspace_bytes, hipStream_t stream);
+
+// ---- attention over the paged cache ----------------------------------------------------------
+int kvcm_attention_generic(const void* q, int dtype, int q_stride, void* out, int out_stride, const void* kcache,
+                           const void* vcache, const int* tables, int table_stride, const int* row_seq,
+                           const int* ctx_lens, int T, int nh, int nkv, int hd, int B, float scale, int window,
+                           hipStream_t s);
+int kvcm_attention_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache, const void* vcache,
+                          const int* tables, int table_stride, const int* row_seq, const int* ctx_lens, int T, int nh,
+                          int nkv, int hd, int B, float scale, int max_context, float* scratch, long long scratch_floats,
+                          hipStream_t s);
+int kvcm_attention_decode_fused(const float* partials, int S, const void* qkv, int qkv_stride, const float* cos_sin,
+                                const int* slots, void* kcache, void* vcache, const int* tables, int table_stride,
+                                const int* row_seq, const int* ctx_lens, int T, int nh, int nkv, int hd, int B, float scale,
+                                void* out, int out_stride, int max_context, float* scratch, long long scratch_floats,
+                                hipStream_t s);
+int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kcache, const void* vcache,
+                           const int* tables, int table_stride, const int* run_start, const int* seq_start, int S,
+                           int max_run, int T, int max_context, int nh, int nkv, int hd, int B, float scale,
+                           float* scratch, long long scratch_floats, hipStream_t s);
+
+// ---- sampling ---------------------------------------------------------------------------------
+int kvcm_sample(const float* logits, int ld, const float* temperature, const uint64_t* seeds, const long long* request_ids,
+                const int* token_index, int* out, int R, int V, hipStream_t s);
+
+// ---- recorded steps ---------------------------------------------------------------------------
+// A step program is the list of launches of one step, recorded once for a step shape and replayed
+// with nothing but the step's metadata changed (the kernels read that from device memory).  The
+// reference issues every launch of every step from its C++ step function
+// (src/model/llama.cpp:54-141); here the parts that decide the launches are assembled per model,
+// so the list is recorded while they run once and replayed natively afterwards.
+//   `entry`  name of one of the launching entries above (the last argument of each is the stream);
+//   `args`   the entry's arguments, one 64-bit slot each: pointers and integers as they are, a float
+//            as its 32 bits in the low half; the stream's slot is ignored (a replay brings its own).
+void* kvcm_program_new();
+void kvcm_program_delete(void* program);
+int kvcm_program_add(void* program, const char* entry, const uint64_t* args, int num_args);
+int kvcm_program_size(void* program);
+int kvcm_program_run(void* program, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -42,9 +42,12 @@ inline int batch_desc_len(int num_groups) { return kGroupBase + kGroupStride * n
 
 // Padding rows have token 0, position 0, context length 0 and slot -1: they write no key and
 // attend to nothing.  Padding sequences have empty runs and tables of zeros.
+// `pad_leading` brings the step's leading single-token runs up to that many: the entries before the
+// first one with more than one token are followed by padding sequences of one padding row each, so
+// that a step recorded for "D single rows, then prompt portions" fits every step with at most D.
 inline void build_batch(const KVManager& kv, const std::vector<BatchEntry>& entries, int pad_rows,
                         int pad_seqs, int pad_logit_rows, int table_stride, int32_t* out, int64_t cap,
-                        int32_t* desc) {
+                        int32_t* desc, int pad_leading = 0) {
   const int G = kv.num_groups();
   const int B = kv.block_size();
   int T = 0, R = 0, max_ctx = 0, max_run = 0;
@@ -67,7 +70,11 @@ inline void build_batch(const KVManager& kv, const std::vector<BatchEntry>& entr
       widest[g] = std::max(widest[g], need);
     }
   }
-  const int S = static_cast<int>(entries.size());
+  int leading = 0;
+  while (leading < static_cast<int>(entries.size()) && entries[leading].count == 1) ++leading;
+  const int filler = std::max(pad_leading - leading, 0);   // padding sequences after the leading single rows
+  T += filler;
+  const int S = static_cast<int>(entries.size()) + filler;
   const int Tp = std::max(T, pad_rows), Sp = std::max(S, pad_seqs), Rp = std::max(R, pad_logit_rows);
   for (int g = 0; g < G; ++g) {
     if (table_stride > 0) {
@@ -114,8 +121,14 @@ inline void build_batch(const KVManager& kv, const std::vector<BatchEntry>& entr
   for (int s = 0; s < Sp; ++s) out[o_state + s] = -1;
 
   int row = 0, lrow = 0;
-  for (int s = 0; s < S; ++s) {
-    const BatchEntry& e = entries[s];
+  for (int s = 0, next = 0; s < S; ++s) {
+    if (s >= leading && s < leading + filler) {   // a padding sequence of one padding row
+      out[o_run + s] = row;
+      out[o_rseq + row] = s;
+      ++row;
+      continue;
+    }
+    const BatchEntry& e = entries[next++];
     const Sequence& q = *e.seq;
     out[o_run + s] = row;
     out[o_sstart + s] = e.start;

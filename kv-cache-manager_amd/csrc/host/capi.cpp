@@ -341,21 +341,28 @@ int kvcm_sched_plan(void* c, int64_t* ids, int32_t* start, int32_t* count, int32
   }));
 }
 // Runs the scheduler and says what it planned without handing the entries over:
-// out = {entries, prompt tokens, decoding sequences, entries that sample, 1 if every entry is a
-// single token that samples (a decode-shaped step), the longest context a row of the step sees}.
+// out[0..9] = {entries, prompt tokens, decoding sequences, entries that sample, 1 if every entry is a
+// single token that samples (a decode-shaped step), the longest context a row of the step sees,
+// rows in all, leading entries of one token, the longest run, 0}.
 int kvcm_sched_schedule_summary(void* c, double now, int64_t* out) {
   return static_cast<int>(guarded([&]() -> int64_t {
     const auto& plan = static_cast<Core*>(c)->sched->schedule(now);
-    int64_t prefill = 0, decode = 0, sampling = 0, single = 1, longest = 0;
+    int64_t prefill = 0, decode = 0, sampling = 0, single = 1, longest = 0, rows = 0, leading = 0, run = 0;
+    bool still_leading = true;
     for (const auto& p : plan) {
       if (p.is_prefill) prefill += p.num_tokens; else ++decode;
       if (p.samples) ++sampling;
       if (p.num_tokens != 1 || !p.samples) single = 0;
       if (p.start + p.num_tokens > longest) longest = p.start + p.num_tokens;
+      rows += p.num_tokens;
+      if (p.num_tokens > run) run = p.num_tokens;
+      if (p.num_tokens != 1) still_leading = false;
+      if (still_leading) ++leading;
     }
     out[0] = static_cast<int64_t>(plan.size()); out[1] = prefill; out[2] = decode; out[3] = sampling;
     out[4] = plan.empty() ? 0 : single;
     out[5] = longest;   // the longest context any row of the step sees
+    out[6] = rows; out[7] = leading; out[8] = run; out[9] = 0;
     return static_cast<int64_t>(plan.size());
   }));
 }
@@ -449,6 +456,34 @@ int kvcm_build_batch(void* c, int n, const int64_t* ids, const int32_t* start, c
 }
 
 // The scheduler's current plan; logits are wanted at the last row of every entry that samples.
+static void plan_entries(Core* core, std::vector<BatchEntry>& entries) {
+  for (const auto& p : core->sched->plan()) {
+    BatchEntry e;
+    e.seq = p.seq;
+    e.start = p.start;
+    e.count = p.num_tokens;
+    if (p.samples) e.want = {p.num_tokens - 1};
+    e.temperature = p.seq->temperature;
+    e.sampler_seed = p.seq->sampler_seed;
+    e.request_id = p.seq->id;
+    e.token_index = p.seq->num_generated();
+    entries.push_back(std::move(e));
+  }
+}
+
+// As kvcm_build_batch_from_plan, padded to a recorded step's shape: `pad_leading` single-row
+// sequences first (see build_batch).
+int kvcm_build_batch_from_plan_shaped(void* c, int pad_rows, int pad_seqs, int pad_logit_rows, int table_stride,
+                                      int pad_leading, int32_t* out, int64_t cap, int32_t* desc) {
+  return static_cast<int>(guarded([&]() -> int64_t {
+    auto* core = static_cast<Core*>(c);
+    std::vector<BatchEntry> entries;
+    plan_entries(core, entries);
+    build_batch(*core->kv, entries, pad_rows, pad_seqs, pad_logit_rows, table_stride, out, cap, desc, pad_leading);
+    return desc[kTotalInts];
+  }));
+}
+
 int kvcm_build_batch_from_plan(void* c, int pad_rows, int pad_seqs, int pad_logit_rows, int table_stride,
                                int32_t* out, int64_t cap, int32_t* desc) {
   return static_cast<int>(guarded([&]() -> int64_t {

@@ -35,15 +35,25 @@ class Engine:
         self.sampler = Sampler(self.runner.ops, self.runner.device, self.runner.limits.max_logit_rows)
         self._next_id = 0
         self._score_id = -1
+        self._forced, self._forced_logits = {}, {}       # request id -> forced tokens / logits kept for them
         self._t0 = time.perf_counter()
         self.config = self.runner.engine_config      # as built (max_seq_len within the model's range)
-        # Recorded steps (graphs) replay a fixed launch sequence: only for models whose parts all
-        # declare that their launches depend on the step's shape alone (Part.capturable).
-        self.decode_graphs = None
-        self.programs = None
-        if self.config.use_graphs and self.model.capturable:
-            from .graphs import DecodeGraphs
-            self.decode_graphs = DecodeGraphs(self)
+        # Recorded steps replay a fixed launch sequence: only for models whose parts all declare that
+        # their launches depend on the step's shape alone (Part.capturable).  use_programs: steps are
+        # recorded per shape and replayed natively; use_graphs: decode-shaped ones also as HIP graphs.
+        self.recorded = None
+        if (self.config.use_programs or self.config.use_graphs) and self.model.capturable:
+            from .graphs import RecordedSteps
+            self.recorded = RecordedSteps(self, use_graphs=self.config.use_graphs)
+
+    @property
+    def decode_graphs(self):
+        """The recorded-steps executor when it captures decode graphs, else None."""
+        return self.recorded if (self.recorded is not None and self.config.use_graphs) else None
+
+    @property
+    def programs(self):
+        return self.recorded if (self.recorded is not None and self.config.use_programs) else None
 
     # ------------------------------------------------------------------------------ clock
     def now(self) -> float:
@@ -54,7 +64,12 @@ class Engine:
 
     # --------------------------------------------------------------------------- requests
     def add_request(self, tokens: Sequence[int], max_new_tokens: int, temperature: float = 0.0, seed: int = 0,
-                    request_id: Optional[int] = None, arrival: Optional[float] = None) -> int:
+                    request_id: Optional[int] = None, arrival: Optional[float] = None,
+                    forced: Optional[Sequence[int]] = None) -> int:
+        """``forced``: the tokens this request "generates", given instead of sampled (teacher forcing):
+        the request runs through admission, portions, preemption and prefix hits like any other, every
+        sampled id is replaced by the next forced token, and ``forced_logits`` returns what it was
+        sampled from.  max_new_tokens is then len(forced)."""
         if request_id is None:
             request_id = self._next_id
         self._next_id = max(self._next_id, request_id + 1)
@@ -64,6 +79,12 @@ class Engine:
             raise ValueError("a request needs at least one token")
         if min(toks) < 0 or max(toks) >= V:
             raise ValueError(f"token id outside the vocabulary of {V}")
+        if forced is not None:
+            forced = [int(t) for t in forced]
+            if not forced or min(forced) < 0 or max(forced) >= V:
+                raise ValueError("forced tokens must be a non-empty list of ids inside the vocabulary")
+            max_new_tokens = len(forced)
+            self._forced[request_id], self._forced_logits[request_id] = forced, {}
         self.core.sched_add(request_id, toks, int(max_new_tokens), float(temperature), int(seed),
                             self.now() if arrival is None else arrival)
         return request_id
@@ -80,25 +101,70 @@ class Engine:
     def step(self) -> StepInfo:
         info = StepInfo()
         t_start = self.now()
-        n, info.prefill_tokens, info.decode_seqs, sampling, decode_shaped = self.core.schedule_summary(t_start)
-        if n == 0:
-            return info
-        if self.decode_graphs is not None and decode_shaped and self.decode_graphs.fits(n):
-            ids = self.decode_graphs.run(n)
-            info.rows = info.seqs = n
+        rec, forcing = self.recorded, bool(self._forced)
+        ids = None
+        if rec is None:
+            n, info.prefill_tokens, info.decode_seqs, sampling, _ = self.core.schedule_summary(t_start)
+            if n:
+                ids = self._step_direct(info, sampling)
         else:
-            layout = self.core.build_batch_from_plan(self.runner.host_buffer())
-            logits = self.runner.execute(layout)
-            info.rows, info.seqs = layout.rows, layout.seqs
-            ids = np.zeros(0, dtype=np.int32)
-            if sampling:
-                ids = self.sampler.sample_on_device(logits, self.runner.last_step.sampling_params())
-            else:
-                torch.cuda.current_stream().synchronize()
-        t_end = self.now()
-        self.core.update_sampled(ids, t_end)
-        info.ms = (t_end - t_start) * 1e3
+            n, info.prefill_tokens, info.decode_seqs, sampling = rec.plan(t_start)
+            if n:
+                # (with use_programs off only the decode-shaped steps that become graphs are recorded)
+                wanted = rec.shape is not None and (self.config.use_programs or rec.wants_graph)
+                ran = rec.replay(t_start, defer_update=forcing) if (wanted and rec.has_program) else None
+                if ran is not None:      # the native engine ran the step (and, unless deferred, the update)
+                    info.rows, info.seqs, ids = ran
+                elif wanted:
+                    layout, ids = rec.record(sampling)
+                    info.rows, info.seqs = layout.rows, layout.seqs
+                else:
+                    with torch.cuda.stream(rec.stream):
+                        ids = self._step_direct(info, sampling)
+        if ids is not None:
+            if forcing:
+                ids = self._force(ids)
+            self.core.update_sampled(ids, self.now())
+        info.ms = (self.now() - t_start) * 1e3
         return info
+
+    def _step_direct(self, info: StepInfo, sampling: int) -> np.ndarray:
+        """The planned step through the model's parts, launch by launch; -> the sampled ids."""
+        layout = self.core.build_batch_from_plan(self.runner.host_buffer())
+        logits = self.runner.execute(layout)
+        info.rows, info.seqs = layout.rows, layout.seqs
+        if sampling:
+            return self.sampler.sample_on_device(logits, self.runner.last_step.sampling_params())
+        torch.cuda.current_stream().synchronize()
+        return np.zeros(0, dtype=np.int32)
+
+    def _force(self, ids: np.ndarray) -> np.ndarray:
+        """Teacher forcing: the step's sampled ids are replaced by the tokens the request brought, and
+        the logits they were sampled from are kept (src/main_correct.cpp:194-222 scores given tokens
+        the same way, one whole sequence at a time)."""
+        R = len(ids)
+        if R == 0:
+            return ids
+        rows = self.runner.workspace.get("logits", (R, self.model.spec.vocab_size), torch.float32).cpu().numpy()
+        out, k = ids.copy(), 0
+        for p in self.core.plan():
+            if not p.samples:
+                continue
+            given = self._forced.get(p.id)
+            if given is not None:
+                self._forced_logits[p.id][p.gen_index] = rows[k].copy()
+                out[k] = given[p.gen_index]
+            k += 1
+        return out
+
+    def forced_logits(self, request_id: int) -> np.ndarray:
+        """Of a request added with ``forced``: the logits each of its forced tokens was to be sampled
+        from, [len(forced), vocab] (a row of NaN where none has been computed yet)."""
+        n, V = len(self._forced[request_id]), self.model.spec.vocab_size
+        out = np.full((n, V), np.nan, dtype=np.float32)
+        for k, row in self._forced_logits[request_id].items():
+            out[k] = row
+        return out
 
     def run_until_idle(self, max_steps: int = 1 << 30) -> List[Finished]:
         done = []
@@ -133,7 +199,10 @@ class Engine:
             self.core.admit(sid)
             try:
                 layout = self.core.build_batch([(sid, 0, len(toks), list(range(len(toks))))], self.runner.host_buffer())
-                return self.runner.execute_to_host(layout)
+                if self.recorded is None:
+                    return self.runner.execute_to_host(layout)
+                with torch.cuda.stream(self.recorded.stream):      # the stream every step of this engine runs on
+                    return self.runner.execute_to_host(layout)
             finally:
                 self.core.release(sid)
         finally:

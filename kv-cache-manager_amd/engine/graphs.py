@@ -1,27 +1,32 @@
-"""Decode-only steps replayed from captured HIP graphs.
+"""Recorded steps: the Python side of the native step loop (csrc/hip/native_engine.hip).
 
-A step in which every scheduled request computes exactly one token has a fixed shape once the
-batch is padded to a bucket size: the same kernels on the same buffers, only the integers in the
-metadata buffer change.  Such a step is captured once per bucket (model step + sampling) and
-replayed afterwards, which removes a few hundred launches' worth of host time per step (the
-reference launches every kernel of every step from the host, src/model/llama.cpp:104-129).
+A step of a model whose parts are all capturable is a fixed list of kernel launches once its shape
+is fixed: the same kernels on the same buffers, only the integers in the metadata buffer change.
+The first step of a shape runs through the parts while every launch is recorded into a step program
+(model step + sampling); later steps of that shape never reach Python's part code: the native engine
+schedules, builds and uploads the metadata, replays the program, downloads the sampled ids and
+updates the scheduler (the reference launches every kernel of every step from its C++ step function,
+src/model/llama.cpp:104-129, inside Engine::step, src/engine/engine.cpp:73-90).
 
-Padding rows have context length 0 and slot -1: they write no key, attend to nothing, and their
-sampled ids are dropped.  Nothing inside a graph clears memory or allocates.
-
-A captured launch must fit every step that replays it, so kernels that size their grid by the
-context are captured for a bound on it.  There is one graph per (bucket, context class): a step
-replays the graph of the smallest class that holds its longest context, so that an engine that
-allows long sequences still runs short ones with the launches made for short ones.
+Shapes are canonical (see native_engine.hip): padding rows have context length 0 and slot -1, they
+write no key, attend to nothing, and their sampled ids are dropped.  Decode-shaped steps (every
+request computes one token) of up to GRAPH_ROWS rows are additionally captured into a HIP graph, one
+per (batch bucket, context class): a launch must fit every step that replays it, so kernels that size
+their grid by the context are recorded for a bound on it, and a step replays the graph of the smallest
+class that holds its longest context.  Nothing inside a recorded step clears memory or allocates.
 """
 import contextlib
+import ctypes as C
 import gc
-from typing import Dict, List
+from dataclasses import dataclass
+from typing import Optional
 
 import numpy as np
 import torch
 
 from .runner import StepContext
+
+GRAPH_ROWS = 256     # decode-shaped steps of more rows replay their program without a graph
 
 
 @contextlib.contextmanager
@@ -30,97 +35,135 @@ def _no_collection():
     there may destroy device objects of an engine that is no longer used (its graphs, their memory
     pools), and releasing device memory during a capture ends the process."""
     was_enabled = gc.isenabled()
-    gc.disable()   # (torch.cuda.graph collects once itself before the capture begins)
+    gc.disable()
     try:
         yield
     finally:
         if was_enabled:
             gc.enable()
 
-_BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256, 384, 512)
-_CONTEXT_CLASSES = (1024, 2048, 8192, 32768)       # and the longest context the engine allows
+
+@dataclass(frozen=True)
+class StepShape:
+    """The canonical shape a step is recorded and replayed in."""
+    rows: int
+    seqs: int
+    leading: int            # single-token runs at the front (padded to a bucket)
+    logit_rows: int
+    max_run: int
+    context_bound: int
+    table_stride: int
 
 
-class DecodeGraphs:
-    def __init__(self, engine):
-        self.engine = engine
-        self.runner = engine.runner
-        self.core = engine.core
-        self.sampler = engine.sampler
+class RecordedStepContext(StepContext):
+    """The step as a recorded program may see it: every host integer is the shape's, not the
+    batch's, so that the launches fit every step of the shape."""
+
+    def __init__(self, runner, layout, shape: StepShape):
+        super().__init__(runner, layout)
+        assert (self.rows, self.seqs, self.logit_rows_padded) == (shape.rows, shape.seqs, shape.logit_rows)
+        self.real_rows, self.real_seqs, self.logit_rows = shape.rows, shape.seqs, shape.logit_rows
+        self.max_run = shape.max_run
+        self.max_context = self.max_context_bound = shape.context_bound
+        self._leading = shape.leading
+        self.recording = True
+
+
+class RecordedSteps:
+    def __init__(self, engine, use_graphs=True):
+        self.engine, self.runner, self.core, self.sampler = engine, engine.runner, engine.core, engine.sampler
+        ops = self.ops = self.runner.ops
+        self.lib = ops.lib()
         lim = self.runner.limits
-        self.buckets = [b for b in _BUCKETS if b <= min(lim.max_seqs, lim.max_logit_rows, lim.max_tokens)]
-        self.table_stride = lim.max_blocks_per_seq
-        self.block_size = engine.config.block_size
-        self.context_classes = [c for c in _CONTEXT_CLASSES if c < lim.max_context_len] + [lim.max_context_len]
-        self.graphs: Dict[tuple, torch.cuda.CUDAGraph] = {}      # (bucket, context class) -> graph
-        self._views = {}      # bucket -> (device view, pinned view, ints) of the metadata a replay uploads
-        self.enabled = bool(self.buckets)
+        self.stream = torch.cuda.Stream()          # default priority; every step of this engine runs on it
+        names = ("kvcm_sched_schedule_summary", "kvcm_build_batch_from_plan_shaped", "kvcm_sched_update_sampled",
+                 "kvcm_last_error")
+        fns = (C.c_uint64 * 4)(*[self.core.native_function(n) for n in names])
+        s = self.sampler
+        self._h = self.lib.kvcm_engine_new(
+            self.core.handle, fns, self.runner._pinned.data_ptr(), self.runner.meta_dev.data_ptr(), self.runner.meta_dev.numel(),
+            s.out.data_ptr(), s._host.data_ptr(), s.max_rows, self.core.num_groups, engine.config.block_size,
+            lim.max_context_len, lim.max_tokens, lim.max_seqs, lim.max_logit_rows, GRAPH_ROWS if use_graphs else 0,
+            self.stream.cuda_stream)
+        if not self._h:
+            raise ops.KernelError(self.lib.kvcm_hip_last_error().decode())
+        self._out = (C.c_int64 * 20)()
+        self._info = (C.c_int64 * 8)()
+        self.last_host_us = 0            # of the last replayed step: host time from scheduling to the last launch
+        self.shape: Optional[StepShape] = None
+        self.recorded_shapes = {}        # StepShape -> "graph" | "program"
+        torch.cuda.synchronize()         # weights and caches were written on other streams
 
-    def fits(self, n: int) -> bool:
-        """May a decode-shaped step of n sequences be replayed from a graph?"""
-        return self.enabled and 0 < n <= self.buckets[-1]
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self.lib.kvcm_engine_delete(self._h)
+            self._h = None
 
-    def usable(self, plan) -> bool:
-        return self.fits(len(plan)) and all(p.count == 1 and p.samples for p in plan)
+    # ------------------------------------------------------------------------------- one step
+    def plan(self, now: float):
+        """Runs the scheduler.  -> (entries, prompt tokens, decoding sequences, sampling entries); sets
+        ``shape`` (None when the plan fits no canonical shape), ``has_program`` and ``wants_graph``."""
+        o = self._out
+        n = self.lib.kvcm_engine_plan(self._h, float(now), o)
+        if n < 0:
+            raise self.ops.KernelError(self.lib.kvcm_hip_last_error().decode())
+        self.core.plan_max_context, self.core.plan_rows, self.core.plan_leading, self.core.plan_max_run = o[5], o[6], o[7], o[8]
+        self.shape = StepShape(*[int(o[k]) for k in range(11, 18)]) if o[10] else None
+        self.has_program, self.wants_graph = bool(o[18]), bool(o[19])
+        return n, int(o[1]), int(o[2]), int(o[3])
 
-    def _bucket(self, n: int) -> int:
-        for b in self.buckets:
-            if n <= b:
-                return b
-        raise RuntimeError("no bucket")
+    def replay(self, now: float, defer_update=False):
+        """The planned step from its program, natively, scheduler update included.  -> (rows, sequences,
+        sampled ids) or None when the shape has no program yet.  ``defer_update``: the update is left
+        to the caller, who gets the sampled ids (else the third value is None)."""
+        rc = self.lib.kvcm_engine_run(self._h, float(now), int(defer_update), self._info)
+        if rc < 0:
+            raise self.ops.KernelError(self.lib.kvcm_hip_last_error().decode())
+        if rc == 0:
+            return None
+        self.runner._upload_pending = False      # the native step waited for its stream
+        self.last_host_us = int(self._info[4])
+        ids = self.sampler._host[:int(self._info[2])].numpy().copy() if defer_update else None
+        return int(self._info[0]), int(self._info[1]), ids
 
-    def _context_class(self, context: int) -> int:
-        for c in self.context_classes:
-            if context <= c:
-                return c
-        raise RuntimeError(f"a context of {context} tokens exceeds what the engine allows")
+    def record(self, sampling: int):
+        """Runs the planned step through the model's parts on this engine's stream, recording every
+        launch, registers the program (captured as a graph where the shape wants one) and returns
+        (layout, sampled ids): this pass's results are the step's results."""
+        shape, runner, ops = self.shape, self.runner, self.ops
+        with torch.cuda.stream(self.stream), _no_collection():
+            layout = self.core.build_batch_from_plan(runner.host_buffer(), pad_rows=shape.rows, pad_seqs=shape.seqs,
+                                                     pad_logit_rows=shape.logit_rows, table_stride=shape.table_stride,
+                                                     pad_leading=shape.leading)
+            assert layout.max_context <= shape.context_bound
+            runner._check(layout)
+            runner.upload(layout)
+            step = RecordedStepContext(runner, layout, shape)
+            program = ops.StepProgram()
+            # only kernels of this package inside a graph: a library product may record nodes that
+            # clear memory, which do not replay reliably
+            keep = ops.LIBRARY_GEMM_MIN_ROWS
+            if self.wants_graph:
+                ops.LIBRARY_GEMM_MIN_ROWS = 0
+            try:
+                with ops.recording(program):
+                    logits = runner.model.forward(step)
+                    t, seeds, ids, idx = step.sampling_params()
+                    ops.sample(logits, self.sampler.out[:shape.logit_rows], t, seeds, ids, idx)
+            finally:
+                ops.LIBRARY_GEMM_MIN_ROWS = keep
+            sampled = self.sampler.download(sampling)
+            if self.lib.kvcm_engine_register(self._h, program.release(), int(self.wants_graph)) != 0:
+                raise ops.KernelError(self.lib.kvcm_hip_last_error().decode())
+            self.recorded_shapes[shape] = "graph" if self.wants_graph else "program"
+        return layout, sampled
 
-    def _forward(self, layout, bucket, bound):
-        """Only kernels of this package inside a graph: a library product may record nodes that
-        clear memory, which do not replay reliably."""
-        ops = self.runner.ops
-        keep, ops.LIBRARY_GEMM_MIN_ROWS = ops.LIBRARY_GEMM_MIN_ROWS, 0
-        try:
-            self._forward_inner(layout, bucket, bound)
-        finally:
-            ops.LIBRARY_GEMM_MIN_ROWS = keep
+    # ---------------------------------------------------------------------------------- info
+    def stats(self) -> dict:
+        out = (C.c_int64 * 4)()
+        self.lib.kvcm_engine_stats(self._h, out)
+        return dict(programs=int(out[0]), graphs=int(out[1]), steps_replayed=int(out[2]), steps_as_graph=int(out[3]))
 
-    def _forward_inner(self, layout, bucket, bound):
-        step = StepContext(self.runner, layout)
-        step.max_context_bound = bound
-        logits = self.runner.model.forward(step)
-        # the sampling parameters lie in the metadata buffer (padding rows: temperature 0, dropped)
-        t, seeds, ids, idx = step.sampling_params()
-        self.runner.ops.sample(logits, self.sampler.out[:bucket], t, seeds, ids, idx)
-
-    def run(self, n: int) -> np.ndarray:
-        """Runs the scheduler's current plan (n decode-shaped entries); returns the n sampled ids."""
-        bucket = self._bucket(n)
-        runner, s = self.runner, self.sampler
-        # the class also fixes how many page ids per sequence a replay uploads and reads
-        bound = self._context_class(max(self.core.plan_max_context, 1))
-        stride = min(self.table_stride, -(-bound // self.block_size))
-        layout = self.core.build_batch_from_plan(runner.host_buffer(), pad_rows=bucket, pad_seqs=bucket,
-                                                 pad_logit_rows=bucket, table_stride=stride)
-        assert layout.max_context <= bound
-        runner._check(layout)
-        views = self._views.get(bucket)
-        if views is None or views[2] != layout.total:
-            views = self._views[bucket] = (runner.meta_dev[:layout.total], runner._pinned[:layout.total], layout.total)
-        views[0].copy_(views[1], non_blocking=True)
-        # no event: the synchronous download below ends after this upload, so the pinned buffer
-        # is free again when the next step fills it
-        runner._upload_pending = False
-        graph = self.graphs.get((bucket, bound))
-        if graph is None:
-            # eager once: creates every work buffer, and its result is this step's result (a capture
-            # runs nothing, so the sampled ids stay where the eager pass left them)
-            self._forward(layout, bucket, bound)
-            torch.cuda.current_stream().synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with _no_collection(), torch.cuda.graph(graph):
-                self._forward(layout, bucket, bound)
-            self.graphs[(bucket, bound)] = graph
-            return s.download(n)
-        graph.replay()
-        return s.download(n)
+    def graph_shapes(self):
+        """(batch bucket, context class) of every captured decode graph."""
+        return sorted((s.rows, s.context_bound) for s, kind in self.recorded_shapes.items() if kind == "graph")

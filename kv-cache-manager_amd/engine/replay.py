@@ -93,6 +93,34 @@ class TraceReplayer:
         return logits
 
 
+def scheduled_replay(engine, requests, arrivals=None, max_steps=1 << 20):
+    """The second way to replay given tokens: through the engine's own scheduler.  Each request is
+    (prompt tokens, continuation tokens): it is admitted, cut into portions, preempted and served
+    from prefix hits as the engine's options decide, and wherever a token would be sampled the next
+    token of the continuation is pushed instead (the sampled id is ignored).  Returns, per request in
+    order, the logits those tokens were to be sampled from: [len(continuation), vocab], i.e. the
+    logits at positions len(prompt) - 1 .. len(prompt) + len(continuation) - 2 of the whole sequence.
+    The reference scores given tokens one whole sequence at a time (src/main_correct.cpp:194-222)
+    and generates through add/step/take_finished (main_correct.cpp:61-80); this does both at once.
+
+    arrivals[i]: the step before which request i is added (default: all before the first step)."""
+    arrivals = list(arrivals) if arrivals is not None else [0] * len(requests)
+    order = sorted(range(len(requests)), key=lambda i: (arrivals[i], i))
+    ids, nxt, steps = {}, 0, 0
+    while nxt < len(order) or not engine.idle():
+        while nxt < len(order) and arrivals[order[nxt]] <= steps:
+            i = order[nxt]
+            prompt, continuation = requests[i]
+            ids[i] = engine.add_request(prompt, len(continuation), forced=continuation)
+            nxt += 1
+        engine.step()
+        engine.take_finished()
+        steps += 1
+        if steps > max_steps:
+            raise ReplayError("scheduled_replay: the engine does not come to an end")
+    return [engine.forced_logits(ids[i]) for i in range(len(requests))]
+
+
 def main(argv=None):
     import argparse
     ap = argparse.ArgumentParser(prog="trace_run", description="replay given token ids step by step and write logits")

@@ -199,12 +199,16 @@ class ModelRunner:
         if layout.rows and (toks.min() < 0 or toks.max() >= self.vocab_size):
             raise ValueError(f"step: token id outside the vocabulary of {self.vocab_size}")
 
-    def _begin(self, layout: BatchLayout, logits_in_portions=False) -> StepContext:
-        self._check(layout, logits_in_portions)
+    def upload(self, layout: BatchLayout):
+        """The one host-to-device copy of a step: its packed metadata."""
         n = layout.total
         self.meta_dev[:n].copy_(self._pinned[:n], non_blocking=True)
         self._upload_done.record()
         self._upload_pending = True
+
+    def _begin(self, layout: BatchLayout, logits_in_portions=False) -> StepContext:
+        self._check(layout, logits_in_portions)
+        self.upload(layout)
         return StepContext(self, layout)
 
     def execute(self, layout: BatchLayout) -> Optional[torch.Tensor]:

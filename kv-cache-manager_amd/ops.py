@@ -3,6 +3,7 @@ the host that their shapes and dtypes are what the kernel assumes, and launches 
 current stream.  There is no fallback: without the library (or without a GPU) these raise.
 """
 import ctypes as C
+import struct as _struct
 import threading
 
 import torch
@@ -64,6 +65,25 @@ def _declare(lib):
     lib.kvcm_attention_decode_scratch.restype = C.c_longlong
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
+    fn("kvcm_gemm_library", vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, vp)
+    lib.kvcm_gemm_library_workspace_bytes.restype = C.c_longlong
+    lib.kvcm_gemm_library_workspace_bytes.argtypes = []
+    lib.kvcm_program_new.restype = vp
+    lib.kvcm_program_new.argtypes = []
+    lib.kvcm_program_delete.restype = None
+    lib.kvcm_program_delete.argtypes = [vp]
+    fn("kvcm_program_add", vp, C.c_char_p, C.POINTER(C.c_uint64), i)
+    fn("kvcm_program_size", vp)
+    fn("kvcm_program_run", vp, vp)
+    lib.kvcm_engine_new.restype = vp
+    lib.kvcm_engine_new.argtypes = [vp, C.POINTER(C.c_uint64), vp, vp, C.c_longlong, vp, vp, i, i, i, i, i, i, i, i, vp]
+    lib.kvcm_engine_delete.restype = None
+    lib.kvcm_engine_delete.argtypes = [vp]
+    fn("kvcm_engine_plan", vp, C.c_double, C.POINTER(C.c_int64))
+    fn("kvcm_engine_register", vp, vp, i)
+    fn("kvcm_engine_run", vp, C.c_double, i, C.POINTER(C.c_int64))
+    lib.kvcm_engine_stats.restype = None
+    lib.kvcm_engine_stats.argtypes = [vp, C.POINTER(C.c_int64)]
 
 
 def lib():
@@ -95,6 +115,81 @@ def _stream():
 def _check(rc):
     if rc != 0:
         raise KernelError(lib().kvcm_hip_last_error().decode())
+
+
+# ------------------------------------------------------------------------------ recorded steps
+class StepProgram:
+    """The launches of one step, kept natively (csrc/hip/step_program.hip): every launching entry that
+    is called while a program records is appended to it with its arguments, and ``run`` calls the same
+    entries again without Python.  Whoever registers the program with the native engine hands its
+    ownership over (``release``)."""
+
+    def __init__(self):
+        self._h = lib().kvcm_program_new()
+
+    def __len__(self):
+        return lib().kvcm_program_size(self._h)
+
+    def add(self, name, slots):
+        arr = (C.c_uint64 * len(slots))(*slots)
+        _check(lib().kvcm_program_add(self._h, name.encode(), arr, len(slots)))
+
+    def run(self, stream=None):
+        _check(lib().kvcm_program_run(self._h, _stream() if stream is None else stream))
+
+    def release(self):
+        h, self._h = self._h, None
+        return h
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().kvcm_program_delete(self._h)
+            self._h = None
+
+
+_recording = None      # the StepProgram that launches are appended to, while one records
+_MASK64 = (1 << 64) - 1
+
+
+class recording:
+    """``with ops.recording(program): ...``: every launch inside also goes into ``program``.  Anything a
+    step does that is not a launching entry of this library (a tensor library's routine, an allocation)
+    would be missing from the replay: parts that do such things are not capturable."""
+
+    def __init__(self, program):
+        self.program = program
+
+    def __enter__(self):
+        global _recording
+        if _recording is not None:
+            raise RuntimeError("a step program is already recording")
+        _recording = self.program
+        return self.program
+
+    def __exit__(self, *exc):
+        global _recording
+        _recording = None
+        return False
+
+
+def _slots(fn, args):
+    out = []
+    for t, a in zip(fn.argtypes, args):
+        if t is C.c_float:
+            out.append(_struct.unpack("<I", _struct.pack("<f", a))[0])
+        elif a is None:
+            out.append(0)
+        else:
+            out.append(int(a) & _MASK64)
+    return out
+
+
+def _call(name, *args):
+    """Calls a launching entry; while a program records, notes the call there first."""
+    fn = getattr(lib(), name)
+    if _recording is not None:
+        _recording.add(name, _slots(fn, args))
+    _check(fn(*args))
 
 
 def _ptr(t):
@@ -132,7 +227,7 @@ def embed(ids, table, out):
     _i32(ids, "ids", T)
     _need(table.dim() == 2 and table.shape[1] == H and table.is_contiguous(), "embedding table must be [V, H]")
     _need(out.dtype == torch.float32 and out.is_contiguous(), "residual stream must be contiguous float32")
-    _check(lib().kvcm_embed(_ptr(ids), _ptr(table), _DT[table.dtype], _ptr(out), T, H, table.shape[0], _stream()))
+    _call("kvcm_embed", _ptr(ids), _ptr(table), _DT[table.dtype], _ptr(out), T, H, table.shape[0], _stream())
 
 
 class PartialSums:
@@ -146,8 +241,8 @@ class PartialSums:
 
     def materialize(self):
         """Adds the splits up into the product's own output buffer [rows, cols] and returns it."""
-        _check(lib().kvcm_reduce_store(_ptr(self.data), _ptr(self.out), _DT[self.out.dtype], self.rows, self.cols,
-                                       self.out.stride(0), self.splits, _stream()))
+        _call("kvcm_reduce_store", _ptr(self.data), _ptr(self.out), _DT[self.out.dtype], self.rows, self.cols,
+                                       self.out.stride(0), self.splits, _stream())
         return self.out
 
 
@@ -170,10 +265,10 @@ def rmsnorm(x, weight, out, eps, add=None, rows=None, write_back=True):
     if add is not None:
         _need(add.shape == x.shape and add.is_contiguous(), "add must match x")
     wb = bool(write_back) and (add is not None or partial is not None) and rows is None
-    _check(lib().kvcm_rmsnorm(_ptr(x), _ptr(add), _DT[add.dtype] if add is not None else 0,
+    _call("kvcm_rmsnorm", _ptr(x), _ptr(add), _DT[add.dtype] if add is not None else 0,
                               _ptr(partial.data) if partial else 0, partial.splits if partial else 0,
                               partial.rows if partial else 0, _ptr(rows), _ptr(weight),
-                              _DT[weight.dtype], _ptr(out), _DT[out.dtype], R, H, float(eps), int(wb), _stream()))
+                              _DT[weight.dtype], _ptr(out), _DT[out.dtype], R, H, float(eps), int(wb), _stream())
 
 
 def rope_table(positions, inv_freq, out, rows=None):
@@ -185,7 +280,7 @@ def rope_table(positions, inv_freq, out, rows=None):
     _need(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous(), "inv_freq must be float32")
     _need(out.dtype == torch.float32 and out.is_contiguous() and out.dim() == 3 and out.shape[1] == inv_freq.numel()
           and out.shape[2] == 2 and out.shape[0] >= T, "the table must be float32 [rows, head_dim/2, 2]")
-    _check(lib().kvcm_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(out), T, inv_freq.numel(), _stream()))
+    _call("kvcm_rope_table", _ptr(positions), _ptr(inv_freq), _ptr(out), T, inv_freq.numel(), _stream())
     return out
 
 
@@ -218,10 +313,10 @@ def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcac
               and tuple(kcache.shape[1:]) == (nkv, block_size, hd), "key cache must be [pages, nkv, block_size, hd]")
         _need(vcache is not None and vcache.dtype == qkv.dtype and vcache.is_contiguous() and vcache.dim() == 4
               and tuple(vcache.shape[1:]) == (nkv, hd, block_size), "value cache must be [pages, nkv, hd, block_size]")
-    _check(lib().kvcm_rope_cache(_ptr(qkv), _DT[qkv.dtype], qkv.stride(0), _ptr(positions), _ptr(inv_freq),
+    _call("kvcm_rope_cache", _ptr(qkv), _DT[qkv.dtype], qkv.stride(0), _ptr(positions), _ptr(inv_freq),
                                  _ptr(slots), _ptr(kcache), _ptr(vcache), T, nh, nkv, hd, block_size,
                                  _ptr(source.data) if source is not None else 0,
-                                 source.splits if source is not None else 0, _ptr(cos_sin), _stream()))
+                                 source.splits if source is not None else 0, _ptr(cos_sin), _stream())
 
 
 def swiglu(gate_up, out):
@@ -229,23 +324,35 @@ def swiglu(gate_up, out):
     T, I = out.shape
     _need(gate_up.shape == (T, 2 * I) and gate_up.is_contiguous() and out.is_contiguous()
           and gate_up.dtype == out.dtype, "swiglu needs [T, 2I] -> [T, I] of one dtype")
-    _check(lib().kvcm_swiglu(_ptr(gate_up), _ptr(out), _DT[out.dtype], T, I, _stream()))
+    _call("kvcm_swiglu", _ptr(gate_up), _ptr(out), _DT[out.dtype], T, I, _stream())
 
 
 def add_residual(x, y):
     _dev(x, y)
     _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape,
           "add_residual needs a float32 x and a y of the same shape")
-    _check(lib().kvcm_add_residual(_ptr(x), _ptr(y), _DT[y.dtype], x.numel(), _stream()))
+    _call("kvcm_add_residual", _ptr(x), _ptr(y), _DT[y.dtype], x.numel(), _stream())
 
 
-# Rows from which a bfloat16 product is handed to the library (hipBLASLt through torch.matmul); the
-# reference leaves every product to its vendor library.  0 = always use the kernels of this package.
-# Below, the weight-streaming kernels of this package run: on the GPU the library wins from about
-# 128 rows on, but a call through torch costs the host about 15 us against 5 us for a kernel of
-# this package, and a step of a few hundred rows (88 products) is bound by the host: measured
-# end to end, a prompt portion is faster with this package's kernels up to about 300 rows.
-LIBRARY_GEMM_MIN_ROWS = 320
+# Rows from which a bfloat16 product is handed to the library (hipBLASLt, called directly:
+# csrc/hip/gemm_library.hip); the reference leaves every product to its vendor library.  0 = always
+# use the kernels of this package.  Below, the weight-streaming kernels of this package run.  Measured
+# end to end at TinyLlama sizes (steps of 16 decoding rows beside a prompt portion, replayed from
+# recorded programs, so that a call costs the host the same either way): 48 rows 2.03 ms with this
+# package's kernels against 2.24 with the library's, 80 rows 2.05 / 2.26, 112 rows 2.83 / 2.61,
+# 176 rows 2.85 / 2.56, 336 rows 3.85 / 2.98.
+LIBRARY_GEMM_MIN_ROWS = 96
+
+
+_library_ws = None
+
+
+def _library_workspace(device):
+    """Device memory the vendor library's product may use (one buffer, kept: recorded steps hold its address)."""
+    global _library_ws
+    if _library_ws is None:
+        _library_ws = torch.empty(lib().kvcm_gemm_library_workspace_bytes(), dtype=torch.uint8, device=device)
+    return _library_ws
 
 
 def skinny_splits(M, N, K):
@@ -270,7 +377,7 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
     _need(w.shape[1] == K and out.shape == (M, N), f"gemm shapes do not agree: {tuple(x.shape)} {tuple(w.shape)} {tuple(out.shape)}")
     if x.dtype == torch.float32:
         _need(w.dtype == torch.float32 and out.dtype == torch.float32, "a float32 gemm needs float32 operands")
-        _check(lib().kvcm_gemm_f32(_ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0), _stream()))
+        _call("kvcm_gemm_f32", _ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0), _stream())
         return out
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm operands must both be bfloat16")
     library = bool(LIBRARY_GEMM_MIN_ROWS) and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 and out.is_contiguous()
@@ -281,17 +388,19 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
     if S >= 1:
         if S > 1:
             _need(scratch.dtype == torch.float32 and scratch.is_contiguous() and scratch.is_cuda, "scratch must be float32")
-        _check(lib().kvcm_gemm_skinny(_ptr(x), _ptr(w), _ptr(scratch) if S > 1 else 0, _ptr(out), _DT[out.dtype], M, N, K,
-                                      x.stride(0), w.stride(0), out.stride(0), S, _stream()))
+        _call("kvcm_gemm_skinny", _ptr(x), _ptr(w), _ptr(scratch) if S > 1 else 0, _ptr(out), _DT[out.dtype], M, N, K,
+                                      x.stride(0), w.stride(0), out.stride(0), S, _stream())
         if S == 1:
             return out
         partial = PartialSums(scratch, S, M, N, out)
         return partial if keep_partial else partial.materialize()
     if library:
-        torch.matmul(x, w.t(), out=out)
+        ws = _library_workspace(out.device)
+        _call("kvcm_gemm_library", _ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0),
+              _ptr(ws), ws.numel(), _stream())
         return out
-    _check(lib().kvcm_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, x.stride(0), w.stride(0),
-                                out.stride(0), _stream()))
+    _call("kvcm_gemm_bf16", _ptr(x), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, x.stride(0), w.stride(0),
+                                out.stride(0), _stream())
     return out
 
 
@@ -311,8 +420,8 @@ def gemm_swiglu(x, w_gate_up, out):
             and w_gate_up.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
             and lib().kvcm_gemm_skinny_swiglu_supported(M, I, K)):
         return False
-    _check(lib().kvcm_gemm_skinny_swiglu(_ptr(x), _ptr(w_gate_up), _ptr(out), _DT[out.dtype], M, I, K, x.stride(0),
-                                         w_gate_up.stride(0), out.stride(0), _stream()))
+    _call("kvcm_gemm_skinny_swiglu", _ptr(x), _ptr(w_gate_up), _ptr(out), _DT[out.dtype], M, I, K, x.stride(0),
+                                         w_gate_up.stride(0), out.stride(0), _stream())
     return True
 
 
@@ -339,9 +448,9 @@ def attention(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_lens, n
     _i32(row_seq, "row_seq", T)
     _i32(ctx_lens, "ctx_lens", T)
     _i32(tables, "tables")
-    _check(lib().kvcm_attention_generic(_ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache),
+    _call("kvcm_attention_generic", _ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache),
                                         _ptr(vcache), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh,
-                                        nkv, hd, kcache.shape[2], float(scale), int(window), _stream()))
+                                        nkv, hd, kcache.shape[2], float(scale), int(window), _stream())
 
 
 def attention_decode_supported(nh, nkv, hd, dtype, block_size=16):
@@ -380,10 +489,10 @@ def attention_decode(q, out, kcache, vcache, tables, table_stride, row_seq, ctx_
     _i32(row_seq, "row_seq", T)
     _i32(ctx_lens, "ctx_lens", T)
     _i32(tables, "tables")
-    _check(lib().kvcm_attention_decode(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
+    _call("kvcm_attention_decode", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
                                        _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh, nkv, hd,
                                        kcache.shape[2], float(scale), int(max_context), _ptr(scratch), scratch.numel(),
-                                       _stream()))
+                                       _stream())
 
 
 def attention_decode_fused_supported(nh, nkv, hd, dtype, block_size=16):
@@ -428,16 +537,17 @@ def attention_decode_fused(projection, out, kcache, vcache, tables, table_stride
     _need(out.shape[0] >= T and out.shape[1] >= nh * hd, "out must be [rows, nh * hd]")
     need = attention_decode_fused_scratch(T, nh, nkv, hd, int(max_context))
     if need and scratch is None:
+        _need(_recording is None, "attention_decode_fused: a recorded step must bring its scratch (an allocation here would not outlive the step)")
         scratch = torch.empty(need, dtype=torch.float32, device=out.device)
     if scratch is not None:
         _dev(scratch)
         _need(scratch.dtype == torch.float32 and scratch.is_contiguous(), "scratch must be contiguous float32")
-    _check(lib().kvcm_attention_decode_fused(
+    _call("kvcm_attention_decode_fused", 
         _ptr(projection.data) if partial else 0, projection.splits if partial else 0,
         0 if partial else _ptr(rows_t), 0 if partial else rows_t.stride(0), _ptr(cos_sin), _ptr(slots), _ptr(kcache),
         _ptr(vcache), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), T, nh, nkv, hd, kcache.shape[2],
         float(scale), _ptr(out), out.stride(0), int(max_context), _ptr(scratch),
-        scratch.numel() if scratch is not None else 0, _stream()))
+        scratch.numel() if scratch is not None else 0, _stream())
 
 
 def attention_prefill_supported(nh, nkv, hd, dtype, block_size=16):
@@ -474,6 +584,7 @@ def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, s
         max_context = table_stride * kcache.shape[2]
     need = attention_prefill_scratch(T, nh, hd, max_context, max_run, num_seqs)
     if need and scratch is None:
+        _need(_recording is None, "attention_prefill: a recorded step must bring its scratch (an allocation here would not outlive the step)")
         scratch = torch.empty(need, dtype=torch.float32, device=q.device)
     if scratch is not None:
         _need(scratch.dtype == torch.float32 and scratch.is_contiguous(), "scratch must be contiguous float32")
@@ -484,10 +595,10 @@ def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, s
     _i32(run_start, "run_start", num_seqs + 1)
     _i32(seq_start, "seq_start", num_seqs)
     _i32(tables, "tables", num_seqs * table_stride)
-    _check(lib().kvcm_attention_prefill(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
+    _call("kvcm_attention_prefill", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
                                         _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), num_seqs, max_run,
                                         T, int(max_context), nh, nkv, hd, kcache.shape[2], float(scale), _ptr(scratch),
-                                        scratch.numel() if scratch is not None else 0, _stream()))
+                                        scratch.numel() if scratch is not None else 0, _stream())
 
 
 def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_index=None):
@@ -502,5 +613,5 @@ def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_in
         _need(seeds is not None and seeds.dtype in (torch.int64, torch.uint64) and seeds.numel() >= R, "seeds must be 64-bit [R]")
         _need(request_ids is not None and request_ids.dtype == torch.int64 and request_ids.numel() >= R, "request ids must be int64 [R]")
         _i32(token_index, "token_index", R)
-    _check(lib().kvcm_sample(_ptr(logits), logits.stride(0), _ptr(temperature), _ptr(seeds), _ptr(request_ids),
-                             _ptr(token_index), _ptr(out), R, V, _stream()))
+    _call("kvcm_sample", _ptr(logits), logits.stride(0), _ptr(temperature), _ptr(seeds), _ptr(request_ids),
+                             _ptr(token_index), _ptr(out), R, V, _stream())

@@ -70,7 +70,7 @@ static int run(int policy, int groups, int block_size, int blocks, bool prefix, 
   int added = 6;
   while (true) {
     if (added < requests && rng() % 3 == 0) { add(); ++added; }
-    int64_t sum[6];
+    int64_t sum[10];
     const int n = kvcm_sched_schedule_summary(core, double(steps), sum);
     CHECK(n >= 0, "schedule");
     if (n == 0) {

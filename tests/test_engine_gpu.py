@@ -17,6 +17,8 @@ def _engine(d, **kw):
     from kvcm_amd import Engine, EngineConfig
     base = dict(block_size=16, num_blocks=64, max_seq_len=256, max_num_seqs=8, max_batched_tokens=256, dtype="float32")
     base.update(kw)
+    if base.get("use_graphs") is False:            # "no graphs" in these tests means: every step launch by launch
+        base.setdefault("use_programs", False)
     return Engine(d, EngineConfig(**base))
 
 
@@ -107,7 +109,10 @@ def test_mixed_steps_at_matrix_core_sizes(tmp_path, raw, chunk, budget, sharpen)
     H.make_model_dir(d, raw, H.WEIGHT_SEED["D"], torch.bfloat16, sharpen=sharpen)
     pm = plain.load_model_dir(d, plain.round_bf16)
     prompts = _prompts(raw, [40, 12, 700, 90, 1200, 25], seed=9)
-    eng = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, prefill_chunk=chunk, max_batched_tokens=budget)
+    # (steps launch by launch, so that the kernels each step takes can be counted here; recorded steps
+    # have a test of their own below)
+    eng = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, prefill_chunk=chunk, max_batched_tokens=budget,
+                  use_programs=False)
     ids = [eng.add_request(p, 10) for p in prompts]
     qkv_width = (raw["num_attention_heads"] + 2 * raw["num_key_value_heads"]) * raw["head_dim"]
     split_seen = False
@@ -135,7 +140,7 @@ def test_mixed_steps_at_matrix_core_sizes(tmp_path, raw, chunk, budget, sharpen)
             info = eng.step()
             # (a plan is in admission order: where an older request still runs its prompt while a
             # younger one decodes, no decode row leads and the tiled kernel takes them all)
-            if info.decode_seqs > 0 and info.prefill_tokens >= chunk - 60 and eng.runner.last_step.leading_single_runs() > 0:
+            if info.decode_seqs > 0 and info.prefill_tokens >= chunk - 60 and eng.core.plan_leading > 0:
                 mixed_big += 1
                 split_seen |= ops.skinny_splits(info.rows, qkv_width, raw["hidden_size"]) > 1
                 calls["fused_in_mixed"] += calls["fused"] > before["fused"] and calls["tiled"] > before["tiled"]
@@ -238,7 +243,7 @@ def test_graph_replays_equal_eager_steps(models, dtype):
             torch.cuda.synchronize()
         for f in eng.take_finished():
             done[f.id] = f.generated
-    assert eng.decode_graphs.graphs, "no graph was captured"
+    assert eng.decode_graphs.graph_shapes(), "no graph was captured"
     assert [done[i] for i in ids] == eager
 
 
@@ -252,7 +257,7 @@ def test_graph_replays_at_matrix_core_sizes(tmp_path):
     prompts = _prompts(H.TINY_D, [250, 20, 505, 65, 1019], seed=11)
     eng = _engine(d, dtype="bfloat16", num_blocks=200, max_seq_len=2048, max_batched_tokens=2048, use_graphs=True)
     got = eng.generate(prompts, 24)
-    assert eng.decode_graphs.graphs, "no graph was captured"
+    assert eng.decode_graphs.graph_shapes(), "no graph was captured"
     for p, g in zip(prompts, got):
         want, margins = pm.generate(p, 24)
         assert _same_up_to_near_ties(g, want, margins, 5e-2), (len(p), g, want, margins)
@@ -272,7 +277,7 @@ def test_graphs_follow_the_context_across_classes(tmp_path):
     kw = dict(dtype="bfloat16", num_blocks=300, max_seq_len=4096, max_batched_tokens=4096, beyond_max_position=True)
     eng = _engine(d, use_graphs=True, **kw)
     got = eng.generate(prompts, 40)
-    assert sorted(eng.decode_graphs.graphs) == [(2, 2048), (2, 4096)]
+    assert eng.decode_graphs.graph_shapes() == [(2, 2048), (2, 4096)]
     assert _engine(d, use_graphs=False, **kw).generate(prompts, 40) == got
     for p, g in zip(prompts, got):
         want, margins = pm.generate(p, 40)
@@ -476,38 +481,55 @@ def test_block_arrangement_alone():
     assert torch.equal(pending, torch.full((2, 4), -11.0, device="cuda:0"))
 
 
-@pytest.mark.parametrize("which", ["D", "E"])
-def test_random_workloads_over_engine_options(tmp_path, which):
+@pytest.mark.parametrize("which,dtype", [("D", "bfloat16"), ("E", "bfloat16"), ("D", "float32"), ("E", "float32")])
+def test_random_workloads_over_engine_options(tmp_path, which, dtype):
     """Requests of random lengths arriving while others run, at the matrix-core sizes, over chunked and
-    whole prompts, small and large budgets, prefix cache, graphs and a pool small enough to preempt:
-    every request ends with the number of tokens it asked for and every page comes back."""
+    whole prompts, small and large budgets, prefix cache, recorded steps (programs, graphs) and a pool
+    small enough to preempt, driven through the real scheduler with their continuations forced: the
+    logits every token would have been sampled from equal the plain implementation's, every request
+    ends with the number of tokens it asked for and every page comes back."""
     import itertools
+    from kvcm_amd.engine.replay import scheduled_replay
     raw, B = H.CONFIGS[which], H.BLOCK_SIZE[which]
     d = str(tmp_path / "m")
-    H.make_model_dir(d, raw, H.WEIGHT_SEED[which], torch.bfloat16, sharpen=H.SHARPEN[which])
-    preempted = 0
-    for combo, (chunk, budget, prefix, graphs) in enumerate(itertools.product((0, 37), (96, 512), (False, True), (True, False))):
-        rng = np.random.default_rng(combo)
-        eng = _engine(d, dtype="bfloat16", block_size=B, num_blocks=70 * 16 // B, max_seq_len=1024, max_num_seqs=8,
-                      max_batched_tokens=budget, prefill_chunk=chunk, prefix_caching=prefix, use_graphs=graphs,
-                      beyond_max_position=True)      # (configuration E states 512 positions; lengths here go to 930)
-        shared = rng.integers(0, raw["vocab_size"], size=100).tolist()
-        pending = []
-        for i in range(16):
-            toks = rng.integers(0, raw["vocab_size"], size=int(rng.choice([1, 2, 16, 17, 60, 130, 257, 400, 700]))).tolist()
-            if prefix and i % 2:
-                toks = (shared + toks)[:900]
-            pending.append((toks, int(rng.integers(1, 30)), float(rng.choice([0.0, 0.8]))))
-        want, done, steps = {}, {}, 0
-        while pending or not eng.idle():
-            if pending and steps % 3 == 0:
-                toks, gen, temp = pending.pop()
-                want[eng.add_request(toks, gen, temperature=temp, seed=7)] = gen
-            eng.step()
-            steps += 1
-            done.update({f.id: f.generated for f in eng.take_finished()})
-            assert steps < 5000
-        assert {r: len(g) for r, g in done.items()} == want, (combo, chunk, budget, prefix, graphs)
+    H.make_model_dir(d, raw, H.WEIGHT_SEED[which], torch.bfloat16 if dtype == "bfloat16" else torch.float32,
+                     sharpen=H.SHARPEN[which])
+    pm = plain.load_model_dir(d, plain.round_bf16 if dtype == "bfloat16" else None)
+    rng = np.random.default_rng(31)
+    V = raw["vocab_size"]
+    shared = rng.integers(0, V, size=100).tolist()
+    requests = []
+    for i, n in enumerate([1, 2, 16, 17, 60, 130, 257, 400, 700, 33, 64, 129, 5, 300]):
+        toks = rng.integers(0, V, size=n).tolist()
+        if i % 2:
+            toks = (shared + toks)[:900]                       # every other request begins with the same 100 tokens
+        requests.append((toks, rng.integers(0, V, size=int(rng.integers(1, 30))).tolist()))
+    ref = []
+    for prompt, cont in requests:
+        ref.append(pm.logits(prompt + cont)[len(prompt) - 1:len(prompt) + len(cont) - 1])
+    scale = max(1.0, max(float(np.abs(r).max()) for r in ref))
+    tol = (1e-2 if dtype == "bfloat16" else 1e-5) * scale
+    arrivals = [3 * i for i in range(len(requests))]
+    preempted = replayed = graphs = 0
+    combos = itertools.product((0, 37), (96, 512), (False, True), (True, False))
+    for combo, (chunk, budget, prefix, recorded) in enumerate(combos):
+        if dtype == "float32" and (combo % 3):                 # 32-bit: a third of the combinations
+            continue
+        eng = _engine(d, dtype=dtype, block_size=B, num_blocks=70 * 16 // B, max_seq_len=1024, max_num_seqs=8,
+                      max_batched_tokens=budget, prefill_chunk=chunk, prefix_caching=prefix, use_graphs=recorded,
+                      use_programs=recorded, beyond_max_position=True)      # (configuration E states 512 positions)
+        got = scheduled_replay(eng, requests, arrivals, max_steps=5000)
+        for i, (g, r) in enumerate(zip(got, ref)):
+            assert not np.isnan(g).any(), (combo, i, "a forced token has no logits")
+            err = np.abs(g - r).max(axis=1)
+            bad = np.nonzero(err > tol)[0]
+            assert len(bad) == 0, (f"options chunk={chunk} budget={budget} prefix={prefix} recorded={recorded}: request {i} "
+                                   f"(prompt {len(requests[i][0])}), generated token {bad[0]}: error {err[bad[0]]:.3g} > {tol:.3g}")
         assert eng.core.blocks_in_use() == 0
         preempted += eng.core.counters()["preemptions"]
+        if recorded:
+            st = eng.recorded.stats()
+            replayed += st["steps_replayed"]
+            graphs += st["steps_as_graph"]
     assert preempted > 0, "the pool was meant to be small enough to preempt"
+    assert replayed > 0 and graphs > 0, "no step was replayed from a recorded program or graph"

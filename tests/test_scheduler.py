@@ -267,3 +267,32 @@ def test_an_uncut_prompt_larger_than_the_budget_runs_whole_in_an_empty_step():
     m.update([42], 0)
     plan = m.schedule(1)
     assert [(p.id, p.start, p.count) for p in plan] == [(0, 300, 1), (1, 0, 40)]
+
+
+def test_batch_padded_to_a_recorded_shape_puts_padding_sequences_after_the_leading_single_rows():
+    core = HostCore(num_blocks=64, block_size=4, max_seq_len=64, max_num_seqs=16, max_batched_tokens=64)
+    core.sched_add(1, [5, 6, 7], 4)
+    core.sched_add(2, [8, 9], 4)
+    core.schedule_summary()
+    core.update_sampled([40, 41])
+    core.sched_add(3, list(range(10, 21)), 4)          # two requests decode, a prompt of 11 tokens arrives
+    n, prefill, decode, sampling, shaped = core.schedule_summary()
+    assert (n, prefill, decode, sampling, shaped) == (3, 11, 2, 3, False)
+    assert (core.plan_rows, core.plan_leading, core.plan_max_run, core.plan_max_context) == (13, 2, 11, 11)
+    out = np.full(4096, 77, dtype=np.int32)
+    L = core.build_batch_from_plan(out, pad_rows=4 + 64, pad_seqs=4 + 2, pad_logit_rows=6, table_stride=16, pad_leading=4)
+    assert (L.rows, L.seqs, L.rows_padded, L.seqs_padded, L.logit_rows, L.logit_rows_padded) == (15, 5, 68, 6, 3, 6)
+    run = out[L.run_start:L.run_start + 7].tolist()
+    assert run == [0, 1, 2, 3, 4, 15, 15]               # two real single rows, two padding ones, the prompt, a padding sequence
+    ctx = out[L.context_lens:L.context_lens + 68]
+    assert ctx[:4].tolist() == [4, 3, 0, 0] and ctx[4:15].tolist() == list(range(1, 12)) and not ctx[15:].any()
+    slots = out[L.slots[0]:L.slots[0] + 68]
+    assert (slots[[0, 1]] >= 0).all() and (slots[[2, 3]] == -1).all() and (slots[4:15] >= 0).all() and (slots[15:] == -1).all()
+    assert out[L.row_seq:L.row_seq + 15].tolist() == [0, 1, 2, 3] + [4] * 11
+    assert out[L.logit_row_index:L.logit_row_index + 6].tolist() == [0, 1, 14, 0, 0, 0]     # the prompt's last row follows the padding
+    tables = out[L.tables[0]:L.tables[0] + 6 * 16].reshape(6, 16)
+    assert not tables[2:4].any() and tables[4, :3].tolist() == core.seq_table(3)
+    assert out[L.state_slots:L.state_slots + 6].tolist()[2:4] == [-1, -1]
+    # without the option nothing changes
+    L0 = core.build_batch_from_plan(out)
+    assert (L0.rows, L0.seqs) == (13, 3) and out[L0.run_start:L0.run_start + 4].tolist() == [0, 1, 2, 13]
