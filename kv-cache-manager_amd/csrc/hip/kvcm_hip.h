@@ -64,6 +64,12 @@ int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dty
 int kvcm_gemm_f32(const float* X, const float* W, float* Y, int M, int N, int K, int ldx, int ldw, int ldy, hipStream_t s);
 int kvcm_gemm_bf16(const void* X, const void* W, void* Y, int out_dtype, int M, int N, int K, int ldx, int ldw, int ldy,
                    hipStream_t s);
+// Products of at most 8 rows with the RMS norm around them folded in (gemm_rows8.hip).
+int kvcm_gemm8_supported(int M, int N, int K);
+int kvcm_gemm8(const void* X, int ldx, const void* W, int ldw, int M, int N, int K, const float* ss_in, int tiles_in,
+               float eps, void* out, int out_dtype, int ldo, int swiglu, hipStream_t stream);
+int kvcm_gemm8_residual_norm(const void* X, int ldx, const void* W, int ldw, int M, int N, int K, float* resid,
+                             const void* g, int g_dtype, void* xg, float* ss_out, hipStream_t stream);
 // The vendor library's product (hipBLASLt), bfloat16 operands and result, 32-bit accumulation, for
 // the many-row products of prompt steps, where the reference calls cuBLAS (src/model/llama.cpp:45-52).
 // `workspace` is device memory the caller owns (at least kvcm_gemm_library_workspace_bytes()).

@@ -82,6 +82,8 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_gemm_f32),
     KVCM_ENTRY(kvcm_gemm_bf16),
     KVCM_ENTRY(kvcm_gemm_library),
+    KVCM_ENTRY(kvcm_gemm8),
+    KVCM_ENTRY(kvcm_gemm8_residual_norm),
     KVCM_ENTRY(kvcm_attention_generic),
     KVCM_ENTRY(kvcm_attention_decode),
     KVCM_ENTRY(kvcm_attention_decode_fused),

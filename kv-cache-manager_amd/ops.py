@@ -66,6 +66,9 @@ def _declare(lib):
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
     fn("kvcm_gemm_library", vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, vp)
+    fn("kvcm_gemm8_supported", i, i, i)
+    fn("kvcm_gemm8", vp, i, vp, i, i, i, i, vp, i, f, vp, i, i, i, vp)
+    fn("kvcm_gemm8_residual_norm", vp, i, vp, i, i, i, i, vp, vp, i, vp, vp, vp)
     lib.kvcm_gemm_library_workspace_bytes.restype = C.c_longlong
     lib.kvcm_gemm_library_workspace_bytes.argtypes = []
     lib.kvcm_program_new.restype = vp
@@ -246,6 +249,80 @@ class PartialSums:
         return self.out
 
 
+# Decode steps of at most this many rows fold their RMS norms into the products around them
+# (csrc/hip/gemm_rows8.hip).
+FUSED_NORM_MAX_ROWS = 8
+
+
+def gemm8_supported(M, N, K):
+    return bool(lib().kvcm_gemm8_supported(M, N, K))
+
+
+class PendingProduct:
+    """A product x @ w^T that has not run yet, handed on so that whoever adds it to the residual
+    stream can choose how it runs: with the addition and the following norm's preparation in its
+    epilogue (``gemm_residual_norm``), or the ordinary way (``run``).  ``out`` and ``scratch`` are the
+    buffers the ordinary way uses."""
+
+    def __init__(self, x, w, out, scratch=None):
+        self.x, self.w, self.out, self.scratch = x, w, out, scratch
+        self.dtype = out.dtype
+
+    def run(self, keep_partial=False):
+        return gemm(self.x, self.w, self.out, scratch=self.scratch, keep_partial=keep_partial)
+
+    def materialize(self):
+        return self.run(False)
+
+
+class NormedRows:
+    """The rows a product after an RMS norm multiplies, with the norm's scale still to be applied:
+    ``xg`` = round(g * round(x)) [rows, H] and ``ss`` [rows, H / 8] sums of x^2 per 8-column tile, left
+    by ``gemm_residual_norm``.  ``gemm`` and ``gemm_swiglu`` take it in x's place and scale their sums
+    by rsqrt(mean x^2 + eps); ``materialize`` gives the ordinary normed rows instead (the residual
+    stream x already holds the addition)."""
+
+    def __init__(self, xg, ss, eps, x, weight, out):
+        self.xg, self.ss, self.eps, self.x, self.weight, self.out = xg, ss, float(eps), x, weight, out
+        self.shape, self.dtype = xg.shape, xg.dtype
+
+    def materialize(self):
+        rmsnorm(self.x, self.weight, self.out, self.eps)
+        return self.out
+
+
+def gemm_residual_norm(product, x, weight, eps, xg, ss, out):
+    """x += round(product); returns NormedRows for the norm (weight, eps) that follows: the producer
+    half of the folded norm.  product: PendingProduct of at most 8 bfloat16 rows; x: the 32-bit residual
+    stream [rows, H]; xg [>= rows, H] bfloat16 and ss [>= rows, H / 8] float32 receive the result; out:
+    where ``materialize`` would put ordinary normed rows."""
+    a, w = product.x, product.w
+    M, K = a.shape
+    H = w.shape[0]
+    _dev(a, w, x, weight, xg, ss)
+    _rows2d(a, "x")
+    _rows2d(w, "w")
+    _need(a.dtype == w.dtype == torch.bfloat16 and w.shape[1] == K, "gemm_residual_norm needs bfloat16 operands [M, K], [H, K]")
+    _need(x.dtype == torch.float32 and x.is_contiguous() and tuple(x.shape) == (M, H), "the residual stream must be contiguous float32 [M, H]")
+    _need(weight.numel() == H and weight.is_contiguous(), "norm weight must have H entries")
+    _need(xg.dtype == torch.bfloat16 and xg.is_contiguous() and xg.shape[0] >= M and xg.shape[1] == H, "xg must be bfloat16 [>= M, H]")
+    _need(ss.dtype == torch.float32 and ss.is_contiguous() and ss.shape[0] >= M and ss.shape[1] == H // 8 and H % 8 == 0,
+          "ss must be float32 [>= M, H / 8]")
+    _call("kvcm_gemm8_residual_norm", _ptr(a), a.stride(0), _ptr(w), w.stride(0), M, H, K, _ptr(x), _ptr(weight),
+          _DT[weight.dtype], _ptr(xg), _ptr(ss), _stream())
+    return NormedRows(xg[:M], ss[:M], eps, x, weight, out)
+
+
+def _gemm8(x, w, out, N, swiglu):
+    """The product of at most 8 rows (gemm_rows8.hip); x: a tensor or NormedRows."""
+    normed = isinstance(x, NormedRows)
+    a = x.xg if normed else x
+    M, K = a.shape
+    _call("kvcm_gemm8", _ptr(a), a.stride(0), _ptr(w), w.stride(0), M, N, K, _ptr(x.ss) if normed else 0,
+          x.ss.shape[1] if normed else 0, x.eps if normed else 0.0, _ptr(out), _DT[out.dtype], out.stride(0), int(swiglu),
+          _stream())
+
+
 def rmsnorm(x, weight, out, eps, add=None, rows=None, write_back=True):
     """v = x[src] (+ add[src]); x[src] = v when write_back; out[r] = weight * round(v * rsqrt(mean v^2 + eps)).
     src = rows[r] if rows is given, else r.  ``add`` is a tensor of x's shape or PartialSums."""
@@ -369,6 +446,17 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
     ``scratch`` (float32, at least splits*M*N elements).  With ``keep_partial``
     the un-added partial sums are returned as PartialSums (for a fused consumer) instead of ``out``.
     """
+    if isinstance(x, NormedRows):
+        M, K = x.shape
+        N = w.shape[0]
+        _dev(x.xg, x.ss, w, out)
+        _rows2d(w, "w")
+        _rows2d(out, "out")
+        if (w.dtype == torch.bfloat16 and w.shape[1] == K and out.shape == (M, N) and gemm8_supported(M, N, K)
+                and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0):
+            _gemm8(x, w, out, N, False)
+            return out
+        x = x.materialize()
     _dev(x, w, out)
     for t, n in ((x, "x"), (w, "w"), (out, "out")):
         _rows2d(t, n)
@@ -408,6 +496,17 @@ def gemm_swiglu(x, w_gate_up, out):
     """out[M, I] = swiglu(x[M, K] @ w_gate_up[2 I, K]^T) in one launch, or False when this shape
     has no fused kernel (then the caller runs the product and ``swiglu`` one after the other:
     the same values up to the order of the sums)."""
+    if isinstance(x, NormedRows):
+        M, K = x.shape
+        I = out.shape[1]
+        _dev(x.xg, x.ss, w_gate_up, out)
+        _rows2d(w_gate_up, "w_gate_up")
+        _rows2d(out, "out")
+        if not (w_gate_up.dtype == out.dtype == torch.bfloat16 and tuple(w_gate_up.shape) == (2 * I, K) and out.shape[0] == M
+                and gemm8_supported(M, I, K) and w_gate_up.stride(0) % 8 == 0 and w_gate_up.data_ptr() % 16 == 0):
+            return False          # the caller materializes the rows and comes again
+        _gemm8(x, w_gate_up, out, I, True)
+        return True
     _dev(x, w_gate_up, out)
     for t, n in ((x, "x"), (w_gate_up, "w_gate_up"), (out, "out")):
         _rows2d(t, n)

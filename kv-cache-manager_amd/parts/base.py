@@ -195,12 +195,17 @@ class Part:
 
 
 class Norm(Part):
-    # True: ``add`` may be a Deferred (un-added split-K sums), which the norm adds up itself.
+    # True: ``add`` may be a Deferred (un-added split-K sums, a product that has not run yet), which
+    # the norm adds up or runs itself; False: the caller hands over a tensor (``as_tensor``).
     accepts_partial_sums = False
+    # True: ``forward`` takes ``defer=True`` and may then return, instead of ``out``, a Deferred whose
+    # scale is still to be applied by the product that consumes it (ops.NormedRows); the arrangement
+    # asks for it only when the consuming part ``accepts_normed_rows``.
+    defers = False
 
     def forward(self, x, out, add=None, rows=None):
         """out = norm(x (+ add)); when ``add`` is given and ``rows`` is not, x += add as well.
-        x is the 32-bit residual stream; rows gathers source rows."""
+        x is the 32-bit residual stream; rows gathers source rows.  Returns the normed rows (``out``)."""
         raise NotImplementedError
 
 
@@ -227,6 +232,9 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True: ``h`` may be a Deferred (ops.NormedRows) that the mixer's first product consumes as it is.
+    accepts_normed_rows = False
+
     def cache_need(self):
         """KVCacheNeed, StateNeed or None."""
         return None
@@ -242,6 +250,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_normed_rows = False      # as Mixer.accepts_normed_rows
+
     def forward(self, step, h):
         raise NotImplementedError
 

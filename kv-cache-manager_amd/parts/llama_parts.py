@@ -21,6 +21,17 @@ def _linear(ctx, step, x, w, name, keep_partial=False, dtype=None):
     return ctx.ops.gemm(x, w, out, scratch=scratch, keep_partial=keep_partial and scratch is not None)
 
 
+def _to_residual(ctx, step, x, w, name):
+    """A part's last product, whose result goes to the residual stream.  For decode steps of a few
+    rows it is handed on unrun (ops.PendingProduct): the norm that follows runs it with the addition
+    and its own preparation in the epilogue.  Otherwise it runs here, split sums left un-added."""
+    ops = ctx.ops
+    if x.dtype == torch.bfloat16 and x.shape[0] <= ops.FUSED_NORM_MAX_ROWS and ops.gemm8_supported(x.shape[0], w.shape[0], w.shape[1]):
+        out = step.ws(name, (x.shape[0], w.shape[0]))
+        return ops.PendingProduct(x, w, out, step.scratch(name, x.shape[0], w.shape[0], w.shape[1]))
+    return _linear(ctx, step, x, w, name, keep_partial=True)
+
+
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     """out = weight * round(x / sqrt(mean(x^2) + eps)); eps inside the root, no mean removed, the
@@ -28,12 +39,29 @@ class RMSNorm(Norm):
 
     capturable = True
     accepts_partial_sums = True
+    defers = True
 
     def param_specs(self):
         return [ParamSpec("weight", ((self.prefix + "weight", (self.params["size"],)),), role="vector")]
 
-    def forward(self, x, out, add=None, rows=None):
-        self.ctx.ops.rmsnorm(x, self.w["weight"], out, self.params["eps"], add=add, rows=rows)
+    def bind(self, tensors):
+        super().bind(tensors)
+        # where the folded form of this norm leaves its rows (ops.NormedRows), kept for good: recorded
+        # steps hold the addresses
+        H, ops = self.params["size"], self.ctx.ops
+        self._folded = None
+        if ops is not None and self.ctx.dtype == torch.bfloat16 and H % 8 == 0 and self.ctx.device.type == "cuda":
+            self._folded = (torch.empty(ops.FUSED_NORM_MAX_ROWS, H, dtype=torch.bfloat16, device=self.ctx.device),
+                            torch.empty(ops.FUSED_NORM_MAX_ROWS, H // 8, dtype=torch.float32, device=self.ctx.device))
+
+    def forward(self, x, out, add=None, rows=None, defer=False):
+        ops = self.ctx.ops
+        if isinstance(add, ops.PendingProduct):
+            if (defer and rows is None and self._folded is not None and add.x.shape[0] == x.shape[0] <= ops.FUSED_NORM_MAX_ROWS
+                    and add.dtype == torch.bfloat16):
+                return ops.gemm_residual_norm(add, x, self.w["weight"], self.params["eps"], *self._folded, out)
+            add = add.run(keep_partial=True)
+        ops.rmsnorm(x, self.w["weight"], out, self.params["eps"], add=add, rows=rows)
         return out
 
 
@@ -101,6 +129,7 @@ class GQAAttention(Mixer):
     params: num_heads, num_kv_heads, head_dim, scale, window (0 = all keys), position (PartSpec)."""
 
     capturable = True
+    accepts_normed_rows = True
 
     def sub_parts(self):
         return (self.position,)
@@ -141,7 +170,7 @@ class GQAAttention(Mixer):
         table = pos.rotation_table(step, self.hd) if pos.rotates else None
         if (table is not None or not pos.rotates) and paged_attention.attend_from_projection(
                 step, ops, res, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window, table, slots):
-            return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
+            return _to_residual(self.ctx, step, attn, self.w["wo"], "mixer_out")
         extra = {"source": res} if hasattr(res, "materialize") else {}
         stored = pos.apply(step, qkv, self.nh, self.nkv, self.hd,
                            cache=(kc, vc) if self.cache_owner else None, slots=slots, **extra)
@@ -149,7 +178,7 @@ class GQAAttention(Mixer):
             ops.rope_cache(qkv, self.nh, self.nkv, self.hd, slots=slots, kcache=kc, vcache=vc,
                            block_size=self.ctx.block_size, rows=step.rows)
         paged_attention.attend(step, ops, qkv, attn, kc, vc, g, self.nh, self.nkv, self.hd, self.scale, self.window)
-        return _linear(self.ctx, step, attn, self.w["wo"], "mixer_out", keep_partial=True)
+        return _to_residual(self.ctx, step, attn, self.w["wo"], "mixer_out")
 
 
 @FEED_FORWARDS.register("swiglu")
@@ -158,6 +187,7 @@ class SwiGLU(FeedForward):
     (src/model/llama.cpp:119-122, src/cuda/kernels.cu:72-82).  params: intermediate_size."""
 
     capturable = True
+    accepts_normed_rows = True
 
     def param_specs(self):
         H, I, pre = self.ctx.hidden_size, self.params["intermediate_size"], self.prefix
@@ -168,9 +198,11 @@ class SwiGLU(FeedForward):
         I = self.params["intermediate_size"]
         act = step.ws("act", (step.rows, I))
         if not self.ctx.ops.gemm_swiglu(h, self.w["w_gate_up"], act):      # few rows: one launch
-            gu = _linear(self.ctx, step, h, self.w["w_gate_up"], "gate_up")
-            self.ctx.ops.swiglu(gu, act)
-        return _linear(self.ctx, step, act, self.w["w_down"], "ffn_out", keep_partial=True)
+            h = as_tensor(h)
+            if not self.ctx.ops.gemm_swiglu(h, self.w["w_gate_up"], act):
+                gu = _linear(self.ctx, step, h, self.w["w_gate_up"], "gate_up")
+                self.ctx.ops.swiglu(gu, act)
+        return _to_residual(self.ctx, step, act, self.w["w_down"], "ffn_out")
 
 
 @EMBEDDINGS.register("token_embedding")
@@ -219,9 +251,13 @@ class PreNormResidual(Block):
     capturable = True
 
     def forward(self, step, x, pending):
-        h = step.ws("normed", (step.rows, x.shape[1]))
+        buf = step.ws("normed", (step.rows, x.shape[1]))
         n1, n2 = self.parts["norm_mixer"], self.parts["norm_ffn"]
-        n1.forward(x, h, add=pending if n1.accepts_partial_sums else as_tensor(pending))
-        a = self.parts["mixer"].forward(step, h)
-        n2.forward(x, h, add=a if n2.accepts_partial_sums else as_tensor(a))
-        return self.parts["ffn"].forward(step, h)
+        mixer, ffn = self.parts["mixer"], self.parts["ffn"]
+        # a norm may leave its scale to the product that follows (Norm.defers) where that part takes it
+        fold1 = {"defer": True} if (n1.defers and mixer.accepts_normed_rows) else {}
+        fold2 = {"defer": True} if (n2.defers and ffn.accepts_normed_rows) else {}
+        h = n1.forward(x, buf, add=pending if n1.accepts_partial_sums else as_tensor(pending), **fold1)
+        a = mixer.forward(step, buf if h is None else h)
+        h = n2.forward(x, buf, add=a if n2.accepts_partial_sums else as_tensor(a), **fold2)
+        return ffn.forward(step, buf if h is None else h)

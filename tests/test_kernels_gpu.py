@@ -1028,3 +1028,107 @@ def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops, B):
         pos = runs[0][0] + r
         ref = plain.attention(Q[r:r + 1], P["Kl"][0][:pos + 1], P["Vl"][0][:pos + 1], [pos], np.arange(pos + 1), 1.0)[0]
         np.testing.assert_allclose(got[r], ref, atol=1e-2, rtol=0, err_msg=f"row {r}")
+
+
+# ------------------------------------- products of at most 8 rows with the norm folded in
+def _folded_reference(a, wo, x, g, eps, w2):
+    """What the producer and the consumer compute, in float64 with the same rounding points:
+    x += round(a wo^T); xg = round(g round(x)); y = round((xg w2^T) rsqrt(mean x^2 + eps))."""
+    x_new = x + _bf16_grid(a @ wo.T)
+    xg = _bf16_grid(g * _bf16_grid(x_new))
+    rstd = 1.0 / np.sqrt((x_new ** 2).mean(-1, keepdims=True) + eps)
+    return x_new, xg, (xg @ w2.T) * rstd
+
+
+@pytest.mark.parametrize("M", [1, 3, 8])
+@pytest.mark.parametrize("H,K,N2", [(2048, 2048, 2560), (2048, 5632, 512), (128, 64, 40), (320, 192, 24), (2048, 2112, 4128)])
+def test_products_with_the_norm_folded_in(ops, M, H, K, N2):
+    """Producer (residual add + the norm's preparation in the epilogue) and consumer (the norm's scale on
+    the finished sums) against the same arithmetic in float64, and against the reference's own form of
+    the norm, whose two roundings fall at other places (kernels.cu:34-49): equal up to bfloat16 rounding.
+    Widths that are no power of two, K slices of unequal length, fewer rows than a tile holds."""
+    rng = np.random.default_rng(M * 13 + H + K)
+    a = _bf16_grid(rng.normal(size=(M, K)))
+    wo = _bf16_grid(rng.normal(size=(H, K)) * 0.05)
+    x = (rng.normal(size=(M, H)) * 2).astype(np.float32).astype(np.float64)
+    g = _bf16_grid(1 + 0.1 * rng.normal(size=H))
+    w2 = _bf16_grid(rng.normal(size=(N2, H)) * 0.05)
+    eps = 1e-5
+    x_new, xg_ref, y_ref = _folded_reference(a, wo, x, g, eps, w2)
+
+    at, wot, w2t = _t(a, torch.bfloat16), _t(wo, torch.bfloat16), _t(w2, torch.bfloat16)
+    xt = _t(x, torch.float32)
+    xg = torch.full((8, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ss = torch.full((8, H // 8), float("nan"), dtype=torch.float32, device=DEV)
+    normed_buf = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
+    product = ops.PendingProduct(at, wot, torch.zeros(M, H, dtype=torch.bfloat16, device=DEV))
+    assert ops.gemm8_supported(M, H, K) and ops.gemm8_supported(M, N2, H)
+    h = ops.gemm_residual_norm(product, xt, _t(g, torch.bfloat16), eps, xg, ss, normed_buf)
+    # the residual stream: a 32-bit sum of x and the rounded product (the product's last bit may fall either way)
+    np.testing.assert_allclose(_np(xt), x_new, rtol=0, atol=2 ** -7 * np.abs(a @ wo.T).max())
+    got_x = _np(xt)
+    np.testing.assert_allclose(_np(ss[:M]).sum(-1), (got_x ** 2).sum(-1), rtol=1e-5)
+    np.testing.assert_array_equal(_np(xg[:M]), _bf16_grid(g * _bf16_grid(got_x)))
+    assert torch.isnan(xg[M:].float()).all() and torch.isnan(ss[M:]).all(), "rows beyond M were written"
+
+    for dtype in (torch.bfloat16, torch.float32):
+        y = torch.full((M, N2), float("nan"), dtype=dtype, device=DEV)
+        assert ops.gemm(h, w2t, y) is y
+        scale = np.abs(y_ref).max()
+        np.testing.assert_allclose(_np(y), y_ref, rtol=0, atol=(2 ** -7 if dtype == torch.bfloat16 else 1e-3) * scale)
+    # against the reference's form: norm rows rounded as kernels.cu does, then the product
+    plain_y = plain.linear(plain.rms_norm(x_new, g, eps, plain.round_bf16), w2)
+    np.testing.assert_allclose(_np(y), plain_y, rtol=0, atol=1.5e-2 * np.abs(plain_y).max())
+    # the ordinary normed rows are still to be had
+    np.testing.assert_allclose(_np(h.materialize()), plain.rms_norm(got_x, g, eps, plain.round_bf16), rtol=2 ** -7, atol=1e-3)
+
+
+@pytest.mark.parametrize("M", [1, 5, 8])
+@pytest.mark.parametrize("H,I", [(2048, 5632), (192, 136), (64, 8)])
+def test_gate_up_product_with_the_norm_folded_in_applies_swiglu(ops, M, H, I):
+    rng = np.random.default_rng(M + H + I)
+    x = (rng.normal(size=(M, H)) * 2).astype(np.float32).astype(np.float64)
+    g = _bf16_grid(1 + 0.1 * rng.normal(size=H))
+    wgu = _bf16_grid(rng.normal(size=(2 * I, H)) * 0.05)
+    eps = 1e-6
+    # a producer with a zero product leaves x as it is and prepares the norm
+    xt = _t(x, torch.float32)
+    xg = torch.zeros(8, H, dtype=torch.bfloat16, device=DEV)
+    ss = torch.zeros(8, H // 8, dtype=torch.float32, device=DEV)
+    zero = ops.PendingProduct(torch.zeros(M, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(H, 64, dtype=torch.bfloat16, device=DEV),
+                              torch.zeros(M, H, dtype=torch.bfloat16, device=DEV))
+    h = ops.gemm_residual_norm(zero, xt, _t(g, torch.bfloat16), eps, xg, ss, torch.zeros(M, H, dtype=torch.bfloat16, device=DEV))
+    np.testing.assert_array_equal(_np(xt), x)
+    act = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert ops.gemm_swiglu(h, _t(wgu, torch.bfloat16), act)
+    xg_ref = _bf16_grid(g * _bf16_grid(x))
+    rstd = 1.0 / np.sqrt((x ** 2).mean(-1, keepdims=True) + eps)
+    gu = _bf16_grid((xg_ref @ wgu.T) * rstd)
+    want = plain.swiglu(gu, plain.round_bf16)
+    got = _np(act)
+    assert np.mean(got == want) > 0.97                       # a sum's last bit may fall the other way before rounding
+    np.testing.assert_allclose(got, want, rtol=2 ** -6, atol=2e-3)
+    # and the reference's form of norm then product then SwiGLU is the same up to rounding
+    ref = plain.swiglu(np.concatenate([plain.linear(plain.rms_norm(x, g, eps, plain.round_bf16), wgu[:I], plain.round_bf16),
+                                       plain.linear(plain.rms_norm(x, g, eps, plain.round_bf16), wgu[I:], plain.round_bf16)], -1),
+                       plain.round_bf16)
+    np.testing.assert_allclose(got, ref, rtol=0, atol=2e-2 * max(np.abs(ref).max(), 1e-3))
+
+
+@pytest.mark.parametrize("M", [1, 8])
+def test_small_product_plain_form_and_refusals(ops, M):
+    """The same kernel without a norm in front (a tensor in x's place), float32 and bfloat16 results,
+    one and two column groups per workgroup; shapes it does not take are refused by the entry."""
+    rng = np.random.default_rng(77 + M)
+    for N, K in ((4096 + 16, 128), (16400, 64), (24, 320)):
+        x = _bf16_grid(rng.normal(size=(M, K)))
+        w = _bf16_grid(rng.normal(size=(N, K)) * 0.05)
+        for dtype in (torch.bfloat16, torch.float32):
+            out = torch.full((M, N), float("nan"), dtype=dtype, device=DEV)
+            ops._gemm8(_t(x, torch.bfloat16), _t(w, torch.bfloat16), out, N, False)
+            tol = dict(rtol=2 ** -7, atol=1e-3) if dtype == torch.bfloat16 else dict(rtol=0, atol=2e-5 * math.sqrt(K))
+            np.testing.assert_allclose(_np(out), plain.linear(x, w), **tol)
+    assert not ops.gemm8_supported(9, 2048, 2048) and not ops.gemm8_supported(4, 2044, 2048) and not ops.gemm8_supported(4, 2048, 96)
+    with pytest.raises(ops.KernelError, match="unsupported shape"):
+        ops._gemm8(torch.zeros(9, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV),
+                   torch.zeros(9, 8, dtype=torch.bfloat16, device=DEV), 8, False)
