@@ -59,33 +59,24 @@ struct Trip {
   Frag x[UT][2];
 };
 
-template <int RG, int UT, bool SCALED, int EPI, class TO>
-__global__ void __launch_bounds__(256) gemm8_kernel(const Gemm8Args a) {
-  __shared__ f32x4 red[4][RG][kWave];
+template <int NW, int RG, int UT, bool SCALED, int EPI, class TO>
+__global__ void __launch_bounds__(NW * kWave) gemm8_kernel(const Gemm8Args a) {
+  static_assert(NW == 4 || NW == 8, "four or eight waves share a tile's K");
+  constexpr int kSlots = 2 * NW, kRowsPerWave = 8 / NW;
+  __shared__ f32x4 red[NW][RG][kWave];
   __shared__ float rstd_s[8];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int r = lane % 16, kq = lane / 16;
   const int half = r / 8, c = r % 8;
   const int n0 = blockIdx.x * (kCols * RG);   // kSwiglu: N is the width of the result, RG == 2 means gate and up
   const int units = a.K / kUnit;
-  // this lane's slice of K: slot = 2 * wave + half of 8
+  // this lane's slice of K: slot = 2 * wave + half of 2 * NW
   const int slot = 2 * wave + half;
-  const int u_lo = units * slot / 8, u_hi = units * (slot + 1) / 8;
+  const int u_lo = units * slot / kSlots, u_hi = units * (slot + 1) / kSlots;
   const int cnt = u_hi - u_lo;
-  const int other = units * (slot ^ 1) / 8;
-  const int cnt_other = units * ((slot ^ 1) + 1) / 8 - other;
+  const int other = units * (slot ^ 1) / kSlots;
+  const int cnt_other = units * ((slot ^ 1) + 1) / kSlots - other;
   const int n_main = cnt < cnt_other ? cnt : cnt_other, n_max = cnt > cnt_other ? cnt : cnt_other;
-
-  // rstd of up to two rows per wave: the tiles' sums are asked for now and added up after the loop
-  float ss_acc[2] = {0.f, 0.f};
-  if constexpr (SCALED) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int m = wave + 4 * i;
-      const float* p = a.ss_in + size_t(m < a.M ? m : 0) * a.tiles_in;
-      for (int t = lane; t < a.tiles_in; t += kWave) ss_acc[i] += p[t];
-    }
-  }
 
   const uint16_t* wrow[RG];
 #pragma unroll
@@ -132,38 +123,79 @@ __global__ void __launch_bounds__(256) gemm8_kernel(const Gemm8Args a) {
       }
     }
   };
+  // What the epilogue needs from memory is asked for ahead of the weights and used behind their
+  // requests, so that it is worked on while the weights are on their way: the tiles' sums of squares
+  // of up to two rows per wave (SCALED; added up in a fixed order), and this thread's element of the
+  // residual stream and of the norm's weight (kResidualNorm; threads of the first wave).
+  constexpr int kSsRegs = 4;   // tiles per lane kept in registers: widths up to 8 * 64 * 4 = 2048; wider rows add the rest directly
+  float ssv[kRowsPerWave][kSsRegs];
+  float ss_more[kRowsPerWave] = {};
+  const int em = threadIdx.x / 8, en = threadIdx.x % 8;   // the epilogue's (row, column) of the first 64 threads
+  float resid_in = 0.f, g_in = 0.f;
+  auto ask_epilogue = [&]() {
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int i = 0; i < kRowsPerWave; ++i) {
+        const int m = wave + NW * i;
+        const float* p = a.ss_in + size_t(m < a.M ? m : 0) * a.tiles_in;
+#pragma unroll
+        for (int q = 0; q < kSsRegs; ++q) {
+          const int t = lane + q * kWave;
+          ssv[i][q] = p[t < a.tiles_in ? t : 0];
+        }
+        for (int t = lane + kSsRegs * kWave; t < a.tiles_in; t += kWave) ss_more[i] += p[t];
+      }
+    }
+    if constexpr (EPI == kResidualNorm) {
+      if (threadIdx.x < kWave) {
+        const int col = n0 + en;
+        resid_in = a.resid[size_t(em < a.M ? em : 0) * a.N + col];
+        g_in = a.g_f32 ? static_cast<const float*>(a.g)[col] : load_f(static_cast<const bf16_t*>(a.g) + col);
+      }
+    }
+  };
+  auto rstd_to_lds = [&]() {
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int i = 0; i < kRowsPerWave; ++i) {
+        float part = ss_more[i];
+#pragma unroll
+        for (int q = 0; q < kSsRegs; ++q) part += (lane + q * kWave < a.tiles_in) ? ssv[i][q] : 0.f;
+        const float s = wave_sum(part);
+        if (lane == 0) rstd_s[wave + NW * i] = rsqrtf(s * a.inv_width + a.eps);
+      }
+    }
+  };
+  ask_epilogue();
   if (n_max > 0) {
     Trip<RG, UT> ta, tb;
     fetch(0, ta);
+    if (UT < n_max) fetch(UT, tb);
+    rstd_to_lds();
     for (int j0 = 0; j0 < n_max; j0 += 2 * UT) {
-      if (j0 + UT < n_max) fetch(j0 + UT, tb);
       multiply(j0, ta);
       if (j0 + UT >= n_max) break;
       if (j0 + 2 * UT < n_max) fetch(j0 + 2 * UT, ta);
       multiply(j0 + UT, tb);
+      if (j0 + 3 * UT < n_max) fetch(j0 + 3 * UT, tb);
     }
+  } else {
+    rstd_to_lds();
   }
 
 #pragma unroll
   for (int g = 0; g < RG; ++g) red[wave][g][lane] = acc[g];
-  if constexpr (SCALED) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const float s = wave_sum(ss_acc[i]);
-      if (lane == 0) rstd_s[wave + 4 * i] = rsqrtf(s * a.inv_width + a.eps);
-    }
-  }
   __syncthreads();
   if (threadIdx.x >= kWave) return;
 
   // thread -> (row m, column n of a group): the two diagonal blocks of every wave's result
-  const int m = threadIdx.x / 8, n = threadIdx.x % 8;
+  const int m = em, n = en;
   float v[RG];
 #pragma unroll
   for (int g = 0; g < RG; ++g) {
     float s = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       s += red[w][g][(m / 4) * 16 + n][m % 4];
       s += red[w][g][(2 + m / 4) * 16 + n + 8][m % 4];
     }
@@ -187,11 +219,9 @@ __global__ void __launch_bounds__(256) gemm8_kernel(const Gemm8Args a) {
     const int col = n0 + n;
     float xn = 0.f;
     if (live) {
-      float* px = a.resid + size_t(m) * a.N + col;
-      xn = *px + round_to<bf16_t>(v[0]);
-      *px = xn;
-      const float gv = a.g_f32 ? static_cast<const float*>(a.g)[col] : load_f(static_cast<const bf16_t*>(a.g) + col);
-      a.xg[size_t(m) * a.N + col] = float_to_bf16_bits(gv * round_to<bf16_t>(xn));
+      xn = resid_in + round_to<bf16_t>(v[0]);
+      a.resid[size_t(m) * a.N + col] = xn;
+      a.xg[size_t(m) * a.N + col] = float_to_bf16_bits(g_in * round_to<bf16_t>(xn));
     }
     float sq = xn * xn;
     sq += __shfl_xor(sq, 1, kWave);
@@ -231,7 +261,12 @@ int kvcm_gemm8(const void* X, int ldx, const void* W, int ldw, int M, int N, int
   a.inv_width = tiles_in > 0 ? 1.0f / float(tiles_in * kCols) : 0.f; a.eps = eps; a.out = out; a.ldo = ldo;
   KVCM_REQUIRE(operands_ok(a), "gemm8: operands must be 16-byte aligned with leading dimensions that are multiples of 8 and at least K");
   const bool scaled = ss_in != nullptr;
-#define KVCM_G8(RG, UT, SC, EP, TO) gemm8_kernel<RG, UT, SC, EP, TO><<<grid, 256, 0, st>>>(a)
+  // longer trips where two trips of UT units per half would not have a tile's whole K on its way at once
+#define KVCM_G8(RG, UT, SC, EP, TO)                                                         \
+  do {                                                                                      \
+    if (K / kUnit > 8 * 2 * UT) gemm8_kernel<4, RG, UT + UT / 2, SC, EP, TO><<<grid, 256, 0, st>>>(a); \
+    else gemm8_kernel<4, RG, UT, SC, EP, TO><<<grid, 256, 0, st>>>(a);                      \
+  } while (0)
   if (swiglu) {
     const dim3 grid(N / kCols);
     if (out_dtype == kBF16) { if (scaled) KVCM_G8(2, 2, true, kSwiglu, bf16_t); else KVCM_G8(2, 2, false, kSwiglu, bf16_t); }
@@ -264,7 +299,8 @@ int kvcm_gemm8_residual_norm(const void* X, int ldx, const void* W, int ldw, int
   a.ss_out = ss_out;
   KVCM_REQUIRE(operands_ok(a), "gemm8_residual_norm: operands must be 16-byte aligned with leading dimensions that are multiples of 8 and at least K");
   const dim3 grid(N / kCols);
-  gemm8_kernel<1, 4, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);
+  if (K / kUnit > 8 * 2 * 4) gemm8_kernel<4, 1, 6, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);
+  else gemm8_kernel<4, 1, 4, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);
   return launch_status("gemm8_residual_norm");
 }
 
