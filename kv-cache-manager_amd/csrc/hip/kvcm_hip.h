@@ -100,6 +100,12 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
 int kvcm_sample(const float* logits, int ld, const float* temperature, const uint64_t* seeds, const long long* request_ids,
                 const int* token_index, int* out, int R, int V, hipStream_t s);
 
+// ---- random weights (fill_normal.hip) ------------------------------------------------------------
+// out[i] = mean + std * n(key, i), n standard normal by a counter-based rule that the host evaluates
+// the same way; integer tables: a counter-based value mod `modulus`.
+int kvcm_fill_normal(void* out, int dtype, long long n, uint64_t key, float mean, float std, hipStream_t s);
+int kvcm_fill_index(int* out, long long n, uint64_t key, int modulus, hipStream_t s);
+
 // ---- recorded steps ---------------------------------------------------------------------------
 // A step program is the list of launches of one step, recorded once for a step shape and replayed
 // with nothing but the step's metadata changed (the kernels read that from device memory).  The

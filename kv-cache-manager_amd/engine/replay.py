@@ -24,14 +24,17 @@ class ReplayError(RuntimeError):
 
 class TraceReplayer:
     def __init__(self, model_dir, dtype="bfloat16", max_tokens=4096, block_size=16, device="cuda:0",
-                 max_live=8, attn="auto"):
+                 max_live=8, attn="auto", architecture=None, model_config=None, tensors=None):
+        """``model_dir``: a model folder; or None with architecture + model_config + tensors (checkpoint
+        names -> tensors in memory), as build_runner takes them."""
         pages = (max_tokens + block_size - 1) // block_size
         span = max(pages * block_size, block_size)
         ec = EngineConfig(policy="paged", block_size=block_size, max_seq_len=span, num_blocks=max(pages, 1),
                           watermark_blocks=0, max_num_seqs=max_live, max_batched_tokens=span,
                           max_logit_rows=min(span, 1024), dtype=dtype, attn=attn, use_graphs=False,
                           beyond_max_position=True)     # a trace's lengths are given, not generated
-        self.runner, self.core, self.model, self.model_config = build_runner(model_dir, ec, device=device)
+        self.runner, self.core, self.model, self.model_config = build_runner(
+            model_dir, ec, device=device, architecture=architecture, model_config=model_config, tensors=tensors)
         self.vocab_size = self.model.spec.vocab_size
         self._ids = {}          # external id -> integer id
         self._next = 0

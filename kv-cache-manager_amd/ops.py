@@ -66,6 +66,8 @@ def _declare(lib):
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
     fn("kvcm_gemm_library", vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, vp)
+    fn("kvcm_fill_normal", vp, i, C.c_longlong, C.c_uint64, f, f, vp)
+    fn("kvcm_fill_index", vp, C.c_longlong, C.c_uint64, i, vp)
     fn("kvcm_gemm8_supported", i, i, i)
     fn("kvcm_gemm8", vp, i, vp, i, i, i, i, vp, i, f, vp, i, i, i, vp)
     fn("kvcm_gemm8_residual_norm", vp, i, vp, i, i, i, i, vp, vp, i, vp, vp, vp)
@@ -698,6 +700,22 @@ def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, s
                                         _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), num_seqs, max_run,
                                         T, int(max_context), nh, nkv, hd, kcache.shape[2], float(scale), _ptr(scratch),
                                         scratch.numel() if scratch is not None else 0, _stream())
+
+
+def fill_normal(out, key, mean=0.0, std=1.0):
+    """out[i] = mean + std * n(key, i) over the flattened tensor: the counter-based normal values of
+    weights/random_init.py, made on the device (float32 or bfloat16)."""
+    _dev(out)
+    _need(out.is_contiguous() and out.dtype in _DT, "fill_normal needs a contiguous float32 or bfloat16 tensor")
+    _check(lib().kvcm_fill_normal(_ptr(out), _DT[out.dtype], out.numel(), int(key) & _MASK64, float(mean), float(std), _stream()))
+    return out
+
+
+def fill_index(out, key, modulus):
+    _dev(out)
+    _need(out.is_contiguous() and out.dtype == torch.int32 and modulus > 0, "fill_index needs a contiguous int32 tensor")
+    _check(lib().kvcm_fill_index(_ptr(out), out.numel(), int(key) & _MASK64, int(modulus), _stream()))
+    return out
 
 
 def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_index=None):

@@ -160,6 +160,45 @@ def sample_row(logits, temperature, seed, request_id, token_index):
     return int(order[0]), float(score[order[0]] - score[order[1]])
 
 
+# ----------------------------------------------------------------- seeded random weights
+def counter_normal(seed, name, count):
+    """Standard normal values of the random-weights rule for one tensor, as float32: a counter-based
+    generator keyed by (seed, tensor name, element index), written here from the rule's description
+    (SplitMix64 mixing, FNV-1a of the name, Box-Muller in double precision) and sharing no code with
+    the engine's.  The reference has no random weights (src/main_bench.cpp:6-7)."""
+    mask = (1 << 64) - 1
+
+    def mix_int(z):
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+        return z ^ (z >> 31)
+
+    def mix(z):
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+    h = 0xCBF29CE484222325
+    for byte in name.encode():
+        h = ((h ^ byte) * 0x100000001B3) & mask
+    key = mix_int(mix_int(seed & mask) ^ h)
+    with np.errstate(over="ignore"):
+        z1 = mix(np.uint64(key) + np.arange(1, count + 1, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15))
+        z2 = mix(z1)
+    u1 = ((z1 >> np.uint64(12)).astype(np.float64) + 0.5) / 2.0 ** 52
+    u2 = (z2 >> np.uint64(12)).astype(np.float64) / 2.0 ** 52
+    return (np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)).astype(np.float32)
+
+
+def counter_weight(seed, name, shape, std=0.02, vector=False, norm_jitter=0.0):
+    """A tensor of the rule: float32(std * n) for matrices and tables, float32(1 + norm_jitter * n) for
+    norm weights, in float32 arithmetic."""
+    n = counter_normal(seed, name, int(np.prod(shape)))
+    if vector:
+        return (np.float32(1.0) + np.float32(norm_jitter) * n).reshape(shape) if norm_jitter else np.ones(shape, np.float32)
+    return (np.float32(std) * n).reshape(shape)
+
+
 # ----------------------------------------------------------------------------- the model
 class PlainLlama:
     """Holds float64 copies of a checkpoint's tensors under their checkpoint names."""

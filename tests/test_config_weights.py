@@ -25,6 +25,35 @@ def _model(raw, dtype=torch.float32):
     return cfg, Model(spec, BuildContext(dtype, torch.device("cpu"), spec.hidden_size, 16, None))
 
 
+# ---------------------------------------------------------------------- seeded random weights
+def test_random_weights_follow_the_counter_rule_of_the_plain_implementation():
+    """The engine's host generator and the plain implementation's, written apart from each other from
+    the same rule, give the same bits; the values are normal; a tensor depends on (seed, name) alone."""
+    from kvcm_amd.weights.random_init import normal_values, random_tensor, tensor_key
+    for seed, name, count in ((0, "model.embed_tokens.weight", 100003), (7, "model.layers.3.mlp.up_proj.weight", 4097),
+                              ((1 << 63) + 5, "x", 1)):
+        got = normal_values(tensor_key(seed, name), count)
+        want = plain.counter_normal(seed, name, count)
+        assert got.dtype == np.float32 and np.array_equal(got, want)
+    big = normal_values(tensor_key(0, "model.embed_tokens.weight"), 400000, chunk=65536)       # chunking changes nothing
+    np.testing.assert_array_equal(big[:100003], plain.counter_normal(0, "model.embed_tokens.weight", 100003))
+    assert abs(big.mean()) < 0.01 and abs(big.std() - 1) < 0.01 and abs((big ** 3).mean()) < 0.03
+    assert abs((big ** 4).mean() - 3) < 0.1 and 4 < np.abs(big).max() < 7
+    # the same tensor whatever else was made before it, another one for another name or seed
+    a = random_tensor(3, "w.weight", (50, 20), "matrix", torch.float32)
+    np.testing.assert_array_equal(a.numpy(), plain.counter_weight(3, "w.weight", (50, 20)))
+    assert not np.array_equal(a.numpy(), plain.counter_weight(3, "v.weight", (50, 20)))
+    assert not np.array_equal(a.numpy(), plain.counter_weight(4, "w.weight", (50, 20)))
+    g = random_tensor(3, "n.weight", (64,), "vector", torch.float32, norm_jitter=0.1)
+    np.testing.assert_array_equal(g.numpy(), plain.counter_weight(3, "n.weight", (64,), vector=True, norm_jitter=0.1))
+    assert torch.equal(random_tensor(3, "n.weight", (64,), "vector", torch.float32), torch.ones(64))
+    idx = random_tensor(3, "table", (1000,), "index")
+    assert idx.dtype == torch.int32 and 0 <= int(idx.min()) and int(idx.max()) < 1024 and len(set(idx.tolist())) > 500
+    # bfloat16 storage is the float32 value rounded
+    b = random_tensor(3, "w.weight", (50, 20), "matrix", torch.bfloat16)
+    np.testing.assert_array_equal(b.float().numpy(), plain.round_bf16(a.numpy()).astype(np.float32))
+
+
 # ------------------------------------------------------------------------------------ config
 def test_config_reads_its_keys_and_defaults():
     c = LlamaConfig.from_dict(H.TINY_A)

@@ -1,0 +1,110 @@
+"""At the layer sizes of a served model (hidden 2048, 32 query and 4 KV heads of 64, SwiGLU 5632,
+vocabulary 32000; two layers): the kernels and kernel choices that only real widths select (split
+counts, long trips, the library's products, 64-row prefill tiles, the products that fold the norms
+in) against the plain implementation, for whole requests, the last 32 tokens one by one, and mixed
+batches with pages used again.  The weights are made on the GPU by the counter-based rule; the plain
+implementation reads those very values, and the rule itself is checked against the host's and the
+plain implementation's own generator on smaller tensors."""
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_llama as plain
+
+pytestmark = pytest.mark.gpu
+
+REAL = dict(architectures=["LlamaForCausalLM"], vocab_size=32000, hidden_size=2048, intermediate_size=5632,
+            num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=4, head_dim=64,
+            max_position_embeddings=2048, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+
+
+def test_device_and_host_make_the_same_random_weights():
+    from kvcm_amd.weights.random_init import random_tensor
+    for name, shape, role, kw in (("model.layers.0.mlp.gate_proj.weight", (1031, 517), "matrix", {}),
+                                  ("model.norm.weight", (4099,), "vector", dict(norm_jitter=0.1)),
+                                  ("model.embed_tokens.weight", (3, 5), "matrix", dict(std=1.0))):
+        for dtype in (torch.float32, torch.bfloat16):
+            host = random_tensor(11, name, shape, role, dtype, device="cpu", **kw)
+            dev = random_tensor(11, name, shape, role, dtype, device="cuda:0", **kw).cpu()
+            same = (host == dev).float().mean().item()
+            # (the two math libraries may round a logarithm or cosine differently: one 32-bit ulp, rarely)
+            assert same > 1 - 1e-5, (name, dtype, same)
+            np.testing.assert_allclose(dev.float().numpy(), host.float().numpy(), rtol=2e-7 if dtype == torch.float32 else 2 ** -7, atol=1e-9)
+    want = plain.counter_weight(11, "model.layers.0.mlp.gate_proj.weight", (1031, 517))
+    got = random_tensor(11, "model.layers.0.mlp.gate_proj.weight", (1031, 517), "matrix", torch.float32, device="cuda:0").cpu().numpy()
+    assert (got == want).mean() > 1 - 1e-5
+    idx_h = random_tensor(11, "t", (777,), "index", device="cpu")
+    idx_d = random_tensor(11, "t", (777,), "index", device="cuda:0").cpu()
+    assert torch.equal(idx_h, idx_d)
+
+
+@pytest.fixture(scope="module")
+def real_width_setup():
+    from kvcm_amd.config.model_config import LlamaConfig
+    from kvcm_amd.weights.random_init import random_tensors
+    cfg = LlamaConfig.from_dict(REAL)
+    # 32-bit values made on the device; q and k projections sharpened and the embedding scaled up as in
+    # the tiny configurations, so that a wrong position or a missing key changes the logits visibly (the
+    # factor is chosen for this width as there: scores spread over a few units, not over tens, where the
+    # rounding of q and k themselves, amplified by exp, would be the largest error in the test)
+    tensors = random_tensors("LlamaForCausalLM", cfg, seed=17, dtype=torch.float32, std=0.02, norm_jitter=0.1, device="cuda:0")
+    for name in tensors:
+        if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
+            tensors[name] *= 1.5
+        if "embed_tokens" in name:
+            tensors[name] *= 20.0
+    reqs = H.requests_for(REAL, [300, 20, 700, 65, 129], seed=5)
+    out = {}
+    for dtype in ("float32", "bfloat16"):
+        tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+        stored = {k: v.to(tdt) for k, v in tensors.items()}
+        host = {k: v.float().cpu().numpy() for k, v in stored.items()}
+        pm = plain.PlainLlama(REAL, host, plain.round_bf16 if dtype == "bfloat16" else None)
+        ref = {rid: pm.logits(t) for rid, t in reqs.items()}
+        out[dtype] = (cfg, stored, reqs, ref)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_real_widths_whole_tail_singly_and_mixed(real_width_setup, dtype):
+    from kvcm_amd.engine.replay import TraceReplayer
+    cfg, tensors, reqs, ref = real_width_setup[dtype]
+    rp = TraceReplayer(None, dtype, max_tokens=H.tokens_needed(reqs), block_size=16, architecture="LlamaForCausalLM",
+                       model_config=cfg, tensors=tensors)
+    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    tol = (1e-4 if dtype == "float32" else 1e-2) * scale
+    for what, steps in (("whole", H.schedule_whole(reqs)), ("tail singly", H.schedule_tail_singly(reqs, 32)),
+                        ("mixed", H.schedule_mixed(reqs, seed=2))):
+        got = H.replay(rp, steps, reqs)
+        assert all(not np.isnan(g).any() for g in got.values()), what
+        worst = max(float(np.abs(got[rid] - ref[rid]).max()) for rid in ref)
+        print(f"{dtype} {what}: largest error {worst:.3g} of tolerance {tol:.3g}")
+        bad = H.first_difference(got, ref, tol)
+        assert bad is None, f"{what}: first wrong logits at request {bad[0]} position {bad[1]}: error {bad[2]:.3g} > {tol:.3g}"
+        assert rp.core.blocks_in_use() == 0
+
+
+def test_real_widths_decode_through_the_engine_with_forced_tokens(real_width_setup):
+    """The scheduler's own decode steps at batch 3 and 8 (graphs, the products that fold the norms in)
+    and its prompt steps (the library's products), teacher-forced: logits against the plain implementation."""
+    from kvcm_amd import Engine, EngineConfig
+    from kvcm_amd.engine.replay import scheduled_replay
+    cfg, tensors, reqs, ref = real_width_setup["bfloat16"]
+    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    for live in (3, 8):
+        eng = Engine(config=EngineConfig(block_size=16, num_blocks=256, max_seq_len=1024, max_num_seqs=live, max_batched_tokens=1024),
+                     architecture="LlamaForCausalLM", model_config=cfg, tensors=tensors)
+        requests = []
+        for rid, toks in reqs.items():
+            n = len(toks)
+            for cut in ((n - 12, n - 5) if live == 8 else (n - 12,)):
+                if cut > 0:
+                    requests.append((rid, cut, toks[:cut], toks[cut:]))
+        got = scheduled_replay(eng, [(p, c) for _, _, p, c in requests])
+        for (rid, cut, p, c), g in zip(requests, got):
+            want = ref[rid][cut - 1:len(p) + len(c) - 1]
+            err = np.abs(g - want).max()
+            assert err <= 1e-2 * scale, (live, rid, cut, err)
+        st = eng.recorded.stats()
+        assert st["steps_as_graph"] > 0 and eng.core.blocks_in_use() == 0
