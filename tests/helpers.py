@@ -172,3 +172,44 @@ def first_difference(got, ref, tol):
         if len(bad):
             return rid, int(bad[0]), float(err[bad[0]])
     return None
+
+
+# ------------------------------------------------------------- inputs where the order of rounding shows
+def norm_rounding_cases(rows=4, width=256, seed=3):
+    """(x float32 rows, w on the bfloat16 grid) for an RMS norm: plenty of elements for which
+    round(w * round(x * inv)) differs from a single rounding after the multiply, and none where x * inv
+    lies so close to a rounding boundary of bfloat16 that 32-bit arithmetic could decide it the other
+    way than exact arithmetic (those elements are nudged away)."""
+    rng = np.random.default_rng(seed)
+    x = rng.normal(size=(rows, width)).astype(np.float32).astype(np.float64)
+    w = plain.round_bf16(1.0 + 0.3 * rng.normal(size=width))
+    for _ in range(4):
+        inv = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + 1e-6)
+        y = x * inv
+        lo = plain.round_bf16(y)
+        ulp = np.abs(lo) * 2.0 ** -8 + 1e-30
+        frac = np.abs(y - lo) / ulp                              # 0 .. 0.5 of a step away from the rounded value
+        near = frac > 0.49                                       # too close to the midpoint between two grid values
+        x = np.where(near, x * (1.0 + 2.0 ** -9), x).astype(np.float32).astype(np.float64)
+        p = w * lo
+        pl = plain.round_bf16(p)
+        near2 = np.abs(p - pl) / (np.abs(pl) * 2.0 ** -8 + 1e-30) > 0.49
+        x = np.where(near2, x * (1.0 - 2.0 ** -9), x).astype(np.float32).astype(np.float64)
+    return x, w
+
+
+def swiglu_rounding_cases(rows=3, width=200, seed=4):
+    """(gate, up) on the bfloat16 grid with silu(gate) safely away from rounding boundaries."""
+    rng = np.random.default_rng(seed)
+    g = plain.round_bf16(rng.normal(size=(rows, width)) * 2.0)
+    u = plain.round_bf16(rng.normal(size=(rows, width)) * 2.0)
+    for _ in range(4):
+        s = g / (1.0 + np.exp(-g))
+        sl = plain.round_bf16(s)
+        near = np.abs(s - sl) / (np.abs(sl) * 2.0 ** -8 + 1e-30) > 0.47
+        g = np.where(near, plain.round_bf16(g * (1.0 + 2.0 ** -6)), g)
+        p = sl * u
+        pl = plain.round_bf16(p)
+        near2 = np.abs(p - pl) / (np.abs(pl) * 2.0 ** -8 + 1e-30) > 0.49
+        u = np.where(near2, plain.round_bf16(u * (1.0 + 2.0 ** -6)), u)
+    return g, u

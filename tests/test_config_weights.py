@@ -312,6 +312,106 @@ def test_plain_swiglu_and_sampling_pins():
                                   [1.0, 1.0, 1.015625, 3.140625])                # ties to even
 
 
+def _tiny_plain(seed=0, **zeroed):
+    raw = H.TINY_A
+    t = {k: v.numpy().astype(np.float64) for k, v in
+         random_tensors("LlamaForCausalLM", LlamaConfig.from_dict(raw), seed=seed, dtype=torch.float32, std=0.2, norm_jitter=0.2).items()}
+    for name in t:
+        if any(name.endswith(z) for z in zeroed.get("zero", ())):
+            t[name] = np.zeros_like(t[name])
+    return raw, t, plain.PlainLlama(raw, t)
+
+
+def test_plain_model_residual_placement_and_layer_order():
+    """What the layers add to the residual stream, where the norms sit and in which order the two
+    halves of a layer run, pinned by cases that reduce to something smaller (src/model/llama.cpp:104-128)."""
+    toks = list(np.random.default_rng(4).integers(0, 256, size=9))
+    pos = np.arange(9)
+    # nothing but the residual path: both output projections zero -> head(final_norm(embedding))
+    raw, t, pm = _tiny_plain(zero=("o_proj.weight", "down_proj.weight"))
+    emb = plain.embedding(t["model.embed_tokens.weight"], toks)
+    bare = plain.rms_norm(emb, t["model.norm.weight"], raw["rms_norm_eps"]) @ t["lm_head.weight"].T
+    np.testing.assert_allclose(pm.logits(toks), bare, atol=1e-12)
+    # ... and the final norm is applied to the stream itself: a larger embedding changes nothing
+    t10 = dict(t)
+    t10["model.embed_tokens.weight"] = t["model.embed_tokens.weight"] * 1000.0
+    np.testing.assert_allclose(plain.PlainLlama(raw, t10).logits(toks), bare, rtol=1e-3, atol=1e-6)   # (eps is what is left)
+
+    # attention alone: down_proj zero -> x += o(attn(rot(q), rot(k), v)) of norm1(x), layer after layer
+    raw, t, pm = _tiny_plain(zero=("down_proj.weight",))
+    x = plain.embedding(t["model.embed_tokens.weight"], toks)
+    for l in range(raw["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        h = plain.rms_norm(x, t[p + "input_layernorm.weight"], raw["rms_norm_eps"])
+        q = plain.rotary(plain.linear(h, t[p + "self_attn.q_proj.weight"]).reshape(9, 4, 16), pos, raw["rope_theta"])
+        k = plain.rotary(plain.linear(h, t[p + "self_attn.k_proj.weight"]).reshape(9, 2, 16), pos, raw["rope_theta"])
+        v = plain.linear(h, t[p + "self_attn.v_proj.weight"]).reshape(9, 2, 16)
+        x = x + plain.linear(plain.attention(q, k, v, pos, pos, 0.25).reshape(9, 64), t[p + "self_attn.o_proj.weight"])
+    want = plain.rms_norm(x, t["model.norm.weight"], raw["rms_norm_eps"]) @ t["lm_head.weight"].T
+    np.testing.assert_allclose(pm.logits(toks), want, atol=1e-10)
+    # a post-norm arrangement (norm after the addition) or an un-normed input to q/k/v would differ
+    post = plain.embedding(t["model.embed_tokens.weight"], toks)
+    for l in range(raw["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        q = plain.rotary(plain.linear(post, t[p + "self_attn.q_proj.weight"]).reshape(9, 4, 16), pos, raw["rope_theta"])
+        k = plain.rotary(plain.linear(post, t[p + "self_attn.k_proj.weight"]).reshape(9, 2, 16), pos, raw["rope_theta"])
+        v = plain.linear(post, t[p + "self_attn.v_proj.weight"]).reshape(9, 2, 16)
+        a = plain.linear(plain.attention(q, k, v, pos, pos, 0.25).reshape(9, 64), t[p + "self_attn.o_proj.weight"])
+        post = plain.rms_norm(post + a, t[p + "input_layernorm.weight"], raw["rms_norm_eps"])
+    assert np.abs(post - x).max() > 1e-2
+
+    # the feed-forward alone: o_proj zero -> rows do not see each other at all, and every layer adds
+    # down(swiglu(gate(h), up(h))) of norm2(x); a position's logits depend on its own token only
+    raw, t, pm = _tiny_plain(zero=("o_proj.weight",))
+    x = plain.embedding(t["model.embed_tokens.weight"], toks)
+    for l in range(raw["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        h = plain.rms_norm(x, t[p + "post_attention_layernorm.weight"], raw["rms_norm_eps"])
+        gu = np.concatenate([plain.linear(h, t[p + "mlp.gate_proj.weight"]), plain.linear(h, t[p + "mlp.up_proj.weight"])], -1)
+        x = x + plain.linear(plain.swiglu(gu), t[p + "mlp.down_proj.weight"])
+    want = plain.rms_norm(x, t["model.norm.weight"], raw["rms_norm_eps"]) @ t["lm_head.weight"].T
+    np.testing.assert_allclose(pm.logits(toks), want, atol=1e-10)
+    np.testing.assert_allclose(pm.logits(toks[3:4])[0], pm.logits(toks)[3], atol=1e-10)
+
+    # order inside a layer: the feed-forward reads the stream after the attention's addition.  With the
+    # first layer's attention swapped for another one the feed-forward's input changes, so its own
+    # contribution (its output for the same tokens) changes too; side by side on one input it would not.
+    raw, t, pm = _tiny_plain()
+    full = pm.logits(toks)
+    t2 = dict(t)
+    t2["model.layers.0.self_attn.o_proj.weight"] = -t["model.layers.0.self_attn.o_proj.weight"]
+    x_a = plain.PlainLlama(raw, t).layer(0, plain.embedding(t["model.embed_tokens.weight"], toks), pos)
+    x_b = plain.PlainLlama(raw, t2).layer(0, plain.embedding(t["model.embed_tokens.weight"], toks), pos)
+    emb = plain.embedding(t["model.embed_tokens.weight"], toks)
+    h = plain.rms_norm(emb, t["model.layers.0.input_layernorm.weight"], raw["rms_norm_eps"])
+    q = plain.rotary(plain.linear(h, t["model.layers.0.self_attn.q_proj.weight"]).reshape(9, 4, 16), pos, raw["rope_theta"])
+    k = plain.rotary(plain.linear(h, t["model.layers.0.self_attn.k_proj.weight"]).reshape(9, 2, 16), pos, raw["rope_theta"])
+    v = plain.linear(h, t["model.layers.0.self_attn.v_proj.weight"]).reshape(9, 2, 16)
+    a = plain.linear(plain.attention(q, k, v, pos, pos, 0.25).reshape(9, 64), t["model.layers.0.self_attn.o_proj.weight"])
+    ffn_a, ffn_b = x_a - (emb + a), x_b - (emb - a)          # what the feed-forward added in each case
+    assert np.abs(ffn_a - ffn_b).max() > 1e-3                # it saw the attention's output
+    assert full.shape == (9, 256)
+
+
+def test_plain_rounding_positions_on_the_16_bit_grid():
+    """The two places where the order of rounding and multiplying matters (src/cuda/kernels.cu:34-49:
+    the normed value is cast to 16 bits, then multiplied by the weight in 16 bits; kernels.cu:72-82:
+    silu is cast to 16 bits, then multiplied by up), with inputs on which another order gives other bits."""
+    r = plain.round_bf16
+    x, w = H.norm_rounding_cases()
+    inv = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + 1e-6)
+    ours = plain.rms_norm(x, w, 1e-6, r)
+    np.testing.assert_array_equal(ours, r(w * r(x * inv)))
+    assert (ours != r(w * x * inv)).mean() > 0.05            # rounding once, after the multiply
+    assert (ours != r(r(w * x) * inv)).mean() > 0.05         # weight first
+    g, u = H.swiglu_rounding_cases()
+    act = plain.swiglu(np.concatenate([g, u], -1), r)
+    silu = g / (1.0 + np.exp(-g))
+    np.testing.assert_array_equal(act, r(r(silu) * u))
+    assert (act != r(silu * u)).mean() > 0.05                # rounding once, after the multiply
+    assert (act != r(g * r(1.0 / (1.0 + np.exp(-g))) * u)).mean() > 0.05     # the sigmoid rounded instead of silu
+
+
 def test_plain_model_cuts_agree_with_itself():
     # logits at position t depend on tokens 0..t only (causal), so a prefix gives the same rows
     raw = H.TINY_A

@@ -1132,3 +1132,65 @@ def test_small_product_plain_form_and_refusals(ops, M):
     with pytest.raises(ops.KernelError, match="unsupported shape"):
         ops._gemm8(torch.zeros(9, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV),
                    torch.zeros(9, 8, dtype=torch.bfloat16, device=DEV), 8, False)
+
+
+# ------------------------------------------------ where the order of rounding and multiplying shows
+def test_norm_and_swiglu_kernels_round_where_the_reference_rounds(ops):
+    """Inputs for which rounding before or after the multiply gives different 16-bit values (and which
+    stay clear of rounding boundaries by far more than 32-bit arithmetic can shift them): the kernels
+    give the plain functions' bits, element for element (src/cuda/kernels.cu:34-49 and 72-82)."""
+    import helpers as H
+    r = plain.round_bf16
+    x, w = H.norm_rounding_cases()
+    want = plain.rms_norm(x, w, 1e-6, r)
+    inv = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + 1e-6)
+    assert (want != r(w * x * inv)).mean() > 0.05
+    out = torch.zeros(x.shape, dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(_t(x, torch.float32), _t(w, torch.bfloat16), out, 1e-6)
+    np.testing.assert_array_equal(_np(out), want)
+    # the norm with the pending addition and the gathered form round at the same places
+    half = (x / 2).astype(np.float32).astype(np.float64)
+    assert np.array_equal(half * 2, x)
+    xt = _t(half, torch.float32)
+    out2 = torch.zeros_like(out)
+    ops.rmsnorm(xt, _t(w, torch.bfloat16), out2, 1e-6, add=_t(half, torch.float32))
+    np.testing.assert_array_equal(_np(out2), want)
+    rows = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
+    out3 = torch.zeros(2, x.shape[1], dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(_t(x, torch.float32), _t(w, torch.bfloat16), out3, 1e-6, rows=rows)
+    np.testing.assert_array_equal(_np(out3), want[[2, 0]])
+
+    g, u = H.swiglu_rounding_cases()
+    rows_, I = g.shape
+    act_want = plain.swiglu(np.concatenate([g, u], -1), r)
+    silu = g / (1.0 + np.exp(-g))
+    assert (act_want != r(silu * u)).mean() > 0.05
+    act = torch.zeros(rows_, I, dtype=torch.bfloat16, device=DEV)
+    ops.swiglu(_t(np.concatenate([g, u], -1), torch.bfloat16), act)
+    np.testing.assert_array_equal(_np(act), act_want)
+    # the same values as the result of a product: row m of X picks column m of the weights, so that the
+    # sums are the chosen gate and up values themselves; the products' SwiGLU epilogues round alike
+    K = 64
+    X = np.zeros((rows_, K))
+    X[np.arange(rows_), np.arange(rows_)] = 1.0
+    W = np.zeros((2 * I, K))
+    W[:I, :rows_] = g.T
+    W[I:, :rows_] = u.T
+    xt, wt = _t(X, torch.bfloat16), _t(W, torch.bfloat16)
+    fused = torch.zeros(rows_, I, dtype=torch.bfloat16, device=DEV)
+    ops._gemm8(xt, wt, fused, I, True)                                   # the product of at most 8 rows
+    np.testing.assert_array_equal(_np(fused), act_want)
+    for M in (rows_, 24):                                                # the weight-streaming products: up to 16 rows, and more
+        Xm = np.zeros((M, K))
+        Xm[:rows_] = X
+        wide = 5632                                                      # wide enough for the one-launch form to be taken
+        Wm = np.zeros((2 * wide, K))
+        Wm[:I, :] = W[:I]
+        Wm[wide:wide + I, :] = W[I:]
+        out_m = torch.zeros(M, wide, dtype=torch.bfloat16, device=DEV)
+        keep, ops.LIBRARY_GEMM_MIN_ROWS = ops.LIBRARY_GEMM_MIN_ROWS, 0
+        try:
+            assert ops.gemm_swiglu(_t(Xm, torch.bfloat16), _t(Wm, torch.bfloat16), out_m)
+        finally:
+            ops.LIBRARY_GEMM_MIN_ROWS = keep
+        np.testing.assert_array_equal(_np(out_m)[:rows_, :I], act_want)
