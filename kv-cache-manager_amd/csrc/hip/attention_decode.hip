@@ -156,8 +156,14 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
       pf.u.z = float_to_bf16_bits(b.x) | (uint32_t(float_to_bf16_bits(b.y)) << 16);
       pf.u.w = float_to_bf16_bits(b.z) | (uint32_t(float_to_bf16_bits(b.w)) << 16);
     }
+    // value slots past the context's end hold stale data, which zero probabilities do not cancel if it is Inf or NaN
+    const int left = end - (start + (wave * VSTEPS + j) * 32 + kq * 8);
 #pragma unroll
-    for (int d = 0; d < DT; ++d) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf[j][d].v, o[d], 0, 0, 0);
+    for (int d = 0; d < DT; ++d) {
+      Frag8 v = vf[j][d];
+      if (left < 8) v.u = keep_first_bf16(v.u, left);
+      o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, v.v, o[d], 0, 0, 0);
+    }
   }
   // accumulator: column = dim n16 of tile d, rows = heads 4*kq..+3
 #pragma unroll

@@ -296,12 +296,19 @@ __global__ void __launch_bounds__(WAVES* kWave, HD == 64 ? 8 / WAVES : 1)
       pf[g].u = uint4{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3]), pack2_bf16(p[4], p[5]), pack2_bf16(p[6], p[7])};
     }
     l_run = l_run * alpha + sum;
+    // this lane's 8 value slots of a group that reach past the context hold stale data: cut them
+    // (only the chunk with the context's end has such slots)
+    const bool cut = base + 40 > ctx;
 #pragma unroll
     for (int d = 0; d < DT; ++d) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
 #pragma unroll
-      for (int g = 0; g < 2; ++g) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ch.v[g][d].v, pf[g].v, o[d], 0, 0, 0);
+      for (int g = 0; g < 2; ++g) {
+        FragF vf = ch.v[g][d];
+        if (cut) vf.u = keep_first_bf16(vf.u, ctx - (base + g * 32));
+        o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[g].v, o[d], 0, 0, 0);
+      }
     }
   };
 

@@ -166,7 +166,7 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   // A thread's key pieces are the same 8 dims of PIECES consecutive tokens (an aligned group, so one
   // page), its value pieces the same 8 tokens of dims 32 apart: one page lookup each per chunk, the
   // other pieces lie a constant away.
-  struct Pieces { u32x4 k[PIECES], v[PIECES]; };
+  struct Pieces { u32x4 k[PIECES], v[PIECES]; int v_left; };   // v_left: how many of a value piece's 8 tokens lie inside what this workgroup may read
   constexpr int KTPR = HD / 8;   // threads per key row
   const int k_p = threadIdx.x / KTPR, k_col = threadIdx.x % KTPR;
   const int v_g = threadIdx.x % 8, v_d = threadIdx.x / 8;
@@ -178,6 +178,7 @@ __global__ void __launch_bounds__(kPfThreads, 2)
     const uint16_t* kp = kbase + size_t(page_lds[(t0 >> b_shift) - page_lo]) * page_elems + size_t(t0 & b_mask) * HD + k_col * 8;
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) pc.k[i] = *reinterpret_cast<const u32x4*>(kp + i * HD);
+    pc.v_left = block_last_pos + 1 - (c0 + v_g * 8);
     const int tv = min(c0 + v_g * 8, last_vgroup);
     const uint16_t* vp = vbase + size_t(page_lds[(tv >> b_shift) - page_lo]) * page_elems + size_t(v_d) * B + (tv & b_mask);
 #pragma unroll
@@ -193,8 +194,12 @@ __global__ void __launch_bounds__(kPfThreads, 2)
         const int r0 = (v_g * 8) % 32, grp = (v_g * 8) / 32;
         const int a = r0 / 16, q0 = (r0 % 16) / 4;
         uint16_t* dst = &v_lds[buf][v_d + 32 * i][grp * 32 + 4 * a];
-        *reinterpret_cast<uint2*>(dst + 8 * q0) = uint2{pc.v[i][0], pc.v[i][1]};
-        *reinterpret_cast<uint2*>(dst + 8 * (q0 + 1)) = uint2{pc.v[i][2], pc.v[i][3]};
+        uint4 piece{pc.v[i][0], pc.v[i][1], pc.v[i][2], pc.v[i][3]};
+        // slots past the last position hold stale data (or, from the clamped address, other tokens):
+        // probabilities there are zero, which does not cancel a stale Inf or NaN
+        if (pc.v_left < 8) piece = keep_first_bf16(piece, pc.v_left);
+        *reinterpret_cast<uint2*>(dst + 8 * q0) = uint2{piece.x, piece.y};
+        *reinterpret_cast<uint2*>(dst + 8 * (q0 + 1)) = uint2{piece.z, piece.w};
       }
     }
   };

@@ -54,6 +54,14 @@ __device__ __forceinline__ void rotate_pair(float& a, float& b, float cs, float 
   b = rb;
 }
 
+// A 16-byte piece of 8 bfloat16 with only its first n (0..8) kept, the others zero.  Value pieces that
+// reach past a context's end hold whatever the page's previous owner left there; their probabilities
+// are zero, but zero times a stale Inf or NaN would not be: such pieces are cut before they are multiplied.
+__device__ __forceinline__ uint4 keep_first_bf16(uint4 v, int n) {
+  auto word = [n](int j) -> uint32_t { return n >= 2 * j + 2 ? 0xFFFFFFFFu : (n == 2 * j + 1 ? 0x0000FFFFu : 0u); };
+  return uint4{v.x & word(0), v.y & word(1), v.z & word(2), v.w & word(3)};
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

@@ -1194,3 +1194,58 @@ def test_norm_and_swiglu_kernels_round_where_the_reference_rounds(ops):
         finally:
             ops.LIBRARY_GEMM_MIN_ROWS = keep
         np.testing.assert_array_equal(_np(out_m)[:rows_, :I], act_want)
+
+
+# ------------------------------------------------ what a page's previous owner left behind
+def _poison_beyond_contexts(P, lens, B):
+    """Every key and value slot that no sequence of the problem owns (the tails of last pages, the spare
+    pages) gets NaN and Inf: what a reused page may hold when its previous owner's values blew up."""
+    owned = np.zeros(P["Kc"].shape[:1] + (B,), dtype=bool)
+    for s, c in enumerate(lens):
+        for t in range(c):
+            owned[P["tables"][s, t // B], t % B] = True
+    bad = np.where(np.arange(owned.size).reshape(owned.shape) % 2 == 0, np.nan, np.inf)
+    for cache in (P["Kc"], P["Vc"]):
+        for h in range(cache.shape[1]):
+            cache[:, h][~owned] = np.broadcast_to(bad[~owned][:, None], cache[:, h][~owned].shape)
+    assert (~owned).sum() > 20
+
+
+@pytest.mark.parametrize("nh,nkv,hd,B", [(8, 2, 64, 16), (6, 2, 128, 32), (32, 4, 64, 8)])
+def test_stale_values_past_a_context_do_not_reach_the_output(ops, nh, nkv, hd, B):
+    """Probabilities of slots past a context's end are zero, but zero times a stale NaN or Inf is not:
+    the matrix-core kernels cut such slots out of their value pieces.  All four attention kernels."""
+    rng = np.random.default_rng(nh + B)
+    lens = [700, 257, 33, 1, 250, 511, 9]
+    P = _paged_problem(rng, lens, nh, nkv, hd, B, all_rows=False)
+    ref = _ref_attention(P, nh, nkv, hd)
+    _poison_beyond_contexts(P, lens, B)
+    R = P["R"]
+    scale = 1.0 / math.sqrt(hd)
+    kc, vc = _t(P["Kc"], torch.bfloat16), _vt(P["Vc"], torch.bfloat16)
+    assert torch.isnan(vc.float()).any() and torch.isinf(kc.float()).any()
+    tables, row_seq, ctx = _t(P["tables"], torch.int32), _t(P["row_seq"], torch.int32), _t(P["ctx"], torch.int32)
+    q = _t(P["Q"].reshape(R, nh * hd), torch.bfloat16)
+
+    generic = torch.zeros(R, nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention(q, generic, kc, vc, tables, P["max_blocks"], row_seq, ctx, nh, nkv, hd, scale)
+    partitioned = torch.zeros_like(generic)
+    scratch = torch.zeros(ops.attention_decode_scratch(R, nh, hd, 1024), dtype=torch.float32, device=DEV)
+    ops.attention_decode(q, partitioned, kc, vc, tables, P["max_blocks"], row_seq, ctx, nh, nkv, hd, scale, 1024, scratch)
+    fused = torch.zeros_like(generic)
+    qkv = torch.zeros(R, (nh + 2 * nkv) * hd, dtype=torch.bfloat16, device=DEV)
+    qkv[:, :nh * hd] = q
+    ops.attention_decode_fused(qkv, fused, kc, vc, tables, P["max_blocks"], row_seq, ctx, nh, nkv, hd, scale, max_context=1024)
+    for name, out in (("generic", generic), ("partitioned", partitioned), ("fused", fused)):
+        got = _np(out).reshape(R, nh, hd)
+        assert np.isfinite(got).all(), name
+        np.testing.assert_allclose(got, ref, atol=1e-2, rtol=0, err_msg=name)
+
+    # runs of positions whose last row lies in the middle of a group of 8 slots and of a page
+    runs = [(0, 130), (77, 2), (200, 51), (15, 64), (0, 3)]
+    Pr = _runs_problem(rng, runs, nh, nkv, hd, B)
+    want = _ref_attention(Pr, nh, nkv, hd)
+    _poison_beyond_contexts(Pr, [s + n for s, n in runs], B)
+    got = _run_prefill(ops, Pr, runs, nh, nkv, hd)
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, want, atol=1.5e-2, rtol=0)
