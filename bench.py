@@ -20,7 +20,8 @@ sys.path.insert(0, ROOT)
 HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 
-# BASELINE.json configs[2]: TinyLlama-1.1B sizes
+# TinyLlama-1.1B sizes: 22 layers of width 2048, 32 query heads and 4 key/value heads of 64, SwiGLU width
+# 5632, vocabulary 32000, context 2048
 SIZES = dict(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_hidden_layers=22,
              num_attention_heads=32, num_key_value_heads=4, head_dim=64, max_position_embeddings=2048,
              rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
@@ -82,6 +83,38 @@ def prefill_run(eng, tokens, vocab, reps=3):
         assert info.prefill_tokens == tokens
         eng.take_finished()
     return sorted(times[1:])[len(times[1:]) // 2]     # median, first one is warm-up
+
+
+def measured_peaks():
+    """What this GPU does in this run, beside the published peaks: GB/s of a copy kernel (1 GiB read and
+    written), GB/s of a read-only kernel over 2 GiB, and TFLOP/s of a loop of bfloat16 matrix instructions
+    that touches no memory.  Median of five launches each, timed by device events."""
+    import torch
+    from kvcm_amd import ops
+    src = torch.zeros(1 << 29, dtype=torch.int32, device="cuda:0")       # 2 GiB
+    dst = torch.empty(1 << 28, dtype=torch.int32, device="cuda:0")       # 1 GiB
+    sink = torch.zeros(256, dtype=torch.float32, device="cuda:0")
+
+    def timed(fn):
+        ms = []
+        for _ in range(6):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            b.synchronize()
+            ms.append(a.elapsed_time(b))
+        return sorted(ms[1:])[2] * 1e-3
+
+    copy_s = timed(lambda: ops.probe_copy(src[:1 << 28], dst, grid=4096))
+    read_s = timed(lambda: ops.probe_read(src, sink, grid=4096))
+    flops = []
+    mfma_s = timed(lambda: flops.append(ops.probe_mfma(20000, sink, grid=2048)))
+    out = {"hbm_copy_GBs": round(2 * (1 << 30) / copy_s / 1e9, 1), "hbm_read_GBs": round((1 << 31) / read_s / 1e9, 1),
+           "mfma_bf16_TFLOPs": round(flops[-1] / mfma_s / 1e12, 1)}
+    del src, dst
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -164,6 +197,8 @@ def main():
             points[f"decode_b{b}_hbm_frac"] = roofline(b, s / k, c)["frac"]
         out["points"] = points
         out["prefill"] = prefill_record()
+        # beside the published peaks the fractions above are taken against: what this GPU reached in this run
+        out["measured"] = measured_peaks()
     print(json.dumps(out), flush=True)
 
 

@@ -23,6 +23,15 @@ at position START of its sequence (default 0), ``--seqs`` such sequences in one 
 and values behind a shuffled block table.  TFLOP/s counts the causal work, 4 * head_dim * heads *
 (keys each row sees), against the bf16 matrix-core peak; the last columns say how the launch was
 cut (query rows per workgroup, keys per segment).
+
+  --floor [--nodes 156]                          (not in the reference)
+
+times what a launch costs and how fast memory streams inside a chain of dependent launches like a
+decode step's: ``--nodes`` launches of one probe kernel after the other, as plain stream launches and
+as one captured HIP graph: an empty kernel (1 and 1,024 workgroups), a kernel that reads what the one
+before it wrote (64 KB, 1 MB), and kernels that stream 8, 23 and 46 MB each from a 2 GiB buffer (the
+sizes of a TinyLlama layer's weight matrices; consecutive launches read consecutive regions, so that
+the bytes come from HBM and not from a cache).
 """
 import sys
 
@@ -33,6 +42,70 @@ from .args import Args
 PEAK_GBS = 8000.0      # MI355X HBM3E
 PEAK_BF16_TFLOPS = 2500.0
 WAVE_SLOTS_PER_CU = 32
+
+
+def _floor(nodes):
+    import torch
+    from .. import ops
+    ops.lib()
+    dev = torch.device("cuda:0")
+    big = torch.zeros(1 << 29, dtype=torch.int32, device=dev)            # 2 GiB
+    ping, pong = torch.zeros(1 << 18, dtype=torch.int32, device=dev), torch.zeros(1 << 18, dtype=torch.int32, device=dev)
+    sink = torch.zeros(256, dtype=torch.float32, device=dev)
+    total = big.numel() * 4
+
+    def chain_empty(grid, block):
+        return lambda i: ops.probe_empty(grid, block)
+
+    def chain_touch(nbytes, grid):
+        n = nbytes // 4
+        return lambda i: ops.probe_copy(ping[:n] if i % 2 == 0 else pong[:n], pong[:n] if i % 2 == 0 else ping[:n], grid=grid)
+
+    def chain_stream(nbytes, grid):
+        n = nbytes // 4
+        def launch(i):
+            lo = (i * n) % (big.numel() - n)
+            lo -= lo % 4
+            ops.probe_read(big[lo:lo + n], sink, grid=grid)
+        return launch
+
+    cases = [("empty <<<1,64>>>", chain_empty(1, 64), 0), ("empty <<<1024,256>>>", chain_empty(1024, 256), 0),
+             ("reads what the last wrote, 64 KB", chain_touch(64 << 10, 16), 0),
+             ("reads what the last wrote, 1 MB", chain_touch(1 << 20, 256), 0),
+             ("streams 8 MB", chain_stream(8 << 20, 512), 8 << 20), ("streams 23 MB", chain_stream(23 << 20, 1024), 23 << 20),
+             ("streams 46 MB", chain_stream(46 << 20, 1024), 46 << 20)]
+    print(f"{nodes} launches in a row; microseconds per launch")
+    print("%-36s %10s %10s %12s" % ("kernel", "stream", "graph", "graph TB/s"))
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for name, launch, nbytes in cases:
+            def run_all():
+                for i in range(nodes):
+                    launch(i)
+            run_all()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            stream.synchronize()
+            e0.record()
+            for _ in range(10):
+                run_all()
+            e1.record()
+            e1.synchronize()
+            eager = 1e3 * e0.elapsed_time(e1) / (10 * nodes)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                run_all()
+            for _ in range(3):
+                graph.replay()
+            stream.synchronize()
+            e0.record()
+            for _ in range(30):
+                graph.replay()
+            e1.record()
+            e1.synchronize()
+            g = 1e3 * e0.elapsed_time(e1) / (30 * nodes)
+            rate = "%.2f" % (nbytes / g / 1e6) if nbytes else ""
+            print("%-36s %10.2f %10.2f %12s" % (name, eager, g, rate))
+    return 0
 
 
 def _ints(s):
@@ -46,9 +119,12 @@ def main(argv=None):
     iters, out_csv = a.i32("iters", 100), a.str("out", "")
     use_graph = a.flag("graph")
     prefill, seqs = a.str("prefill", ""), a.i32("seqs", 1)
+    floor, nodes = a.flag("floor"), a.i32("nodes", 156)
     a.warn_unused()
     if prefill:
         return _prefill(prefill, seqs, blocks, heads, kvh, hd, iters, out_csv, use_graph)
+    if floor:
+        return _floor(nodes)
 
     import torch
     from .. import ops

@@ -106,6 +106,12 @@ int kvcm_sample(const float* logits, int ld, const float* temperature, const uin
 int kvcm_fill_normal(void* out, int dtype, long long n, uint64_t key, float mean, float std, hipStream_t s);
 int kvcm_fill_index(int* out, long long n, uint64_t key, int modulus, hipStream_t s);
 
+// ---- probes of the machine (probe.hip) -----------------------------------------------------------
+int kvcm_probe_empty(int grid, int block, hipStream_t s);
+int kvcm_probe_copy(const void* src, void* dst, long long bytes, int grid, hipStream_t s);      // moves 2 * bytes
+int kvcm_probe_read(const void* src, long long bytes, void* sink, int grid, hipStream_t s);
+int kvcm_probe_mfma(int iters, void* sink, int grid, hipStream_t s);   // grid * 4 waves * iters * 4 * 32768 flops
+
 // ---- recorded steps ---------------------------------------------------------------------------
 // A step program is the list of launches of one step, recorded once for a step shape and replayed
 // with nothing but the step's metadata changed (the kernels read that from device memory).  The

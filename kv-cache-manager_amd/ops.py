@@ -66,6 +66,10 @@ def _declare(lib):
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
     fn("kvcm_gemm_library", vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, vp)
+    fn("kvcm_probe_empty", i, i, vp)
+    fn("kvcm_probe_copy", vp, vp, C.c_longlong, i, vp)
+    fn("kvcm_probe_read", vp, C.c_longlong, vp, i, vp)
+    fn("kvcm_probe_mfma", i, vp, i, vp)
     fn("kvcm_fill_normal", vp, i, C.c_longlong, C.c_uint64, f, f, vp)
     fn("kvcm_fill_index", vp, C.c_longlong, C.c_uint64, i, vp)
     fn("kvcm_gemm8_supported", i, i, i)
@@ -700,6 +704,34 @@ def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, s
                                         _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), num_seqs, max_run,
                                         T, int(max_context), nh, nkv, hd, kcache.shape[2], float(scale), _ptr(scratch),
                                         scratch.numel() if scratch is not None else 0, _stream())
+
+
+# ------------------------------------------------------------------------- probes of the machine
+def probe_empty(grid=1, block=64):
+    _check(lib().kvcm_probe_empty(int(grid), int(block), _stream()))
+
+
+def probe_copy(src, dst, grid=2048):
+    """dst = src + 1 over 16-byte pieces; moves 2 * src.nbytes."""
+    _dev(src, dst)
+    n = src.numel() * src.element_size()
+    _need(src.is_contiguous() and dst.is_contiguous() and dst.numel() * dst.element_size() >= n and n % 16 == 0, "probe_copy needs contiguous buffers of whole 16-byte pieces")
+    _check(lib().kvcm_probe_copy(_ptr(src), _ptr(dst), n, int(grid), _stream()))
+
+
+def probe_read(src, sink, grid=2048, nbytes=None):
+    _dev(src, sink)
+    n = src.numel() * src.element_size() if nbytes is None else int(nbytes)
+    _need(src.is_contiguous() and n % 16 == 0 and n <= src.numel() * src.element_size() and sink.numel() * sink.element_size() >= 1024, "probe_read needs whole 16-byte pieces and a sink of 1 KiB")
+    _check(lib().kvcm_probe_read(_ptr(src), n, _ptr(sink), int(grid), _stream()))
+
+
+def probe_mfma(iters, sink, grid=2048):
+    """-> flops of the launch: grid workgroups x 4 waves x iters x 4 instructions x 32768."""
+    _dev(sink)
+    _need(sink.numel() * sink.element_size() >= 1024, "probe_mfma needs a sink of 1 KiB")
+    _check(lib().kvcm_probe_mfma(int(iters), _ptr(sink), int(grid), _stream()))
+    return int(grid) * 4 * int(iters) * 4 * 32768
 
 
 def fill_normal(out, key, mean=0.0, std=1.0):
