@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine at TinyLlama-1.1B sizes with random weights.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512] [--layers L]
+                  [--sizes tinyllama-1.1b|llama-2-7b|llama-3-8b] [--context-limit 2048]
 
 A "step" is one decode step of the whole engine (schedule, batch metadata, upload, model step on
 the GPU, sampling, download, update).  W untimed steps, then exactly K timed steps between two
@@ -27,13 +28,22 @@ SIZES = dict(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_hid
              rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
 
 
-def build_engine(cfg, dtype, max_num_seqs, max_batched_tokens, tensors):
+def build_engine(cfg, dtype, max_num_seqs, max_batched_tokens, tensors, context_limit=2048):
     from kvcm_amd.config.engine_config import EngineConfig
     from kvcm_amd.engine.engine import Engine
-    ec = EngineConfig(block_size=16, max_seq_len=2048, num_blocks=max_num_seqs * 2048 // 16,
+    ec = EngineConfig(block_size=16, max_seq_len=context_limit, num_blocks=max_num_seqs * context_limit // 16,
                       max_num_seqs=max_num_seqs, max_batched_tokens=max_batched_tokens, dtype=dtype,
-                      max_logit_rows=max(max_num_seqs, 64))
+                      max_logit_rows=max(max_num_seqs, 64),
+                      # random weights rotate any position: a context limit beyond the sizes' own is allowed
+                      beyond_max_position=context_limit > cfg.max_position_embeddings)
     return Engine(config=ec, architecture="LlamaForCausalLM", model_config=cfg, tensors=tensors)
+
+
+def prompt_step_count(batch, prompt_len, budget=4096):
+    """Steps that the prompts of a batch take at most: whole prompts, as many a step as the token budget
+    holds beside the tokens of the requests that decode already."""
+    per_step = max(1, (budget - batch) // prompt_len)
+    return -(-batch // per_step) + 2
 
 
 def decode_run(eng, batch, prompt_len, steps, warmup, vocab, seed=1):
@@ -42,7 +52,7 @@ def decode_run(eng, batch, prompt_len, steps, warmup, vocab, seed=1):
     import torch
     rng = np.random.default_rng(seed)
     # requests admitted first decode while the others' prompts still run: room for those steps too
-    prompt_steps = -(-batch * prompt_len // 3584) + 2
+    prompt_steps = prompt_step_count(batch, prompt_len, eng.config.max_batched_tokens)
     for _ in range(batch):
         eng.add_request(rng.integers(3, vocab, size=prompt_len).tolist(), max_new_tokens=warmup + steps + 24 + prompt_steps)
     extra = 0
@@ -126,6 +136,8 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--sizes", default="tinyllama-1.1b", help="layer sizes by name (tinyllama-1.1b, llama-2-7b, llama-3-8b)")
+    ap.add_argument("--context-limit", type=int, default=2048, help="most tokens a request may hold; sizes the cache pool")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
@@ -138,7 +150,12 @@ def main():
     from kvcm_amd.config.model_config import LlamaConfig
     from kvcm_amd.weights.random_init import random_tensors
 
-    sizes = dict(SIZES)
+    from kvcm_amd.cli.common import NAMED_SIZES
+    if args.sizes not in NAMED_SIZES:
+        print("bench.py: unknown --sizes %r; known: %s" % (args.sizes, sorted(NAMED_SIZES)))
+        sys.exit(2)
+    sizes = dict(SIZES if args.sizes == "tinyllama-1.1b" else NAMED_SIZES[args.sizes])
+    label = {"tinyllama-1.1b": "TinyLlama-1.1B", "llama-2-7b": "Llama-2-7B", "llama-3-8b": "Llama-3-8B"}.get(args.sizes, args.sizes)
     full_layers = sizes["num_hidden_layers"]
     if args.layers:
         sizes["num_hidden_layers"] = args.layers
@@ -158,7 +175,14 @@ def main():
         return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_GBS, 4)}
 
-    eng = build_engine(cfg, args.dtype, max_num_seqs=max(64, args.batch), max_batched_tokens=4096, tensors=tensors)
+    limit = args.context_limit
+    budget = max(4096, args.prompt_len + args.batch)     # a whole prompt fits a step beside the decoding requests
+    if args.prompt_len + args.warmup + args.steps + 24 + prompt_step_count(args.batch, args.prompt_len, budget) > limit:
+        print("bench.py: --prompt-len %d plus the decoded tokens does not fit --context-limit %d" % (args.prompt_len, limit))
+        sys.exit(2)
+    # the pool holds every request of the largest batch at the context limit
+    seqs = args.batch if (args.no_points or args.only_prefill) else max(64, args.batch)
+    eng = build_engine(cfg, args.dtype, max_num_seqs=seqs, max_batched_tokens=budget, tensors=tensors, context_limit=limit)
     del tensors
     torch.cuda.empty_cache()
 
@@ -177,15 +201,15 @@ def main():
     seconds, ctx = decode_run(eng, args.batch, args.prompt_len, args.steps, args.warmup, V)
     value = args.batch * args.steps / seconds
     out = {
-        "metric": "decode tok/s at batch %d (TinyLlama-1.1B sizes, %d-token prompts)" % (args.batch, args.prompt_len),
+        "metric": "decode tok/s at batch %d (%s sizes, %d-token prompts)" % (args.batch, label, args.prompt_len),
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(1e3 * seconds / args.steps, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": key, "data": "synthetic",
-        "config": {"model": "TinyLlama-1.1B sizes, random weights N(0,0.02)", "global_batch": args.batch,
+        "config": {"model": "%s sizes, random weights N(0,0.02)" % label, "global_batch": args.batch,
                    "seq_len": args.prompt_len, "parallelism": "single GPU", "layers": L, "layers_full": full_layers,
                    "hidden": H, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": I, "vocab": V, "kv_block": 16,
-                   "context_limit": 2048, "generated": args.warmup + args.steps},
+                   "context_limit": limit, "generated": args.warmup + args.steps},
         "roofline": roofline(args.batch, seconds / args.steps, ctx),
     }
     if not args.no_points:
