@@ -28,12 +28,12 @@ SIZES = dict(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_hid
              rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
 
 
-def build_engine(cfg, dtype, max_num_seqs, max_batched_tokens, tensors, context_limit=2048):
+def build_engine(cfg, dtype, max_num_seqs, max_batched_tokens, tensors, context_limit=2048, tune_products="heuristic"):
     from kvcm_amd.config.engine_config import EngineConfig
     from kvcm_amd.engine.engine import Engine
     ec = EngineConfig(block_size=16, max_seq_len=context_limit, num_blocks=max_num_seqs * context_limit // 16,
                       max_num_seqs=max_num_seqs, max_batched_tokens=max_batched_tokens, dtype=dtype,
-                      max_logit_rows=max(max_num_seqs, 64),
+                      max_logit_rows=max(max_num_seqs, 64), tune_products=tune_products,
                       # random weights rotate any position: a context limit beyond the sizes' own is allowed
                       beyond_max_position=context_limit > cfg.max_position_embeddings)
     return Engine(config=ec, architecture="LlamaForCausalLM", model_config=cfg, tensors=tensors)
@@ -137,6 +137,10 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--sizes", default="tinyllama-1.1b", help="layer sizes by name (tinyllama-1.1b, llama-2-7b, llama-3-8b)")
+    ap.add_argument("--tune-products", default="heuristic", choices=["off", "heuristic", "all"],
+                    help="which of the vendor library's algorithms the many-row products of prompt steps run: its first "
+                         "choice, the fastest of its choices (the engine's default), or the fastest of all; timed at a "
+                         "shape's first use, before anything is measured")
     ap.add_argument("--context-limit", type=int, default=2048, help="most tokens a request may hold; sizes the cache pool")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true",
@@ -182,7 +186,8 @@ def main():
         sys.exit(2)
     # the pool holds every request of the largest batch at the context limit
     seqs = args.batch if (args.no_points or args.only_prefill) else max(64, args.batch)
-    eng = build_engine(cfg, args.dtype, max_num_seqs=seqs, max_batched_tokens=budget, tensors=tensors, context_limit=limit)
+    eng = build_engine(cfg, args.dtype, max_num_seqs=seqs, max_batched_tokens=budget, tensors=tensors, context_limit=limit,
+                       tune_products=args.tune_products)
     del tensors
     torch.cuda.empty_cache()
 
@@ -209,7 +214,8 @@ def main():
                    "seq_len": args.prompt_len, "parallelism": "single GPU", "layers": L, "layers_full": full_layers,
                    "hidden": H, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": I, "vocab": V, "kv_block": 16,
-                   "context_limit": limit, "generated": args.warmup + args.steps},
+                   "context_limit": limit, "generated": args.warmup + args.steps,
+                   "tune_products": args.tune_products},
         "roofline": roofline(args.batch, seconds / args.steps, ctx),
     }
     if not args.no_points:

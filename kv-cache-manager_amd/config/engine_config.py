@@ -25,6 +25,8 @@ class EngineConfig:
     use_graphs: bool = True          # replay decode-only steps from captured HIP graphs (models whose parts are all capturable)
     use_programs: bool = True        # replay other step shapes from natively recorded launch lists (same condition)
     beyond_max_position: bool = False  # False: max_seq_len is cut down to the model's max_position_embeddings (with a notice)
+    tune_products: str = "heuristic"   # which library algorithm a many-row product runs: "off" the library's first choice,
+                                       # "heuristic" its choices timed at a shape's first use, "all" every algorithm (seconds per shape)
 
     def validate(self):
         if self.policy not in ("paged", "contiguous"):
@@ -33,6 +35,8 @@ class EngineConfig:
             raise ValueError(f"unknown attention version: {self.attn} (v1 | v2 | auto)")
         if self.dtype not in ("bfloat16", "float32", "bf16", "fp32"):
             raise ValueError(f"unknown dtype: {self.dtype} (bfloat16 | float32)")
+        if self.tune_products not in ("off", "heuristic", "all"):
+            raise ValueError(f"unknown tune_products: {self.tune_products} (off | heuristic | all)")
         for name in ("block_size", "max_seq_len", "max_num_seqs", "max_batched_tokens"):
             if getattr(self, name) <= 0:
                 raise ValueError(f"{name} must be positive")

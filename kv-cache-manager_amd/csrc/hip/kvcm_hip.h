@@ -76,6 +76,17 @@ int kvcm_gemm8_residual_norm(const void* X, int ldx, const void* W, int ldw, int
 long long kvcm_gemm_library_workspace_bytes();
 int kvcm_gemm_library(const void* X, const void* W, void* out, int M, int N, int K, int ldx, int ldw, int ldo,
                       void* workspace, long long workspace_bytes, hipStream_t stream);
+// Which algorithm of the library a shape runs: the heuristic's first choice until this has timed
+// candidates on the shape's own operands (mode 1: the heuristic's choices, a few milliseconds; mode 2:
+// every algorithm that supports the shape, at most max_seconds) and kept the fastest whose result
+// agrees with the first choice's.  W: w_copies copies of the weights, w_copy_bytes apart, which timed
+// calls go round (enough of them keep the weights out of the caches, as in a model of many layers).
+// `check`: M * N bfloat16 + 8 bytes of device memory; `report` (host, may be null): microseconds of the
+// first choice, of the kept one, candidates timed.  Synchronises the stream.
+int kvcm_gemm_library_tuned(int M, int N, int K, int ldx, int ldw, int ldo);
+int kvcm_gemm_library_tune(const void* X, const void* W, int w_copies, long long w_copy_bytes, void* out, int M, int N, int K,
+                           int ldx, int ldw, int ldo, void* workspace, long long workspace_bytes, void* check, int mode,
+                           double max_seconds, double* report, hipStream_t stream);
 
 // ---- attention over the paged cache ----------------------------------------------------------
 int kvcm_attention_generic(const void* q, int dtype, int q_stride, void* out, int out_stride, const void* kcache,

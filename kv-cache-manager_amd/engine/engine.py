@@ -38,6 +38,7 @@ class Engine:
         self._forced, self._forced_logits = {}, {}       # request id -> forced tokens / logits kept for them
         self._t0 = time.perf_counter()
         self.config = self.runner.engine_config      # as built (max_seq_len within the model's range)
+        self.runner.ops.LIBRARY_TUNING = self.config.tune_products      # process-wide, like the library's plans
         # Recorded steps replay a fixed launch sequence: only for models whose parts all declare that
         # their launches depend on the step's shape alone (Part.capturable).  use_programs: steps are
         # recorded per shape and replayed natively; use_graphs: decode-shaped ones also as HIP graphs.

@@ -66,6 +66,9 @@ def _declare(lib):
     lib.kvcm_attention_decode_scratch.argtypes = [i, i, i, i]
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
     fn("kvcm_gemm_library", vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, vp)
+    fn("kvcm_gemm_library_tuned", i, i, i, i, i, i)
+    fn("kvcm_gemm_library_tune", vp, vp, i, C.c_longlong, vp, i, i, i, i, i, i, vp, C.c_longlong, vp, i, C.c_double,
+       C.POINTER(C.c_double), vp)
     fn("kvcm_probe_empty", i, i, vp)
     fn("kvcm_probe_copy", vp, vp, C.c_longlong, i, vp)
     fn("kvcm_probe_read", vp, C.c_longlong, vp, i, vp)
@@ -427,6 +430,17 @@ def add_residual(x, y):
 LIBRARY_GEMM_MIN_ROWS = 96
 
 
+# Which of the library's algorithms a shape runs.  "off": the first choice of the library's heuristic.
+# "heuristic": at a shape's first use the heuristic's choices (up to 16) are timed on the call's own
+# operands and the fastest is kept (a few milliseconds per shape).  "all": every algorithm of the library
+# that supports the shape is timed (1 to 4 seconds per shape, at most LIBRARY_TUNING_SECONDS): for
+# long-running servers and measurements, switched on by the engine's configuration.
+LIBRARY_TUNING = "heuristic"
+LIBRARY_TUNING_SECONDS = 6.0
+LIBRARY_TUNING_BYTES = 512 << 20
+_TUNING_MODES = {"off": 0, "heuristic": 1, "all": 2}
+library_tuning_log = []          # (M, N, K, first choice's us, kept us, candidates timed) per tuned shape
+
 _library_ws = None
 
 
@@ -490,6 +504,24 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
         return partial if keep_partial else partial.materialize()
     if library:
         ws = _library_workspace(out.device)
+        mode = _TUNING_MODES[LIBRARY_TUNING]
+        shape = (M, N, K, x.stride(0), w.stride(0), out.stride(0))
+        if mode and lib().kvcm_gemm_library_tuned(*shape) < mode:
+            # not a recorded launch: it runs here, once, whoever is recording
+            check = torch.empty(M * N + 4, dtype=torch.bfloat16, device=out.device)
+            # copies of the weights that timed calls go round, about LIBRARY_TUNING_BYTES in all: a model's layers
+            # bring theirs from memory, not from a cache that one matrix alone would stay in
+            span = (N - 1) * w.stride(0) + K
+            copies = max(1, min(16, LIBRARY_TUNING_BYTES // (2 * span)))
+            rows = torch.empty(copies, span, dtype=torch.bfloat16, device=out.device)
+            rows.copy_(torch.as_strided(w, (span,), (1,)).unsqueeze(0).expand(copies, span))
+            report = (C.c_double * 3)()
+            rc = lib().kvcm_gemm_library_tune(_ptr(x), _ptr(rows), copies, 2 * span, _ptr(out), *shape, _ptr(ws), ws.numel(),
+                                              _ptr(check), mode, float(LIBRARY_TUNING_SECONDS), report, _stream())
+            del rows, check
+            if rc != 0:
+                raise KernelError(lib().kvcm_hip_last_error().decode())
+            library_tuning_log.append((M, N, K, report[0], report[1], int(report[2])))
         _call("kvcm_gemm_library", _ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0),
               _ptr(ws), ws.numel(), _stream())
         return out

@@ -594,6 +594,42 @@ def test_gemm_shared_rows_beyond_64_rows(ops, M, N, K):
         ops.LIBRARY_GEMM_MIN_ROWS = keep
 
 
+@pytest.mark.parametrize("mode", ["off", "heuristic", "all"])
+@pytest.mark.parametrize("M,N,K", [(96, 192, 320), (200, 2560, 512), (333, 328, 136)])
+def test_library_product_with_each_choice_of_algorithm(ops, mode, M, N, K):
+    """Many-row products go to the vendor library; which of its algorithms runs is its heuristic's first
+    choice, or the fastest of the timed candidates whose result agrees with that one's.  Whatever was
+    chosen, the product is x w^T, the choice is made once per shape, and a view with a row stride works."""
+    rng = np.random.default_rng(M + N + K)
+    x = _bf16_grid(rng.normal(size=(M, K)))
+    w_all = _bf16_grid(rng.normal(size=(N, K + 8)) * 0.05)
+    w = w_all[:, :K]
+    ref = plain.linear(x, w)
+    xt = _t(x, torch.bfloat16)
+    wt = _t(w_all, torch.bfloat16)[:, :K]                    # rows K + 8 apart
+    keep = ops.LIBRARY_TUNING
+    ops.LIBRARY_TUNING = mode
+    try:
+        shape = (M, N, K, K, K + 8, N)
+        want = {"off": 0, "heuristic": 1, "all": 2}[mode]
+        out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        before = len(ops.library_tuning_log)
+        ops.gemm(xt, wt, out)
+        np.testing.assert_allclose(_np(out), ref, rtol=2 ** -7, atol=1e-3)
+        assert ops.lib().kvcm_gemm_library_tuned(*shape) >= want
+        logged = len(ops.library_tuning_log)
+        assert logged - before <= (1 if want else 0)
+        if logged > before:
+            m, n, k, first_us, kept_us, timed = ops.library_tuning_log[-1]
+            assert (m, n, k) == (M, N, K) and timed >= 1 and 0 < kept_us and 0 < first_us
+        again = torch.zeros_like(out)
+        ops.gemm(xt, wt, again)                               # the shape is tuned: nothing is timed again
+        assert len(ops.library_tuning_log) == logged
+        assert torch.equal(again, out)
+    finally:
+        ops.LIBRARY_TUNING = keep
+
+
 def test_partial_sums_feed_the_fused_norm_and_rope(ops):
     rng = np.random.default_rng(30)
     M, H, K = 5, 2048, 2048
