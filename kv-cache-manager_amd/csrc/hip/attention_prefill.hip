@@ -4,10 +4,18 @@
 // (src/cuda/paged_attention.cu:50-183, docs/design.md:113-114): every row re-reads all its keys.
 //
 // Here a workgroup takes 128 query rows of one head, each of its four waves 32 of them (two
-// 16-row tiles; in small launches at head_dim 64: 64 rows, one tile per wave), and walks the keys
-// 64 at a time with a running maximum (no score buffer).  A
+// 16-row tiles), and walks the keys 64 at a time with a running maximum (no score buffer).  A
 // chunk of keys and values is staged in LDS once per workgroup, double-buffered: the next chunk's
 // global loads are in flight while the current one is multiplied.
+//
+// A launch ends when its longest walk does, and a wave needs about a microsecond for a chunk
+// whatever else the chip does.  Launches of little work at head_dim 64 take 64 rows per workgroup
+// (one tile per wave: twice the workgroups, each with fewer registers), and those that leave CUs
+// without a full set of waves (a prompt of up to 1,024 tokens: 512 workgroups) eight waves: four
+// groups of 16 rows times two halves of a 128-key trip, so that the longest walk is half as many
+// trips; the halves' running maxima, sums and outputs meet in LDS at the end (1,024 tokens: 17.1 ->
+// 14.7 us; where every CU has work for all its waves anyway the eight waves are slower: 2,048 tokens
+// 43.5 against 37.3 us, eight portions of 300 tokens 23.9 against 19.9 us).
 //
 // Both products run on the matrix cores (v_mfma_f32_16x16x32_bf16), transposed:
 //   S^T[token][row] = K[token][dim] * Q^T[dim][row]      A = keys as they lie ([slot][dim]),  B = Q
@@ -49,16 +57,16 @@ union PFrag {
   bf16x8 v;
 };
 
-constexpr int kPfWaves = 4;
-constexpr int kPfThreads = kPfWaves * kWave;
+constexpr int kPfWaves = 4;                      // row groups of a workgroup (waves, or pairs of waves that halve a trip's keys)
+constexpr int kPfGroupThreads = kPfWaves * kWave;
 // A wave takes RT tiles of 16 query rows, a workgroup 64 RT rows: two tiles (128 rows) by default, one
 // (64 rows) for launches of little work at head_dim 64, where twice the workgroups, each with fewer
 // registers (four to a CU instead of two), hide one another's waits better than a workgroup's
 // larger share of every staged chunk saves.
 constexpr int kPfMaxRT = 2;
 constexpr int kPfSmallWork = 35 * 256;           // 128-row workgroup chunks (about 35 per CU) up to which hd 64 takes 64-row tiles
-constexpr int kPfChunk = 64;                     // keys per trip
-constexpr int kPfPad = 8;                        // bfloat16 of padding per LDS row (keeps 16-byte alignment)
+constexpr long long kPfFewGroups = 512;           // workgroups (two per CU) up to which a 64-row tile takes eight waves (two halves of a 128-key trip)
+constexpr int kPfChunk = 64;                     // keys a wave multiplies per trip (a trip stages KH chunks)
 constexpr int kPfSeg = 512;                      // keys per segment: a multiple of this, chosen per launch
 constexpr int kPfSegMax = 16384;                 // at most (its page ids lie in LDS)
 constexpr long long kPfFill = 512;               // workgroups a launch should have before segments grow (two per CU)
@@ -80,8 +88,10 @@ __device__ __forceinline__ float quad_rows_max(float v) {
 
 // Two waves per SIMD at least: with that bound the compiler keeps the accumulators of the matrix
 // instructions in ordinary registers (no copies to and from the accumulation registers around the softmax).
-template <int HD, int RT>
-__global__ void __launch_bounds__(kPfThreads, 2)
+// At head_dim 64 the kernel fits three (two tiles a wave: 168 registers) or four (one tile); the bound
+// keeps it there, since one register more than 168 costs a third of the waves.
+template <int HD, int RT, int KH>
+__global__ void __launch_bounds__(kPfGroupThreads * KH, HD == 64 ? (RT == 1 ? 4 : 3) : 2)
     attention_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                              const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                              const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
@@ -90,8 +100,14 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   constexpr int kPfRT = RT, kPfWaveRows = 16 * RT, kPfRows = kPfWaveRows * kPfWaves;   // tiles per wave, rows per wave and workgroup
   constexpr int KSTEPS = HD / 32;                          // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;                              // 16-dim tiles of the output
-  constexpr int PIECES = kPfChunk * HD / 8 / kPfThreads;   // 16-byte pieces of a chunk per thread (keys; as many of values)
-  constexpr int KPITCH = HD + kPfPad, VPITCH = kPfChunk + kPfPad;
+  constexpr int kPfThreads = kPfGroupThreads * KH, TRIP = kPfChunk * KH;   // threads, and keys staged per trip
+  constexpr int PIECES = TRIP * HD / 8 / kPfThreads;       // 16-byte pieces of a trip per thread (keys; as many of values)
+  // LDS rows are unpadded; the 16-byte columns of a row are permuted instead: column c of row r lies at
+  // c ^ (r mod columns).  A wave's 16-byte reads (16 rows x 4 columns) then take the 8 cycles that 1 KiB
+  // costs at 128 bytes a cycle; with rows padded by 16 bytes they took 12 (measured: 12.9 against 8.8
+  // cycles per instruction and CU), and the counters showed 38 % of the LDS cycles as bank conflicts.
+  constexpr int KPITCH = HD, VPITCH = TRIP;
+  constexpr int KCOLS = HD / 8, VCOLS = TRIP / 8;   // 16-byte columns per row (the permutation uses the low three bits)
   // Workgroups are handed out in the order of blockIdx.x, round-robin over the chip's eight parts:
   // neighbours in that order are the heads of one (tile, segment), so that every part gets the
   // same mix of long and short walks.
@@ -105,7 +121,8 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   const int row0 = run_start[seq], n_rows = run_start[seq + 1] - row0;
   const int block_first = tile * kPfRows;
   if (block_first >= n_rows) return;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int wave = wave_id % kPfWaves, half = wave_id / kPfWaves;   // row group, and which chunk of a trip
   const int n16 = lane % 16, kq = lane / 16;
   const int pos0 = seq_start[seq];
   const int kvh = head / (nh / nkv);
@@ -125,13 +142,17 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   const float scale_log2 = scale * 1.4426950408889634f;   // scores are kept in units of log2: exp(x) = exp2(x log2 e)
   const int b_mask = B - 1;
 
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][kPfChunk][KPITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][HD][VPITCH];
-  // the sequence's page ids up to the workgroup's last position: the address of a piece is one
-  // LDS read away instead of one more trip to global memory
-  extern __shared__ int page_lds[];
-  const int page_lo = seg_first >> b_shift;
-  for (int i = threadIdx.x; i <= (block_last_pos >> b_shift) - page_lo; i += kPfThreads) page_lds[i] = table[page_lo + i];
+  // LDS: keys [2][TRIP][HD], values [2][HD][TRIP], then the sequence's page ids up to the workgroup's
+  // last position (the address of a piece is one LDS read away instead of one more trip to global memory)
+  extern __shared__ __attribute__((aligned(16))) unsigned char pf_lds[];
+  uint16_t (*k_lds)[TRIP][KPITCH] = reinterpret_cast<uint16_t (*)[TRIP][KPITCH]>(pf_lds);
+  uint16_t (*v_lds)[HD][VPITCH] = reinterpret_cast<uint16_t (*)[HD][VPITCH]>(pf_lds + sizeof(uint16_t) * 2 * TRIP * KPITCH);
+  int* page_lds = reinterpret_cast<int*>(pf_lds + sizeof(uint16_t) * 4 * TRIP * HD);
+  // Entries past the last page the workgroup may read repeat that page: a chunk's pieces beyond the
+  // last position then come from valid memory without a clamp per piece (the mask keeps them out).
+  const int page_lo = seg_first >> b_shift, page_hi = block_last_pos >> b_shift;
+  const int page_slots = (((block_last_pos | (TRIP - 1)) >> b_shift) - page_lo) + 1;   // through the last trip's end
+  for (int i = threadIdx.x; i < page_slots; i += kPfThreads) page_lds[i] = table[min(page_lo + i, page_hi)];
 
   // B operand of the scores: lane holds 8 dims of query row n16 of each tile (rows past the run
   // repeat its last row; they are never stored).  That row's position is what the lane may see.
@@ -166,53 +187,60 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   // A thread's key pieces are the same 8 dims of PIECES consecutive tokens (an aligned group, so one
   // page), its value pieces the same 8 tokens of dims 32 apart: one page lookup each per chunk, the
   // other pieces lie a constant away.
-  struct Pieces { u32x4 k[PIECES], v[PIECES]; int v_left; };   // v_left: how many of a value piece's 8 tokens lie inside what this workgroup may read
+  struct Pieces { u32x4 k[PIECES], v[PIECES]; };
   constexpr int KTPR = HD / 8;   // threads per key row
   const int k_p = threadIdx.x / KTPR, k_col = threadIdx.x % KTPR;
-  const int v_g = threadIdx.x % 8, v_d = threadIdx.x / 8;
-  const int last_chunk = block_last_pos & ~(kPfChunk - 1), last_kgroup = block_last_pos & ~(PIECES - 1),
-            last_vgroup = block_last_pos & ~7;
+  const int v_g = threadIdx.x % VCOLS, v_d = threadIdx.x / VCOLS;
+  const int last_chunk = block_last_pos & ~(TRIP - 1);   // the last trip's first key
+  const uint16_t* k_thread = kbase + k_col * 8;          // this thread's 8 dims of a key
+  const uint16_t* v_thread = vbase + size_t(v_d) * B;    // this thread's first dim row of a page's values
+  const int* pages = page_lds - page_lo;
   auto request = [&](int c0, Pieces& pc) {
     c0 = min(c0, last_chunk);   // past the last chunk: the last chunk again (no load behind a branch)
-    const int t0 = min(c0 + k_p * PIECES, last_kgroup);
-    const uint16_t* kp = kbase + size_t(page_lds[(t0 >> b_shift) - page_lo]) * page_elems + size_t(t0 & b_mask) * HD + k_col * 8;
+    const int tk = c0 + k_p * PIECES;
+    const uint16_t* kp = k_thread + size_t(pages[tk >> b_shift]) * page_elems + size_t(tk & b_mask) * HD;
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) pc.k[i] = *reinterpret_cast<const u32x4*>(kp + i * HD);
-    pc.v_left = block_last_pos + 1 - (c0 + v_g * 8);
-    const int tv = min(c0 + v_g * 8, last_vgroup);
-    const uint16_t* vp = vbase + size_t(page_lds[(tv >> b_shift) - page_lo]) * page_elems + size_t(v_d) * B + (tv & b_mask);
+    const int tv = c0 + v_g * 8;
+    const uint16_t* vp = v_thread + size_t(pages[tv >> b_shift]) * page_elems + (tv & b_mask);
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) pc.v[i] = *reinterpret_cast<const u32x4*>(vp + size_t(i) * 32 * B);
+    for (int i = 0; i < PIECES; ++i) pc.v[i] = *reinterpret_cast<const u32x4*>(vp + size_t(i) * (kPfThreads / VCOLS) * B);
   };
-  auto stage = [&](int buf, const Pieces& pc) {
+  // c0: the chunk the pieces belong to.  Only in the workgroup's last chunk can value slots lie past
+  // the last position; they hold stale data there, and probabilities of zero do not cancel a stale
+  // Inf or NaN, so they are cut out.
+  auto stage = [&](int buf, const Pieces& pc, int c0) {
+    const bool tail = c0 >= last_chunk;                                // the same for every thread: a jump, no selects
+    const int v_left = block_last_pos + 1 - (last_chunk + v_g * 8);    // n <= 0 keeps nothing, n >= 8 everything
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
-      *reinterpret_cast<u32x4*>(&k_lds[buf][k_p * PIECES + i][k_col * 8]) = pc.k[i];
+      *reinterpret_cast<u32x4*>(&k_lds[buf][k_p * PIECES + i][(k_col ^ ((k_p * PIECES + i) & (KCOLS - 1))) * 8]) = pc.k[i];
       // tokens 8 g .. 8 g + 7 of the chunk: inside their group of 32 tokens, token 16 a + 4 q + e goes to
       // place 8 q + 4 a + e, so that the 8 tokens a lane multiplies in one step lie together
       {
         const int r0 = (v_g * 8) % 32, grp = (v_g * 8) / 32;
         const int a = r0 / 16, q0 = (r0 % 16) / 4;
-        uint16_t* dst = &v_lds[buf][v_d + 32 * i][grp * 32 + 4 * a];
+        uint16_t* row = &v_lds[buf][v_d + (kPfThreads / VCOLS) * i][4 * a];
+        const int col = grp * 4 + q0, swz = v_d & 7;   // (v_d + rows-per-pass * i) mod 8
         uint4 piece{pc.v[i][0], pc.v[i][1], pc.v[i][2], pc.v[i][3]};
-        // slots past the last position hold stale data (or, from the clamped address, other tokens):
-        // probabilities there are zero, which does not cancel a stale Inf or NaN
-        if (pc.v_left < 8) piece = keep_first_bf16(piece, pc.v_left);
-        *reinterpret_cast<uint2*>(dst + 8 * q0) = uint2{piece.x, piece.y};
-        *reinterpret_cast<uint2*>(dst + 8 * (q0 + 1)) = uint2{piece.z, piece.w};
+        if (tail) piece = keep_first_bf16(piece, v_left);
+        *reinterpret_cast<uint2*>(row + 8 * (col ^ swz)) = uint2{piece.x, piece.y};
+        *reinterpret_cast<uint2*>(row + 8 * ((col + 1) ^ swz)) = uint2{piece.z, piece.w};
       }
     }
   };
 
-  auto compute = [&](int c0, int buf) {
-    if (wave_on && c0 <= wave_last_pos) {
+  auto compute = [&](int t0, int buf) {
+    const int c0 = t0 + half * kPfChunk;   // this wave's chunk of the trip
+    if (wave_on && c0 <= wave_last_pos && c0 <= block_last_pos) {
       // ---- S^T: s[rt][j][i] = k[token c0 + 16 j + 4 kq + i] . q[row n16 of tile rt]
       f32x4 s[kPfRT][4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         PFrag kf[KSTEPS];
 #pragma unroll
-        for (int c = 0; c < KSTEPS; ++c) kf[c].u = *reinterpret_cast<const uint4*>(&k_lds[buf][j * 16 + n16][c * 32 + kq * 8]);
+        for (int c = 0; c < KSTEPS; ++c)
+          kf[c].u = *reinterpret_cast<const uint4*>(&k_lds[buf][half * kPfChunk + j * 16 + n16][((c * 4 + kq) ^ (n16 & (KCOLS - 1))) * 8]);
 #pragma unroll
         for (int rt = 0; rt < kPfRT; ++rt) {
           s[rt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -286,7 +314,7 @@ __global__ void __launch_bounds__(kPfThreads, 2)
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
           PFrag vf;
-          vf.u = *reinterpret_cast<const uint4*>(&v_lds[buf][d * 16 + n16][c * 32 + 8 * kq]);
+          vf.u = *reinterpret_cast<const uint4*>(&v_lds[buf][d * 16 + n16][((half * 8 + c * 4 + kq) ^ (n16 & 7)) * 8]);
 #pragma unroll
           for (int rt = 0; rt < kPfRT; ++rt) o[rt][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][c].v, o[rt][d], 0, 0, 0);
         }
@@ -299,19 +327,57 @@ __global__ void __launch_bounds__(kPfThreads, 2)
   {
     Pieces pa, pb;
     request(seg_first, pa);
-    request(seg_first + kPfChunk, pb);
-    stage(0, pa);
+    request(seg_first + TRIP, pb);
+    stage(0, pa, seg_first);
     __syncthreads();
-    for (int c0 = seg_first; c0 <= block_last_pos; c0 += 2 * kPfChunk) {
-      request(c0 + 2 * kPfChunk, pa);
-      compute(c0, 0);
-      stage(1, pb);
+    for (int t0 = seg_first; t0 <= block_last_pos; t0 += 2 * TRIP) {
+      request(t0 + 2 * TRIP, pa);
+      compute(t0, 0);
+      stage(1, pb, t0 + TRIP);
       __syncthreads();
-      if (c0 + kPfChunk > block_last_pos) break;
-      request(c0 + 3 * kPfChunk, pb);
-      compute(c0 + kPfChunk, 1);
-      stage(0, pa);
+      if (t0 + TRIP > block_last_pos) break;
+      request(t0 + 3 * TRIP, pb);
+      compute(t0 + TRIP, 1);
+      stage(0, pa, t0 + 2 * TRIP);
       __syncthreads();
+    }
+  }
+
+  if constexpr (KH == 2) {
+    // The waves of the second half hand what their rows have gathered (output, maximum, sum) to the
+    // waves of the first half through LDS (every wave has passed the loop's last barrier: the staging
+    // buffers are free), lane to lane: both halves hold a row's numbers in the same lanes.
+    float* hand = reinterpret_cast<float*>(pf_lds);
+    constexpr int ITEMS = DT * 4 + 2;   // per tile of a wave
+    auto slot = [&](int rt, int item) { return hand + ((rt * ITEMS + item) * kPfWaves + wave) * kWave + lane; };
+    if (half == 1 && wave_on) {
+#pragma unroll
+      for (int rt = 0; rt < kPfRT; ++rt) {
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) *slot(rt, d * 4 + i) = o[rt][d][i];
+        *slot(rt, DT * 4) = m[rt];
+        *slot(rt, DT * 4 + 1) = l[rt][0];
+      }
+    }
+    __syncthreads();
+    if (half == 1) return;
+    if (wave_on) {
+#pragma unroll
+      for (int rt = 0; rt < kPfRT; ++rt) {
+        const float m1 = *slot(rt, DT * 4), l1 = *slot(rt, DT * 4 + 1);
+        const float m_all = fmaxf(m[rt], m1);
+        // a half that has seen no key (maximum -FLT_MAX, sum 0) gets weight 0
+        const float w0 = m[rt] > -0.5f * FLT_MAX ? __builtin_amdgcn_exp2f((m[rt] - m_all) * scale_log2) : 0.f;
+        const float w1 = m1 > -0.5f * FLT_MAX ? __builtin_amdgcn_exp2f((m1 - m_all) * scale_log2) : 0.f;
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[rt][d][i] = w0 * o[rt][d][i] + w1 * *slot(rt, d * 4 + i);
+        l[rt][0] = w0 * l[rt][0] + w1 * l1;
+        m[rt] = m_all;
+      }
     }
   }
 
@@ -393,15 +459,17 @@ int kvcm_attention_prefill_supported(int nh, int nkv, int hd, int B) {
 // chunks of 128-row workgroups).  Keys per segment: 512 while that gives the chip fewer than kPfFill
 // workgroups, longer (in multiples of 512) when tiles x heads x sequences already fill it, since
 // every segment beyond the first costs a partial result per row and head in scratch.
-struct PfPlan { int tile_rows, seg_len; };
+struct PfPlan { int tile_rows, seg_len, halves; };
 static PfPlan pf_plan(int T, int nh, int hd, int max_context, int max_run, int S) {
-  PfPlan p{64 * kPfMaxRT, kPfSeg};
+  PfPlan p{64 * kPfMaxRT, kPfSeg, 1};
   if (max_run <= 0 || S <= 0 || nh <= 0 || max_context <= 0) return p;
   if (T < max_run) T = max_run;
   const double seen = max_context - 0.5 * max_run > 64.0 ? max_context - 0.5 * max_run : 64.0;
   const double work = double(T) / 128.0 * (seen / kPfChunk) * nh;
   if (hd == 64 && work <= kPfSmallWork) p.tile_rows = 64;
+
   const long long base = static_cast<long long>((max_run + p.tile_rows - 1) / p.tile_rows) * nh * S;
+  if (hd == 64 && p.tile_rows == 64 && base <= kPfFewGroups) p.halves = 2;
   const long long want = (kPfFill + base - 1) / base;
   long long len = (max_context + want - 1) / want;
   len = (len + kPfSeg - 1) / kPfSeg * kPfSeg;
@@ -455,18 +523,29 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
   const long long units = static_cast<long long>((max_run + plan.tile_rows - 1) / plan.tile_rows) * max_segs * nh;
   KVCM_REQUIRE(units < (1ll << 31), "attention_prefill: too many workgroups");
   const dim3 grid(static_cast<unsigned>(units), S, 1);
-  const size_t page_bytes = sizeof(int) * size_t(seg_len / B + 2);   // the pages of one segment
   const uint16_t *qq = static_cast<const uint16_t*>(q), *kc = static_cast<const uint16_t*>(kcache),
                  *vc = static_cast<const uint16_t*>(vcache);
   const int merge_rows = 256 / (hd / 4);   // rows per workgroup of the merge
   const dim3 mgrid((max_run + merge_rows - 1) / merge_rows, S, nh);
-#define KVCM_PF(HD, RT)                                                                                                        \
-  attention_prefill_kernel<HD, RT><<<grid, kPfThreads, page_bytes, s>>>(qq, q_stride, static_cast<uint16_t*>(out), out_stride, \
-                                                                        kc, vc, tables, table_stride, run_start, seq_start,  \
-                                                                        nh, nkv, B, b_shift, scale, seg_len, max_segs, scratch)
-  if (hd == 64 && plan.tile_rows == 64) KVCM_PF(64, 1);
-  else if (hd == 64) KVCM_PF(64, 2);
-  else KVCM_PF(128, 2);
+  // LDS of a workgroup: two buffers of a trip's keys and values, and the page ids of one segment
+#define KVCM_PF(HD, RT, KH)                                                                                                  \
+  do {                                                                                                                       \
+    const size_t lds = size_t(8) * kPfChunk * KH * HD + sizeof(int) * size_t(seg_len / B + 2);                              \
+    static bool raised = false; /* a kernel may use more than 64 KiB of LDS once it has been told so */                    \
+    if (lds > 65536 && !raised) {                                                                                            \
+      KVCM_REQUIRE(hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HD, RT, KH>),                 \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess,               \
+                   "attention_prefill: the kernel may not use %zu bytes of LDS", lds);                                       \
+      raised = true;                                                                                                         \
+    }                                                                                                                        \
+    attention_prefill_kernel<HD, RT, KH><<<grid, kPfGroupThreads * KH, lds, s>>>(                                            \
+        qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc, tables, table_stride, run_start, seq_start, nh, nkv, \
+        B, b_shift, scale, seg_len, max_segs, scratch);                                                                      \
+  } while (0)
+  if (hd == 64 && plan.tile_rows == 64 && plan.halves == 2) KVCM_PF(64, 1, 2);
+  else if (hd == 64 && plan.tile_rows == 64) KVCM_PF(64, 1, 1);
+  else if (hd == 64) KVCM_PF(64, 2, 1);
+  else KVCM_PF(128, 2, 1);
 #undef KVCM_PF
   if (max_segs > 1) {
     if (hd == 64)
