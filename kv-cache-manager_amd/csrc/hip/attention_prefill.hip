@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(kPfGroupThreads * KH, HD == 64 ? (RT == 1 ? 4 
                              const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                              const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
                              const int* __restrict__ seq_start, int nh, int nkv, int B, int b_shift, float scale,
-                             int seg_len, int max_segs, float* __restrict__ scratch) {
+                             int seg_len, int max_segs, float* __restrict__ scratch, const float2* __restrict__ cos_sin) {
   constexpr int kPfRT = RT, kPfWaveRows = 16 * RT, kPfRows = kPfWaveRows * kPfWaves;   // tiles per wave, rows per wave and workgroup
   constexpr int KSTEPS = HD / 32;                          // matrix instructions per 16-token tile of scores
   constexpr int DT = HD / 16;                              // 16-dim tiles of the output
@@ -165,6 +165,27 @@ __global__ void __launch_bounds__(kPfGroupThreads * KH, HD == 64 ? (RT == 1 ? 4 
 #pragma unroll
     for (int c = 0; c < KSTEPS; ++c)
       qf[rt][c].u = *reinterpret_cast<const uint4*>(q + size_t(row0 + r) * q_stride + size_t(head) * HD + c * 32 + kq * 8);
+    if (cos_sin) {
+      // q as the projection left it: rotated here by pairs (j, j + HD / 2), which one lane holds in its
+      // fragments c and c + KSTEPS / 2, with the step's table of cos and sin ([row][HD / 2]), in 32-bit,
+      // rounded to bfloat16 as the rotation kernel stores it
+      const float2* tab = cos_sin + size_t(row0 + r) * (HD / 2) + kq * 8;
+#pragma unroll
+      for (int c = 0; c < KSTEPS / 2; ++c) {
+        uint32_t* lo = reinterpret_cast<uint32_t*>(&qf[rt][c].u);
+        uint32_t* hi = reinterpret_cast<uint32_t*>(&qf[rt][c + KSTEPS / 2].u);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const float4 t2 = *reinterpret_cast<const float4*>(tab + c * 32 + 2 * w);   // cos, sin of two dims
+          float a0 = bf16_bits_to_float(lo[w] & 0xFFFFu), a1 = bf16_bits_to_float(lo[w] >> 16);
+          float b0 = bf16_bits_to_float(hi[w] & 0xFFFFu), b1 = bf16_bits_to_float(hi[w] >> 16);
+          rotate_pair(a0, b0, t2.x, t2.y);
+          rotate_pair(a1, b1, t2.z, t2.w);
+          lo[w] = pack_bf16(a0, a1);
+          hi[w] = pack_bf16(b0, b1);
+        }
+      }
+    }
   }
   float m[kPfRT];
   f32x4 l[kPfRT];   // every element: the sum of the lane's query row (a product with a matrix of ones)
@@ -497,11 +518,12 @@ long long kvcm_attention_prefill_scratch(int T, int nh, int hd, int max_context,
 // run_start [S+1]: first row of each sequence's run of consecutive positions (rows of a run are
 // consecutive); seq_start [S]: position of a run's first row; tables [S][table_stride];
 // max_run: the longest run (it sizes the launch); T: rows in all (run_start[S]); max_context: an
-// upper bound of every row's context length (position + 1); scratch: see above.
+// upper bound of every row's context length (position + 1); scratch: see above; cos_sin: null when q is
+// rotated already, else the step's table [T][hd / 2][2] (cos, sin) that q is rotated with as it is read.
 int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                            const void* vcache, const int* tables, int table_stride, const int* run_start,
                            const int* seq_start, int S, int max_run, int T, int max_context, int nh, int nkv, int hd,
-                           int B, float scale, float* scratch, long long scratch_floats, hipStream_t s) {
+                           int B, float scale, float* scratch, long long scratch_floats, const float* cos_sin, hipStream_t s) {
   if (S == 0 || max_run == 0) return 0;
   KVCM_REQUIRE(kvcm_attention_prefill_supported(nh, nkv, hd, B),
                "attention_prefill: unsupported shape heads=%d kv_heads=%d head_dim=%d page=%d", nh, nkv, hd, B);
@@ -512,6 +534,7 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(kcache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(vcache) % 16 == 0, "attention_prefill: operands must be 16-byte aligned");
   KVCM_REQUIRE(out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0, "attention_prefill: output must be 8-byte aligned");
+  KVCM_REQUIRE(reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0, "attention_prefill: the table of cos and sin must be 16-byte aligned");
   const PfPlan plan = pf_plan(T, nh, hd, max_context, max_run, S);
   const int seg_len = plan.seg_len;
   const int max_segs = (max_context + seg_len - 1) / seg_len;
@@ -540,7 +563,7 @@ int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_strid
     }                                                                                                                        \
     attention_prefill_kernel<HD, RT, KH><<<grid, kPfGroupThreads * KH, lds, s>>>(                                            \
         qq, q_stride, static_cast<uint16_t*>(out), out_stride, kc, vc, tables, table_stride, run_start, seq_start, nh, nkv, \
-        B, b_shift, scale, seg_len, max_segs, scratch);                                                                      \
+        B, b_shift, scale, seg_len, max_segs, scratch, reinterpret_cast<const float2*>(cos_sin));                            \
   } while (0)
   if (hd == 64 && plan.tile_rows == 64 && plan.halves == 2) KVCM_PF(64, 1, 2);
   else if (hd == 64 && plan.tile_rows == 64) KVCM_PF(64, 1, 1);

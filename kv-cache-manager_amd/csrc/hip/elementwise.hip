@@ -215,9 +215,11 @@ template <class T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, const int* __restrict__ slots,
                                   T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int hd, int B,
-                                  const float* __restrict__ partials, int S, const float2* __restrict__ cos_sin) {
-  // one workgroup per (row, head): q heads, then k heads, then v heads
-  const int t = blockIdx.x, h = blockIdx.y;
+                                  const float* __restrict__ partials, int S, const float2* __restrict__ cos_sin,
+                                  int first_head) {
+  // one workgroup per (row, head): q heads, then k heads, then v heads (from first_head on: the
+  // q heads are left alone when the attention kernel rotates them as it reads them)
+  const int t = blockIdx.x, h = blockIdx.y + first_head;
   T* row = qkv + size_t(t) * row_stride;
   const int half = hd / 2;
   const int width = (nh + 2 * nkv) * hd;
@@ -327,15 +329,15 @@ __global__ void __launch_bounds__(256)
     rope_cache_vec_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                           const float* __restrict__ inv_freq, const int* __restrict__ slots, T* __restrict__ kcache,
                           T* __restrict__ vcache, int nh, int nkv, int hd, int B, const float2* __restrict__ cos_sin,
-                          int rows, long long qk_items, long long items) {
+                          int rows, long long qk_items, long long items, int first_head) {
   const long long item = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x;
   if (item >= items) return;
   if (item >= qk_items) {
     v_page_item<T>(qkv, row_stride, slots, vcache, nh, nkv, hd, B, rows, item - qk_items);
     return;
   }
-  const int cph = hd / 16, heads = nh + nkv, half = hd / 2;
-  const int c = int(item % cph), h = int((item / cph) % heads), t = int(item / (static_cast<long long>(cph) * heads));
+  const int cph = hd / 16, heads = nh + nkv - first_head, half = hd / 2;   // first_head = nh: the k heads only
+  const int c = int(item % cph), h = first_head + int((item / cph) % heads), t = int(item / (static_cast<long long>(cph) * heads));
   T* row = qkv + size_t(t) * row_stride + size_t(h) * hd;
   const int slot = slots ? slots[t] : -1;
   const size_t page = slot >= 0 ? slot / B : 0;
@@ -480,9 +482,12 @@ int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const float* partials
 
 int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, const float* inv_freq,
                     const int* slots, void* kcache, void* vcache, int T, int nh, int nkv, int hd, int B,
-                    const float* partials, int S, const float* cos_sin, hipStream_t s) {
+                    const float* partials, int S, const float* cos_sin, int skip_q, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(hd > 0 && hd % 2 == 0, "rope: head_dim %d must be even", hd);
+  KVCM_REQUIRE(!skip_q || !partials, "rope: the q heads of un-added partial sums cannot be left alone");
+  const int first_head = skip_q ? nh : 0;
+  if (nh + 2 * nkv - first_head == 0) return 0;
   KVCM_REQUIRE(nh >= 0 && nkv >= 0 && row_stride >= (nh + 2 * nkv) * hd, "rope: row stride %d too small", row_stride);
   KVCM_REQUIRE(!slots || (kcache && vcache && B > 0), "rope: cache write without a cache");
   KVCM_REQUIRE(!inv_freq || positions || cos_sin, "rope: rotation without positions");
@@ -495,7 +500,7 @@ int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, 
     // q and k heads: 8 pairs per item; v heads (only when there is a cache to store them to): one
     // dim of 8 rows per item, one group more than the rows fill because groups start at a slot
     // that is a multiple of 8
-    const long long qk_items = static_cast<long long>(T) * (nh + nkv) * (hd / 16);
+    const long long qk_items = static_cast<long long>(T) * (nh + nkv - first_head) * (hd / 16);
     const long long v_items = slots ? static_cast<long long>((T + kVGroup - 1) / kVGroup + 1) * nkv * hd : 0;
     const long long items = qk_items + v_items;
     const long long blocks = (items + 255) / 256;
@@ -504,24 +509,24 @@ int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, 
     if (dtype == kF32)
       rope_cache_vec_kernel<float><<<static_cast<unsigned>(blocks), 256, 0, s>>>(
           static_cast<float*>(qkv), row_stride, positions, inv_freq, slots, static_cast<float*>(kcache),
-          static_cast<float*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), T, qk_items, items);
+          static_cast<float*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), T, qk_items, items, first_head);
     else if (dtype == kBF16)
       rope_cache_vec_kernel<bf16_t><<<static_cast<unsigned>(blocks), 256, 0, s>>>(
           static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots, static_cast<bf16_t*>(kcache),
-          static_cast<bf16_t*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), T, qk_items, items);
+          static_cast<bf16_t*>(vcache), nh, nkv, hd, B, reinterpret_cast<const float2*>(cos_sin), T, qk_items, items, first_head);
     else KVCM_REQUIRE(false, "rope: unknown dtype %d", dtype);
     return launch_status("rope_cache");
   }
-  const dim3 grid(T, nh + 2 * nkv);
+  const dim3 grid(T, nh + 2 * nkv - first_head);
   const int threads = 64;
   if (dtype == kF32)
     rope_cache_kernel<float><<<grid, threads, 0, s>>>(static_cast<float*>(qkv), row_stride, positions, inv_freq, slots,
                                                   static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, hd, B,
-                                                  partials, S, reinterpret_cast<const float2*>(cos_sin));
+                                                  partials, S, reinterpret_cast<const float2*>(cos_sin), first_head);
   else if (dtype == kBF16)
     rope_cache_kernel<bf16_t><<<grid, threads, 0, s>>>(static_cast<bf16_t*>(qkv), row_stride, positions, inv_freq, slots,
                                                    static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, hd, B,
-                                                   partials, S, reinterpret_cast<const float2*>(cos_sin));
+                                                   partials, S, reinterpret_cast<const float2*>(cos_sin), first_head);
   else KVCM_REQUIRE(false, "rope: unknown dtype %d", dtype);
   return launch_status("rope_cache");
 }

@@ -52,7 +52,7 @@ int kvcm_rmsnorm(float* x, const void* add, int add_dtype, const float* partials
                  hipStream_t s);
 int kvcm_rope_cache(void* qkv, int dtype, int row_stride, const int* positions, const float* inv_freq, const int* slots,
                     void* kcache, void* vcache, int T, int nh, int nkv, int hd, int B, const float* partials, int S,
-                    const float* cos_sin, hipStream_t s);
+                    const float* cos_sin, int skip_q, hipStream_t s);
 int kvcm_rope_table(const int* positions, const float* inv_freq, float* cos_sin, int T, int half, hipStream_t s);
 int kvcm_swiglu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t s);
 int kvcm_add_residual(float* x, const void* y, int dtype, long long n, hipStream_t s);
@@ -105,7 +105,7 @@ int kvcm_attention_decode_fused(const float* partials, int S, const void* qkv, i
 int kvcm_attention_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kcache, const void* vcache,
                            const int* tables, int table_stride, const int* run_start, const int* seq_start, int S,
                            int max_run, int T, int max_context, int nh, int nkv, int hd, int B, float scale,
-                           float* scratch, long long scratch_floats, hipStream_t s);
+                           float* scratch, long long scratch_floats, const float* cos_sin, hipStream_t s);
 
 // ---- sampling ---------------------------------------------------------------------------------
 int kvcm_sample(const float* logits, int ld, const float* temperature, const uint64_t* seeds, const long long* request_ids,

@@ -32,7 +32,7 @@ def _declare(lib):
     lib.kvcm_hip_last_error.restype = C.c_char_p
     fn("kvcm_embed", vp, vp, i, vp, i, i, i, vp)
     fn("kvcm_rmsnorm", vp, vp, i, vp, i, i, vp, vp, i, vp, i, i, i, f, i, vp)
-    fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp, vp)
+    fn("kvcm_rope_cache", vp, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp, i, vp, i, vp)
     fn("kvcm_rope_table", vp, vp, vp, i, i, vp)
     fn("kvcm_attention_decode_info", i, i, i, vp)
     fn("kvcm_attention_decode_fused_supported", i, i, i, i)
@@ -55,7 +55,7 @@ def _declare(lib):
     fn("kvcm_sample", vp, i, vp, vp, vp, vp, vp, i, i, vp)
     fn("kvcm_attention_decode_supported", i, i, i, i)
     fn("kvcm_attention_prefill_supported", i, i, i, i)
-    fn("kvcm_attention_prefill", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, i, i, i, f, vp, C.c_longlong, vp)
+    fn("kvcm_attention_prefill", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, i, i, i, f, vp, C.c_longlong, vp, vp)
     lib.kvcm_attention_prefill_scratch.restype = C.c_longlong
     lib.kvcm_attention_prefill_scratch.argtypes = [i, i, i, i, i, i]
     lib.kvcm_attention_prefill_segment.restype = i
@@ -371,12 +371,13 @@ def rope_table(positions, inv_freq, out, rows=None):
 
 
 def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcache=None, vcache=None,
-               block_size=0, rows=None, source=None, cos_sin=None):
+               block_size=0, rows=None, source=None, cos_sin=None, skip_q=False):
     """Rotates the q and k heads of the fused rows in place (by the angles position * inv_freq, or
     by a table ``cos_sin`` [rows, hd/2, 2] computed beforehand; neither: no rotation) and copies k
     (rotated) and v to the paged cache (slots given).  Keys [pages, nkv, block_size, hd], values
     [pages, nkv, hd, block_size].  With ``source`` (PartialSums of the projection) the rows are read
-    from there; q lands in ``qkv``."""
+    from there; q lands in ``qkv``.  ``skip_q``: the q heads are left as they are (``attention_prefill``
+    rotates them as it reads them when it is given the same table)."""
     _dev(qkv, positions, inv_freq, slots, kcache, vcache)
     _rows2d(qkv, "qkv")
     T = qkv.shape[0] if rows is None else rows
@@ -402,7 +403,7 @@ def rope_cache(qkv, nh, nkv, hd, positions=None, inv_freq=None, slots=None, kcac
     _call("kvcm_rope_cache", _ptr(qkv), _DT[qkv.dtype], qkv.stride(0), _ptr(positions), _ptr(inv_freq),
                                  _ptr(slots), _ptr(kcache), _ptr(vcache), T, nh, nkv, hd, block_size,
                                  _ptr(source.data) if source is not None else 0,
-                                 source.splits if source is not None else 0, _ptr(cos_sin), _stream())
+                                 source.splits if source is not None else 0, _ptr(cos_sin), 1 if skip_q else 0, _stream())
 
 
 def swiglu(gate_up, out):
@@ -708,10 +709,12 @@ def attention_prefill_tile_rows(rows, nh, hd, max_context, max_run, num_seqs):
 
 
 def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, seq_start, num_seqs, max_run, nh, nkv, hd,
-                      scale, rows=None, max_context=None, scratch=None):
+                      scale, rows=None, max_context=None, scratch=None, cos_sin=None):
     """Causal attention for runs of consecutive positions (bfloat16): sequence s owns rows
     run_start[s] .. run_start[s+1]-1, the first of them at position seq_start[s]; every row sees the
     sequence's cached tokens up to its own position.  The same result as ``attention``.
+    ``cos_sin`` (float32 [rows, hd/2, 2]): q is not rotated yet; the kernel rotates it with this table
+    as it reads it (the keys in the cache are rotated already).
     ``rows``: rows in all; ``max_context``: a bound of every row's context length (default: what the
     block tables can hold); contexts beyond one segment of keys need ``scratch`` (float32,
     attention_prefill_scratch elements; allocated here when not given)."""
@@ -732,10 +735,13 @@ def attention_prefill(q, out, kcache, vcache, tables, table_stride, run_start, s
     _i32(run_start, "run_start", num_seqs + 1)
     _i32(seq_start, "seq_start", num_seqs)
     _i32(tables, "tables", num_seqs * table_stride)
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.numel() >= T * hd
+              and cos_sin.is_cuda, "cos_sin must be float32 [rows, head_dim/2, 2]")
     _call("kvcm_attention_prefill", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
                                         _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), num_seqs, max_run,
                                         T, int(max_context), nh, nkv, hd, kcache.shape[2], float(scale), _ptr(scratch),
-                                        scratch.numel() if scratch is not None else 0, _stream())
+                                        scratch.numel() if scratch is not None else 0, _ptr(cos_sin), _stream())
 
 
 # ------------------------------------------------------------------------- probes of the machine

@@ -30,10 +30,11 @@ def _decode_parts_scratch(step, ops, rows, nh, nkv, hd, bound):
 
 
 def attend_from_projection(step, ops, projection, out, kcache, vcache, g, nh, nkv, hd, scale, window, cos_sin, slots):
-    """Decode-shaped steps: one launch (and a small merge when few rows have long contexts).  Mixed
-    steps whose first sequences run one token each (the scheduler puts decoding requests first):
-    those rows take that launch too, the rows after them are rotated and stored, then attended by
-    the tiled kernel; a single-token run there would otherwise cost a whole tile of its own.
+    """Decode-shaped steps: one launch (and a small merge when few rows have long contexts).  Steps
+    with runs of positions: the keys of those rows are rotated and stored with their values, the tiled
+    kernel rotates their queries as it reads them; where the first sequences of such a step run one
+    token each (the scheduler puts decoding requests first) those rows take the decode launch: a
+    single-token run would otherwise cost a whole tile of its own.
     Returns False when this step or shape has no such kernel (then the caller rotates, stores and
     calls ``attend``: the same values up to rounding)."""
     if (step.attention_mode != "auto" or window != 0 or out.dtype != torch.bfloat16
@@ -48,27 +49,29 @@ def attend_from_projection(step, ops, projection, out, kcache, vcache, g, nh, nk
                                    max_context=bound, scratch=_decode_parts_scratch(step, ops, step.rows, nh, nkv, hd, bound))
         return True
     D, T, S = step.leading_single_runs(), step.real_rows, step.real_seqs
-    if (D == 0 or D > DECODE_ATTENTION_MAX_ROWS
-            or not ops.attention_prefill_supported(nh, nkv, hd, out.dtype, kcache.shape[2])):
+    if D > DECODE_ATTENTION_MAX_ROWS or not ops.attention_prefill_supported(nh, nkv, hd, out.dtype, kcache.shape[2]):
         return False
     if isinstance(projection, ops.PartialSums):
-        # three consumers here (decode rows, rotation of the others, tiled attention): add the
+        # several consumers here (decode rows, rotation of the others, tiled attention): add the
         # split sums up once instead of handing every single-token run to the tiled kernel
         projection = projection.materialize()
     stride = step.table_stride(g)
     bound = step.max_context_bound
-    ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), stride, step.row_seq, step.ctx_lens,
-                               nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=D, max_context=bound,
-                               scratch=_decode_parts_scratch(step, ops, D, nh, nkv, hd, bound))
+    if D > 0:
+        ops.attention_decode_fused(projection, out, kcache, vcache, step.tables(g), stride, step.row_seq, step.ctx_lens,
+                                   nh, nkv, hd, scale, cos_sin=cos_sin, slots=slots, rows=D, max_context=bound,
+                                   scratch=_decode_parts_scratch(step, ops, D, nh, nkv, hd, bound))
+    # the other rows: their keys are rotated and stored with their values; their queries stay as the
+    # projection left them and the tiled kernel rotates them as it reads them (one pass over q less)
     if (cos_sin is not None or slots is not None) and T > D:
         ops.rope_cache(projection[D:T], nh, nkv, hd, cos_sin=cos_sin[D:T] if cos_sin is not None else None,
                        slots=slots[D:T] if slots is not None else None, kcache=kcache, vcache=vcache,
-                       block_size=kcache.shape[2], rows=T - D)
+                       block_size=kcache.shape[2], rows=T - D, skip_q=True)
     need = ops.attention_prefill_scratch(T, nh, hd, bound, step.max_run, S - D)
     scratch = step.flat("prefill_partials", need) if need else None
     ops.attention_prefill(projection, out, kcache, vcache, step.tables(g)[D * stride:], stride, step.run_start[D:],
                           step.seq_start[D:], S - D, step.max_run, nh, nkv, hd, scale, rows=T,
-                          max_context=bound, scratch=scratch)
+                          max_context=bound, scratch=scratch, cos_sin=cos_sin)
     return True
 
 

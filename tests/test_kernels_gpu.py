@@ -972,6 +972,45 @@ def test_prefill_attention_runs_anywhere(ops, nh, nkv, hd, B):
     np.testing.assert_allclose(got, generic, atol=2e-2, rtol=0)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,B", [(8, 2, 64, 16), (4, 4, 128, 8), (32, 4, 64, 32)])
+def test_prefill_attention_rotates_unrotated_queries_itself(ops, nh, nkv, hd, B):
+    """Given the step's table of cos and sin, the tiled kernel rotates q as it reads it: bit for bit what
+    it computes from queries that the rotation kernel rotated (the same pairs, the same 32-bit
+    multiply-adds, the same rounding to bfloat16; that kernel has its own test against the plain rotation)."""
+    rng = np.random.default_rng(nh * hd + B)
+    runs = [(0, 130), (77, 2), (15, 64), (63, 65), (300, 1)]
+    P = _runs_problem(rng, runs, nh, nkv, hd, B)
+    R, half = P["R"], hd // 2
+    pos = np.concatenate([np.arange(s, s + n) for s, n in runs]).astype(np.int32)
+    inv_freq = (1.0 / (10000.0 ** (np.arange(half, dtype=np.float64) * 2 / hd))).astype(np.float32)
+    table = torch.empty(R, half, 2, dtype=torch.float32, device=DEV)
+    ops.rope_table(_t(pos, torch.int32), _t(inv_freq, torch.float32), table)
+    q_plain = _t(P["Q"].reshape(R, nh * hd), torch.bfloat16)
+    q_rot = q_plain.clone()
+    ops.rope_cache(q_rot, nh, 0, hd, cos_sin=table)                      # q heads only, no cache
+    run_start = _t(np.concatenate([[0], np.cumsum([n for _, n in runs])]).astype(np.int32), torch.int32)
+    args = (_t(P["Kc"], torch.bfloat16), _vt(P["Vc"], torch.bfloat16), _t(P["tables"], torch.int32), P["max_blocks"], run_start,
+            _t([s for s, _ in runs], torch.int32), len(runs), max(n for _, n in runs), nh, nkv, hd, 1.0 / math.sqrt(hd))
+    a = torch.full((R, nh * hd), 3.0, dtype=torch.bfloat16, device=DEV)
+    b = torch.full((R, nh * hd), 5.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(q_rot, a, *args)
+    ops.attention_prefill(q_plain, b, *args, cos_sin=table)
+    assert torch.equal(a, b)
+    # and the rotation itself moved something: unrotated queries give another result
+    c = torch.full((R, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(q_plain, c, *args)
+    assert not torch.equal(a, c)
+    # the k heads alone: skip_q leaves q as it was and still rotates and stores the keys
+    fused = torch.zeros(R, (nh + 2 * nkv) * hd, dtype=torch.bfloat16, device=DEV)
+    fused[:, :nh * hd] = q_plain
+    fused[:, nh * hd:] = torch.randn(R, 2 * nkv * hd, device=DEV).to(torch.bfloat16)
+    both, only_k = fused.clone(), fused.clone()
+    ops.rope_cache(both, nh, nkv, hd, cos_sin=table)
+    ops.rope_cache(only_k, nh, nkv, hd, cos_sin=table, skip_q=True)
+    assert torch.equal(only_k[:, :nh * hd], fused[:, :nh * hd])
+    assert torch.equal(only_k[:, nh * hd:], both[:, nh * hd:])
+
+
 def test_prefill_attention_is_causal_at_tile_and_page_edges(ops):
     """A huge key at position t must be seen by rows t, t+1, .. and by no row before it."""
     rng = np.random.default_rng(50)
