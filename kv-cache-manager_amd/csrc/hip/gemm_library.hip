@@ -195,8 +195,9 @@ int kvcm_gemm_library_tune(const void* X, const void* W, int w_copies, long long
   };
   struct Timed { float us; hipblasLtMatmulAlgo_t algo; size_t need; };
   std::vector<Timed> timed;
-  // the reference result and the first choice's time
+  // the reference result and the first choice's time (after enough calls for the clock to have settled)
   hipblasLtMatmulAlgo_t first = plan->choices[0].algo;
+  time_of(first, plan->choices[0].workspaceSize, 48);
   const float first_us = time_of(first, plan->choices[0].workspaceSize, 8);
   int rc = 0;
   unsigned* flags = reinterpret_cast<unsigned*>(static_cast<uint16_t*>(check) + size_t(M) * N);
@@ -237,13 +238,17 @@ int kvcm_gemm_library_tune(const void* X, const void* W, int w_copies, long long
       while (at < timed.size() && memcmp(&timed[at].algo, &first, sizeof(first)) != 0) ++at;
       if (at >= finalists && at < timed.size()) std::swap(timed[finalists - 1], timed[at]);
     }
-    std::vector<float> best(finalists, 1e30f);
-    for (int round = 0; round < 3; ++round)
+    // (each finalist's time: the median of five rounds, which a single slow or fast round does not move)
+    std::vector<std::vector<float>> rounds(finalists);
+    for (int round = 0; round < 5; ++round)
       for (size_t i = 0; i < finalists; ++i) {
         const float us = time_of(timed[i].algo, timed[i].need, 16);
-        best[i] = us > 0.f ? std::min(best[i], us) : 1e30f;
+        rounds[i].push_back(us > 0.f ? us : 1e30f);
       }
-    for (size_t i = 0; i < finalists; ++i) timed[i].us = best[i];
+    for (size_t i = 0; i < finalists; ++i) {
+      std::sort(rounds[i].begin(), rounds[i].end());
+      timed[i].us = rounds[i][2];
+    }
     std::sort(timed.begin(), timed.begin() + finalists, [](const Timed& x, const Timed& y) { return x.us < y.us; });
     bool kept = false;
     for (size_t i = 0; i < finalists && !kept && timed[i].us < 1e29f; ++i) {
