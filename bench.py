@@ -139,8 +139,9 @@ def main():
     ap.add_argument("--sizes", default="tinyllama-1.1b", help="layer sizes by name (tinyllama-1.1b, llama-2-7b, llama-3-8b)")
     ap.add_argument("--tune-products", default="heuristic", choices=["off", "heuristic", "all"],
                     help="which of the vendor library's algorithms the many-row products of prompt steps run: its first "
-                         "choice, the fastest of its choices (the engine's default), or the fastest of all; timed at a "
-                         "shape's first use, before anything is measured")
+                         "choice (the engine's default), the fastest of its choices, or the fastest of all; timed at a "
+                         "shape's first use, before anything is measured (tens of milliseconds per shape: worth it "
+                         "for shapes that run thousands of times, as a benchmark's do)")
     ap.add_argument("--context-limit", type=int, default=2048, help="most tokens a request may hold; sizes the cache pool")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true",
@@ -230,6 +231,10 @@ def main():
         # beside the published peaks the fractions above are taken against: what this GPU reached in this run
         out["measured"] = measured_peaks()
     print(json.dumps(out), flush=True)
+    if os.environ.get("KVCM_BENCH_TUNING_LOG"):       # which shapes were tuned, the first choice's and the kept algorithm's microseconds
+        from kvcm_amd import ops
+        for row in ops.library_tuning_log:
+            print("tuned M=%d N=%d K=%d: %.1f -> %.1f us (%d candidates)" % row, file=sys.stderr)
 
 
 if __name__ == "__main__":

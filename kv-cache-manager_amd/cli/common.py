@@ -35,7 +35,7 @@ def engine_config_from_args(a, **overrides) -> EngineConfig:
         max_batched_tokens=a.i32("max-batched-tokens", 4096), attn=a.str("attn", "auto"),
         dtype=a.str("dtype", "bfloat16"), prefill_chunk=a.i32("prefill-chunk", 0), eos_id=a.i32("eos-id", -1),
         use_graphs=not a.flag("no-graphs"), use_programs=not a.flag("no-programs"),
-        tune_products=a.str("tune-products", "heuristic"))
+        tune_products=a.str("tune-products", "off"))
     for k, v in overrides.items():
         setattr(ec, k, v)
     return ec.validate()

@@ -197,7 +197,7 @@ int kvcm_gemm_library_tune(const void* X, const void* W, int w_copies, long long
   std::vector<Timed> timed;
   // the reference result and the first choice's time (after enough calls for the clock to have settled)
   hipblasLtMatmulAlgo_t first = plan->choices[0].algo;
-  time_of(first, plan->choices[0].workspaceSize, 48);
+  time_of(first, plan->choices[0].workspaceSize, 32);
   const float first_us = time_of(first, plan->choices[0].workspaceSize, 8);
   int rc = 0;
   unsigned* flags = reinterpret_cast<unsigned*>(static_cast<uint16_t*>(check) + size_t(M) * N);

@@ -433,10 +433,13 @@ LIBRARY_GEMM_MIN_ROWS = 96
 
 # Which of the library's algorithms a shape runs.  "off": the first choice of the library's heuristic.
 # "heuristic": at a shape's first use the heuristic's choices (up to 16) are timed on the call's own
-# operands and the fastest is kept (a few milliseconds per shape).  "all": every algorithm of the library
-# that supports the shape is timed (1 to 4 seconds per shape, at most LIBRARY_TUNING_SECONDS): for
-# long-running servers and measurements, switched on by the engine's configuration.
-LIBRARY_TUNING = "heuristic"
+# operands and the fastest is kept: some 400 launches of the product, 20 to 40 milliseconds per shape, for
+# about 5 % of its time afterwards, which pays after thousands of calls of that shape.  "all": every
+# algorithm of the library that supports the shape is timed (seconds per shape, at most
+# LIBRARY_TUNING_SECONDS).  Off unless the engine's configuration asks for it: a serving run meets a few
+# hundred shapes (rows in steps of 64, four products) and most of them only a few times; measured on a
+# burst of 400 requests, tuning each at its first use took longer than the whole run without it.
+LIBRARY_TUNING = "off"
 LIBRARY_TUNING_SECONDS = 6.0
 LIBRARY_TUNING_BYTES = 512 << 20
 _TUNING_MODES = {"off": 0, "heuristic": 1, "all": 2}
