@@ -151,6 +151,12 @@ def main():
         print("bench.py: this engine runs on one GPU; --gpus N with N > 1 is not supported")
         sys.exit(2)
 
+    limit = args.context_limit
+    budget = max(4096, args.prompt_len + args.batch)     # a whole prompt fits a step beside the decoding requests
+    if args.prompt_len + args.warmup + args.steps + 24 + prompt_step_count(args.batch, args.prompt_len, budget) > limit:
+        print("bench.py: --prompt-len %d plus the decoded tokens does not fit --context-limit %d" % (args.prompt_len, limit))
+        sys.exit(2)
+
     import torch
     from kvcm_amd.config.model_config import LlamaConfig
     from kvcm_amd.weights.random_init import random_tensors
@@ -180,11 +186,6 @@ def main():
         return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_GBS, 4)}
 
-    limit = args.context_limit
-    budget = max(4096, args.prompt_len + args.batch)     # a whole prompt fits a step beside the decoding requests
-    if args.prompt_len + args.warmup + args.steps + 24 + prompt_step_count(args.batch, args.prompt_len, budget) > limit:
-        print("bench.py: --prompt-len %d plus the decoded tokens does not fit --context-limit %d" % (args.prompt_len, limit))
-        sys.exit(2)
     # the pool holds every request of the largest batch at the context limit
     seqs = args.batch if (args.no_points or args.only_prefill) else max(64, args.batch)
     eng = build_engine(cfg, args.dtype, max_num_seqs=seqs, max_batched_tokens=budget, tensors=tensors, context_limit=limit,
