@@ -1105,7 +1105,7 @@ def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops, B):
         np.testing.assert_allclose(got[r], ref, atol=1e-2, rtol=0, err_msg=f"row {r}")
 
 
-# ------------------------------------- products of at most 8 rows with the norm folded in
+# ------------------------------------- products of at most 16 rows with the norm folded in
 def _folded_reference(a, wo, x, g, eps, w2):
     """What the producer and the consumer compute, in float64 with the same rounding points:
     x += round(a wo^T); xg = round(g round(x)); y = round((xg w2^T) rsqrt(mean x^2 + eps))."""
@@ -1115,13 +1115,14 @@ def _folded_reference(a, wo, x, g, eps, w2):
     return x_new, xg, (xg @ w2.T) * rstd
 
 
-@pytest.mark.parametrize("M", [1, 3, 8])
-@pytest.mark.parametrize("H,K,N2", [(2048, 2048, 2560), (2048, 5632, 512), (128, 64, 40), (320, 192, 24), (2048, 2112, 4128)])
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16])
+@pytest.mark.parametrize("H,K,N2", [(2048, 2048, 2560), (2048, 5632, 512), (128, 64, 48), (320, 192, 32), (2048, 2112, 4128)])
 def test_products_with_the_norm_folded_in(ops, M, H, K, N2):
     """Producer (residual add + the norm's preparation in the epilogue) and consumer (the norm's scale on
     the finished sums) against the same arithmetic in float64, and against the reference's own form of
     the norm, whose two roundings fall at other places (kernels.cu:34-49): equal up to bfloat16 rounding.
-    Widths that are no power of two, K slices of unequal length, fewer rows than a tile holds."""
+    Widths that are no power of two, K slices of unequal length, fewer rows than a tile holds; up to 8
+    rows and 9 to 16 rows are two kernels that leave and read the same sums of squares."""
     rng = np.random.default_rng(M * 13 + H + K)
     a = _bf16_grid(rng.normal(size=(M, K)))
     wo = _bf16_grid(rng.normal(size=(H, K)) * 0.05)
@@ -1133,8 +1134,8 @@ def test_products_with_the_norm_folded_in(ops, M, H, K, N2):
 
     at, wot, w2t = _t(a, torch.bfloat16), _t(wo, torch.bfloat16), _t(w2, torch.bfloat16)
     xt = _t(x, torch.float32)
-    xg = torch.full((8, H), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ss = torch.full((8, H // 8), float("nan"), dtype=torch.float32, device=DEV)
+    xg = torch.full((16, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ss = torch.full((16, H // 8), float("nan"), dtype=torch.float32, device=DEV)
     normed_buf = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
     product = ops.PendingProduct(at, wot, torch.zeros(M, H, dtype=torch.bfloat16, device=DEV))
     assert ops.gemm8_supported(M, H, K) and ops.gemm8_supported(M, N2, H)
@@ -1158,8 +1159,8 @@ def test_products_with_the_norm_folded_in(ops, M, H, K, N2):
     np.testing.assert_allclose(_np(h.materialize()), plain.rms_norm(got_x, g, eps, plain.round_bf16), rtol=2 ** -7, atol=1e-3)
 
 
-@pytest.mark.parametrize("M", [1, 5, 8])
-@pytest.mark.parametrize("H,I", [(2048, 5632), (192, 136), (64, 8)])
+@pytest.mark.parametrize("M", [1, 5, 8, 11, 16])
+@pytest.mark.parametrize("H,I", [(2048, 5632), (192, 144), (64, 16)])
 def test_gate_up_product_with_the_norm_folded_in_applies_swiglu(ops, M, H, I):
     rng = np.random.default_rng(M + H + I)
     x = (rng.normal(size=(M, H)) * 2).astype(np.float32).astype(np.float64)
@@ -1168,8 +1169,8 @@ def test_gate_up_product_with_the_norm_folded_in_applies_swiglu(ops, M, H, I):
     eps = 1e-6
     # a producer with a zero product leaves x as it is and prepares the norm
     xt = _t(x, torch.float32)
-    xg = torch.zeros(8, H, dtype=torch.bfloat16, device=DEV)
-    ss = torch.zeros(8, H // 8, dtype=torch.float32, device=DEV)
+    xg = torch.zeros(16, H, dtype=torch.bfloat16, device=DEV)
+    ss = torch.zeros(16, H // 8, dtype=torch.float32, device=DEV)
     zero = ops.PendingProduct(torch.zeros(M, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(H, 64, dtype=torch.bfloat16, device=DEV),
                               torch.zeros(M, H, dtype=torch.bfloat16, device=DEV))
     h = ops.gemm_residual_norm(zero, xt, _t(g, torch.bfloat16), eps, xg, ss, torch.zeros(M, H, dtype=torch.bfloat16, device=DEV))
@@ -1190,12 +1191,12 @@ def test_gate_up_product_with_the_norm_folded_in_applies_swiglu(ops, M, H, I):
     np.testing.assert_allclose(got, ref, rtol=0, atol=2e-2 * max(np.abs(ref).max(), 1e-3))
 
 
-@pytest.mark.parametrize("M", [1, 8])
+@pytest.mark.parametrize("M", [1, 8, 10, 16])
 def test_small_product_plain_form_and_refusals(ops, M):
     """The same kernel without a norm in front (a tensor in x's place), float32 and bfloat16 results,
     one and two column groups per workgroup; shapes it does not take are refused by the entry."""
     rng = np.random.default_rng(77 + M)
-    for N, K in ((4096 + 16, 128), (16400, 64), (24, 320)):
+    for N, K in ((4096 + 16, 128), (16400, 64), (48, 320)):
         x = _bf16_grid(rng.normal(size=(M, K)))
         w = _bf16_grid(rng.normal(size=(N, K)) * 0.05)
         for dtype in (torch.bfloat16, torch.float32):
@@ -1203,10 +1204,11 @@ def test_small_product_plain_form_and_refusals(ops, M):
             ops._gemm8(_t(x, torch.bfloat16), _t(w, torch.bfloat16), out, N, False)
             tol = dict(rtol=2 ** -7, atol=1e-3) if dtype == torch.bfloat16 else dict(rtol=0, atol=2e-5 * math.sqrt(K))
             np.testing.assert_allclose(_np(out), plain.linear(x, w), **tol)
-    assert not ops.gemm8_supported(9, 2048, 2048) and not ops.gemm8_supported(4, 2044, 2048) and not ops.gemm8_supported(4, 2048, 96)
+    assert not ops.gemm8_supported(17, 2048, 2048) and not ops.gemm8_supported(4, 2044, 2048) and not ops.gemm8_supported(4, 2048, 96)
+    assert ops.gemm8_supported(8, 24, 64) and not ops.gemm8_supported(9, 24, 64)      # 9 to 16 rows: whole 16-column tiles
     with pytest.raises(ops.KernelError, match="unsupported shape"):
-        ops._gemm8(torch.zeros(9, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV),
-                   torch.zeros(9, 8, dtype=torch.bfloat16, device=DEV), 8, False)
+        ops._gemm8(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(16, 64, dtype=torch.bfloat16, device=DEV),
+                   torch.zeros(17, 16, dtype=torch.bfloat16, device=DEV), 16, False)
 
 
 # ------------------------------------------------ where the order of rounding and multiplying shows

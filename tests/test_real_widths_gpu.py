@@ -86,19 +86,22 @@ def test_real_widths_whole_tail_singly_and_mixed(real_width_setup, dtype):
 
 
 def test_real_widths_decode_through_the_engine_with_forced_tokens(real_width_setup):
-    """The scheduler's own decode steps at batch 3 and 8 (graphs, the products that fold the norms in)
-    and its prompt steps (the library's products), teacher-forced: logits against the plain implementation."""
+    """The scheduler's own decode steps at batch 3, 8 and 13 (graphs; the products that fold the norms in,
+    in their form for up to 8 rows and in the one for 9 to 16) and its prompt steps (the library's products),
+    teacher-forced: logits against the plain implementation."""
     from kvcm_amd import Engine, EngineConfig
     from kvcm_amd.engine.replay import scheduled_replay
     cfg, tensors, reqs, ref = real_width_setup["bfloat16"]
     scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
-    for live in (3, 8):
-        eng = Engine(config=EngineConfig(block_size=16, num_blocks=256, max_seq_len=1024, max_num_seqs=live, max_batched_tokens=1024),
+    for live in (3, 8, 13):
+        # (13 live: a budget that takes all prompts in one step, so that they decode side by side)
+        eng = Engine(config=EngineConfig(block_size=16, num_blocks=512 if live == 13 else 256, max_seq_len=1024, max_num_seqs=live,
+                                         max_batched_tokens=4096 if live == 13 else 1024),
                      architecture="LlamaForCausalLM", model_config=cfg, tensors=tensors)
         requests = []
         for rid, toks in reqs.items():
             n = len(toks)
-            for cut in ((n - 12, n - 5) if live == 8 else (n - 12,)):
+            for cut in ((n - 12,) if live == 3 else (n - 12, n - 5) if live == 8 else (n - 14, n - 12, n - 5)):
                 if cut > 0:
                     requests.append((rid, cut, toks[:cut], toks[cut:]))
         got = scheduled_replay(eng, [(p, c) for _, _, p, c in requests])
@@ -108,3 +111,6 @@ def test_real_widths_decode_through_the_engine_with_forced_tokens(real_width_set
             assert err <= 1e-2 * scale, (live, rid, cut, err)
         st = eng.recorded.stats()
         assert st["steps_as_graph"] > 0 and eng.core.blocks_in_use() == 0
+        if live == 13:       # some steps did run more than 8 requests at once
+            shapes = {(shape.rows, shape.max_run, kind) for shape, kind in eng.recorded.recorded_shapes.items()}
+            assert (13, 1, "graph") in shapes, shapes   # (the batch bucket of 16 rows, cut down to this engine's 13 sequences)
