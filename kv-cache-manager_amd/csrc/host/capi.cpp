@@ -208,7 +208,7 @@ int kvcm_seq_info(void* c, int64_t id, int64_t* out) {
     const Sequence* s = static_cast<Core*>(c)->find(id);
     out[0] = s->size(); out[1] = s->prompt_len; out[2] = s->num_computed; out[3] = s->cached_tokens;
     out[4] = s->state_slot; out[5] = s->num_preemptions; out[6] = s->max_new_tokens;
-    out[7] = static_cast<int64_t>(s->block_hashes.size());
+    out[7] = static_cast<int64_t>(s->page_hashes.size());
     out[8] = s->prefill_tokens_computed; out[9] = s->prefill_tokens_saved;
     return 0;
   }));
@@ -329,13 +329,13 @@ int kvcm_sched_plan(void* c, int64_t* ids, int32_t* start, int32_t* count, int32
     const auto& plan = static_cast<Core*>(c)->sched->plan();
     if (static_cast<int>(plan.size()) > cap) throw std::length_error("plan buffer too small");
     for (size_t i = 0; i < plan.size(); ++i) {
-      ids[i] = plan[i].seq->id;
-      start[i] = plan[i].start;
-      count[i] = plan[i].num_tokens;
-      flags[i] = (plan[i].is_prefill ? 1 : 0) | (plan[i].samples ? 2 : 0);
-      gen_index[i] = plan[i].seq->num_generated();
-      temperature[i] = plan[i].seq->temperature;
-      seed[i] = plan[i].seq->sampler_seed;
+      ids[i] = plan[i].request->id;
+      start[i] = plan[i].first;
+      count[i] = plan[i].count;
+      flags[i] = (plan[i].given ? 1 : 0) | (plan[i].samples ? 2 : 0);
+      gen_index[i] = plan[i].request->num_generated();
+      temperature[i] = plan[i].request->temperature;
+      seed[i] = plan[i].request->sampler_seed;
     }
     return static_cast<int64_t>(plan.size());
   }));
@@ -350,13 +350,13 @@ int kvcm_sched_schedule_summary(void* c, double now, int64_t* out) {
     int64_t prefill = 0, decode = 0, sampling = 0, single = 1, longest = 0, rows = 0, leading = 0, run = 0;
     bool still_leading = true;
     for (const auto& p : plan) {
-      if (p.is_prefill) prefill += p.num_tokens; else ++decode;
+      if (p.given) prefill += p.count; else ++decode;
       if (p.samples) ++sampling;
-      if (p.num_tokens != 1 || !p.samples) single = 0;
-      if (p.start + p.num_tokens > longest) longest = p.start + p.num_tokens;
-      rows += p.num_tokens;
-      if (p.num_tokens > run) run = p.num_tokens;
-      if (p.num_tokens != 1) still_leading = false;
+      if (p.count != 1 || !p.samples) single = 0;
+      if (p.first + p.count > longest) longest = p.first + p.count;
+      rows += p.count;
+      if (p.count > run) run = p.count;
+      if (p.count != 1) still_leading = false;
       if (still_leading) ++leading;
     }
     out[0] = static_cast<int64_t>(plan.size()); out[1] = prefill; out[2] = decode; out[3] = sampling;
@@ -459,14 +459,14 @@ int kvcm_build_batch(void* c, int n, const int64_t* ids, const int32_t* start, c
 static void plan_entries(Core* core, std::vector<BatchEntry>& entries) {
   for (const auto& p : core->sched->plan()) {
     BatchEntry e;
-    e.seq = p.seq;
-    e.start = p.start;
-    e.count = p.num_tokens;
-    if (p.samples) e.want = {p.num_tokens - 1};
-    e.temperature = p.seq->temperature;
-    e.sampler_seed = p.seq->sampler_seed;
-    e.request_id = p.seq->id;
-    e.token_index = p.seq->num_generated();
+    e.seq = p.request;
+    e.start = p.first;
+    e.count = p.count;
+    if (p.samples) e.want = {p.count - 1};
+    e.temperature = p.request->temperature;
+    e.sampler_seed = p.request->sampler_seed;
+    e.request_id = p.request->id;
+    e.token_index = p.request->num_generated();
     entries.push_back(std::move(e));
   }
 }
@@ -491,14 +491,14 @@ int kvcm_build_batch_from_plan(void* c, int pad_rows, int pad_seqs, int pad_logi
     std::vector<BatchEntry> entries;
     for (const auto& p : core->sched->plan()) {
       BatchEntry e;
-      e.seq = p.seq;
-      e.start = p.start;
-      e.count = p.num_tokens;
-      if (p.samples) e.want = {p.num_tokens - 1};
-      e.temperature = p.seq->temperature;
-      e.sampler_seed = p.seq->sampler_seed;
-      e.request_id = p.seq->id;
-      e.token_index = p.seq->num_generated();
+      e.seq = p.request;
+      e.start = p.first;
+      e.count = p.count;
+      if (p.samples) e.want = {p.count - 1};
+      e.temperature = p.request->temperature;
+      e.sampler_seed = p.request->sampler_seed;
+      e.request_id = p.request->id;
+      e.token_index = p.request->num_generated();
       entries.push_back(std::move(e));
     }
     build_batch(*core->kv, entries, pad_rows, pad_seqs, pad_logit_rows, table_stride, out, cap, desc);

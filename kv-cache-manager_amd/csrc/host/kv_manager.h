@@ -190,14 +190,14 @@ class PagedManager : public KVManager {
       if (!t.empty()) throw std::logic_error("admit: the sequence already holds pages");
     if (seq.state_slot >= 0) throw std::logic_error("admit: the sequence already holds a state slot");
     prepare(seq);
-    seq.block_hashes.clear();
+    seq.page_hashes.clear();
     int hits = 0;
     if (prefix_) {
       hits = common_hits(seq, nullptr);
       for (int g = 0; g < num_groups(); ++g) {
         std::vector<uint64_t> hashes;
         pools_[g]->cache.match_and_acquire(seq.tokens.data(), hits, matchable(seq), seq.tables[g], hashes);
-        if (g == 0) seq.block_hashes = hashes;
+        if (g == 0) seq.page_hashes = hashes;
       }
     }
     seq.cached_tokens = hits * bs_;
@@ -226,12 +226,12 @@ class PagedManager : public KVManager {
   void commit(Sequence& seq) override {
     if (prefix_) {
       const int full = seq.num_computed / bs_;
-      for (int b = static_cast<int>(seq.block_hashes.size()); b < full; ++b) {
-        const uint64_t parent = b ? seq.block_hashes[b - 1] : 0;
+      for (int b = static_cast<int>(seq.page_hashes.size()); b < full; ++b) {
+        const uint64_t parent = b ? seq.page_hashes[b - 1] : 0;
         const int32_t* t = seq.tokens.data() + static_cast<size_t>(b) * bs_;
         const uint64_t h = chain_hash(parent, t, bs_);
         for (int g = 0; g < num_groups(); ++g) pools_[g]->cache.insert(seq.tables[g][b], parent, h, t);
-        seq.block_hashes.push_back(h);
+        seq.page_hashes.push_back(h);
       }
     }
     // The next query sits at position >= num_computed and sees keys t > position - window.
@@ -260,7 +260,7 @@ class PagedManager : public KVManager {
       slots_.give_back(seq.state_slot);
       seq.state_slot = -1;
     }
-    seq.block_hashes.clear();
+    seq.page_hashes.clear();
     seq.num_computed = 0;
   }
 

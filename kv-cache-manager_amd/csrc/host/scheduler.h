@@ -1,24 +1,24 @@
 // Continuous batching, first come first served, with preemption by recomputation.
 //
 // A step is planned in three passes over one token budget:
-//   room      every running request gets the page its next token needs; when the pool is empty the
-//             youngest running request gives its pages back and waits again (its tokens stay, its
-//             keys are computed again later);
-//   running   requests that decode take one token each (all of them, before anything else is
+//   pages     every active request gets the page its next token needs; when the pool is empty the
+//             youngest active request gives its pages back and queues again at the front (its
+//             tokens stay, its keys are computed again later);
+//   active    requests that decode take one token each (all of them, before anything else is
 //             counted against the budget); requests still inside their prompt take a portion;
-//   waiting   the queue is admitted strictly in arrival order while sequences, tokens and pages
-//             allow; a request that could never fit an empty pool is finished without a token.
+//   queue     requests are admitted strictly in arrival order while sequences, tokens and pages
+//             allow; a request that could never fit an empty pool is retired without a token.
 // A portion is the part of a request's uncomputed tokens that runs in one step.  Its size is
 // bounded by `prefill_chunk`; 0 means portions are never cut, and then a portion is everything that
 // is left, a request enters a step only if all of it fits the budget (or the step is empty), and
 // every plan equals the reference scheduler's (src/core/scheduler.cpp:25-105).  A portion that does
 // not reach the request's last token samples nothing.
 #pragma once
-#include <algorithm>
 #include <cstdint>
 #include <deque>
 #include <limits>
 #include <memory>
+#include <stdexcept>
 #include <utility>
 #include <vector>
 
@@ -27,194 +27,207 @@
 namespace kvcm {
 
 struct SchedulerConfig {
-  int max_num_seqs = 256;         // most sequences running at once
-  int max_batched_tokens = 4096;  // token budget of a step
-  int prefill_chunk = 0;          // 0 = prompts are never cut
-  int eos_id = -1;                // >= 0: a sampled token equal to it finishes the request
+  int max_num_seqs = 256, max_batched_tokens = 4096;   // most active requests; token budget of a step
+  int prefill_chunk = 0;                               // 0 = prompts are never cut
+  int eos_id = -1;                                     // >= 0: a sampled token equal to it ends the request
 };
 
-struct ScheduledSeq {
-  Sequence* seq;
-  int start;
-  int num_tokens;
-  bool is_prefill;  // the run covers tokens that were given (prompt, or all of them after a preemption)
-  bool samples;     // the run reaches the last token, so a token is sampled from its last row
+// What one step runs of one request: tokens [first, first + count).
+struct PlannedRun {
+  Sequence* request;
+  int first, count;
+  bool given;     // the tokens were given to the engine (prompt, or all of them after a preemption), not sampled by it
+  bool samples;   // the run reaches the request's last token, so a token is sampled from its last row
 };
 
 struct SchedulerCounters {
   int64_t steps = 0, preemptions = 0, admissions = 0, admission_blocked_steps = 0, rejected = 0;
   int64_t prefill_tokens = 0, decode_tokens = 0, prefill_tokens_saved = 0, batch_size_sum = 0;
-  int max_running = 0;
+  int64_t max_running = 0;
 };
 
 class Scheduler {
  public:
-  Scheduler(KVManager& kv, SchedulerConfig cfg) : kv_(kv), cfg_(cfg) {}
+  using Owned = std::unique_ptr<Sequence>;
 
-  void add(std::unique_ptr<Sequence> s) { waiting_.push_back(std::move(s)); }
+  Scheduler(KVManager& pool, const SchedulerConfig& limits) : pool_(pool), limits_(limits) {}
 
-  const std::vector<ScheduledSeq>& schedule(double now) {
-    plan_.clear();
-    make_room();
-    int budget = cfg_.max_batched_tokens;
-    plan_running(budget);
-    if (admit_waiting(budget, now)) ++ctr_.admission_blocked_steps;
-    ++ctr_.steps;
-    ctr_.batch_size_sum += static_cast<int64_t>(running_.size());
-    ctr_.max_running = std::max(ctr_.max_running, static_cast<int>(running_.size()));
-    return plan_;
+  void add(Owned request) { queue_.push_back(std::move(request)); }
+
+  const std::vector<PlannedRun>& schedule(double now) {
+    runs_.clear();
+    tokens_left_ = limits_.max_batched_tokens;
+    secure_next_pages();
+    plan_active();
+    if (admit_from_queue(now) == Held::ByPool) tally_.admission_blocked_steps += 1;
+    const int64_t n = static_cast<int64_t>(active_.size());
+    tally_.steps += 1;
+    tally_.batch_size_sum += n;
+    if (n > tally_.max_running) tally_.max_running = n;
+    return runs_;
   }
 
-  // next_tokens[i] belongs to plan entry i; it is ignored where that entry samples nothing.
-  void update(const std::vector<int32_t>& next_tokens, double now) {
-    if (next_tokens.size() < plan_.size()) throw std::invalid_argument("update: one token per plan entry");
-    bool any_finished = false;
-    for (size_t i = 0; i < plan_.size(); ++i) {
-      const ScheduledSeq& run = plan_[i];
-      Sequence& s = *run.seq;
-      s.num_computed = run.start + run.num_tokens;
-      kv_.commit(s);
-      if (!run.samples) continue;
-      s.in_prompt = false;
-      s.tokens.push_back(next_tokens[i]);
-      if (s.first_token < 0) s.first_token = now;
-      const bool stop = s.done() || s.size() >= kv_.max_seq_len() || (cfg_.eos_id >= 0 && next_tokens[i] == cfg_.eos_id);
-      if (stop) {
-        s.finished = now;
-        any_finished = true;
+  // sampled[k] belongs to run k of the plan; it is ignored where that run samples nothing.
+  void update(const std::vector<int32_t>& sampled, double now) {
+    if (sampled.size() < runs_.size()) throw std::invalid_argument("update: one token per plan entry");
+    bool some_ended = false;
+    for (size_t k = 0; k < runs_.size(); ++k) {
+      const PlannedRun& r = runs_[k];
+      Sequence& q = *r.request;
+      q.num_computed = r.first + r.count;
+      pool_.commit(q);
+      if (!r.samples) continue;
+      const int32_t token = sampled[k];
+      q.in_prompt = false;
+      q.tokens.push_back(token);
+      if (q.first_token < 0) q.first_token = now;
+      if (q.done() || q.size() >= pool_.max_seq_len() || (limits_.eos_id >= 0 && token == limits_.eos_id)) {
+        q.finished = now;
+        some_ended = true;
       }
     }
-    if (any_finished) {
-      std::deque<std::unique_ptr<Sequence>> still;
-      for (auto& s : running_) {
-        if (s->finished < 0) {
-          still.push_back(std::move(s));
-          continue;
-        }
-        kv_.release(*s);
-        finished_.push_back(std::move(s));
-      }
-      running_.swap(still);
-    }
-    plan_.clear();
+    if (some_ended) retire_ended();
+    runs_.clear();
   }
 
-  std::vector<std::unique_ptr<Sequence>> take_finished() { return std::exchange(finished_, {}); }
+  std::vector<Owned> take_finished() { return std::exchange(retired_, {}); }
 
-  bool idle() const { return waiting_.empty() && running_.empty(); }
-  size_t num_waiting() const { return waiting_.size(); }
-  size_t num_running() const { return running_.size(); }
-  const std::deque<std::unique_ptr<Sequence>>& running() const { return running_; }
-  const std::vector<ScheduledSeq>& plan() const { return plan_; }
+  bool idle() const { return queue_.empty() && active_.empty(); }
+  size_t num_waiting() const { return queue_.size(); }
+  size_t num_running() const { return active_.size(); }
+  const std::vector<PlannedRun>& plan() const { return runs_; }
+  // The requests that hold pages, in admission order.
   std::vector<const Sequence*> live() const {
-    std::vector<const Sequence*> v;
-    v.reserve(running_.size());
-    for (const auto& s : running_) v.push_back(s.get());
-    return v;
+    std::vector<const Sequence*> out(active_.size());
+    for (size_t i = 0; i < active_.size(); ++i) out[i] = active_[i].get();
+    return out;
   }
-  const SchedulerCounters& counters() const { return ctr_; }
-  void reset_counters() { ctr_ = {}; }
-  KVManager& kv() { return kv_; }
-  const SchedulerConfig& config() const { return cfg_; }
+  const SchedulerCounters& counters() const { return tally_; }
+  void reset_counters() { tally_ = SchedulerCounters{}; }
+  const SchedulerConfig& config() const { return limits_; }
 
  private:
-  bool cuts_prompts() const { return cfg_.prefill_chunk > 0; }
+  enum class Held { No, ByPool };
+
+  bool cuts_prompts() const { return limits_.prefill_chunk > 0; }
   // The most tokens of one request a step takes, given what is left of the budget: a prompt that
   // may be cut shrinks to what is left (a new request always gets one token), one that may not is
   // taken whole.
-  int portion_limit(int budget_left, int at_least) const {
+  int portion_limit(int left, int at_least) const {
     if (!cuts_prompts()) return std::numeric_limits<int>::max();
-    return std::min(cfg_.prefill_chunk, std::max(budget_left, at_least));
+    const int room = left > at_least ? left : at_least;
+    return room < limits_.prefill_chunk ? room : limits_.prefill_chunk;
   }
-  static int uncomputed(const Sequence& s) { return s.size() - s.num_computed; }
+  static int uncomputed(const Sequence& q) { return q.size() - q.num_computed; }
 
-  // Adds a run of `n` tokens of `s` to the plan and books it.
-  void take(Sequence& s, int n, int& budget) {
-    const bool given = s.in_prompt;   // tokens that were given to the engine, not sampled by it
-    plan_.push_back({&s, s.num_computed, n, given, n == uncomputed(s)});
-    budget -= n;
-    if (given) {
-      ctr_.prefill_tokens += n;
-      s.prefill_tokens_computed += n;
+  // Adds a run of `n` tokens of `q` to the plan and books it.
+  void take(Sequence& q, int n) {
+    runs_.push_back(PlannedRun{&q, q.num_computed, n, q.in_prompt, n == uncomputed(q)});
+    tokens_left_ -= n;
+    if (q.in_prompt) {
+      tally_.prefill_tokens += n;
+      q.prefill_tokens_computed += n;
     } else {
-      ctr_.decode_tokens += n;
+      tally_.decode_tokens += n;
     }
   }
 
-  // A page for the next token of every running request, oldest first.  The victim of an empty
-  // pool is always the youngest; when that is the request asking, nothing younger is left to ask.
-  void make_room() {
-    size_t i = 0;
-    while (i < running_.size()) {
-      if (kv_.append_slot(*running_[i])) {
-        ++i;
+  // A page for the next token of every active request, oldest first.  An empty pool takes the
+  // pages of the youngest; when that is the request asking, nothing younger is left to ask.
+  void secure_next_pages() {
+    for (size_t at = 0; at < active_.size();) {
+      if (pool_.append_slot(*active_[at])) {
+        ++at;
         continue;
       }
-      const bool asked_for_itself = i + 1 == running_.size();
-      std::unique_ptr<Sequence> victim = std::move(running_.back());
-      running_.pop_back();
-      kv_.release(*victim);
-      ++victim->num_preemptions;
-      ++ctr_.preemptions;
-      waiting_.push_front(std::move(victim));
-      if (asked_for_itself) break;
+      const bool was_asking = at + 1 == active_.size();
+      Owned youngest = std::move(active_.back());
+      active_.pop_back();
+      pool_.release(*youngest);
+      youngest->num_preemptions += 1;
+      tally_.preemptions += 1;
+      queue_.push_front(std::move(youngest));
+      if (was_asking) return;
     }
   }
 
-  // Running requests in admission order.  The tokens of decoding requests are set aside first, so
+  // Active requests in admission order.  The tokens of decoding requests are set aside first, so
   // that a prompt's portion earlier in the order cannot starve them of budget.
-  void plan_running(int& budget) {
-    int decoding = 0;
-    for (const auto& s : running_)
-      if (!s->in_prompt) decoding += uncomputed(*s);
-    int for_prompts = budget - decoding;
-    for (auto& s : running_) {
-      if (!s->in_prompt) {
-        take(*s, uncomputed(*s), budget);
+  void plan_active() {
+    int for_prompts = tokens_left_;
+    for (const Owned& q : active_)
+      if (!q->in_prompt) for_prompts -= uncomputed(*q);
+    for (const Owned& q : active_) {
+      const int open = uncomputed(*q);
+      if (!q->in_prompt) {
+        take(*q, open);
         continue;
       }
-      const int n = std::min(uncomputed(*s), portion_limit(for_prompts, 0));
+      const int cap = portion_limit(for_prompts, 0);
+      const int n = open < cap ? open : cap;
       if (n <= 0) continue;   // no budget left in this step: the request waits with its pages
-      take(*s, n, budget);
+      take(*q, n);
       for_prompts -= n;
     }
   }
 
-  // Returns true when the head of the queue was held back by the pool (not by the budget).
-  bool admit_waiting(int& budget, double now) {
-    while (!waiting_.empty() && static_cast<int>(running_.size()) < cfg_.max_num_seqs) {
-      Sequence& head = *waiting_.front();
+  // Admits from the front of the queue; says whether the front was held back by the pool (and not
+  // by the budget or the limit of active requests).
+  Held admit_from_queue(double now) {
+    while (!queue_.empty() && static_cast<int>(active_.size()) < limits_.max_num_seqs) {
+      Sequence& next = *queue_.front();
       // what the step must still have room for: one token of a prompt that may be cut, all of
       // one that may not; an empty step takes its first request whatever its size
-      const int least = cuts_prompts() ? 1 : head.size();
-      if (!plan_.empty() && budget < least) return false;
-      if (!kv_.can_admit(head)) {
-        if (!running_.empty()) return true;
-        head.finished = now;  // it fits not even an empty pool: finished without a token
-        ++ctr_.rejected;
-        finished_.push_back(std::move(waiting_.front()));
-        waiting_.pop_front();
+      const int least = cuts_prompts() ? 1 : next.size();
+      if (!runs_.empty() && tokens_left_ < least) return Held::No;
+      if (!pool_.can_admit(next)) {
+        if (!active_.empty()) return Held::ByPool;
+        next.finished = now;   // it fits not even an empty pool: retired without a token
+        tally_.rejected += 1;
+        retired_.push_back(pop_queue());
         continue;
       }
-      kv_.admit(head);  // pages for all its tokens; prefix hits move num_computed forward
-      if (head.admitted < 0) head.admitted = now;
-      head.in_prompt = true;
-      ++ctr_.admissions;
-      ctr_.prefill_tokens_saved += head.cached_tokens;
-      take(head, std::min(uncomputed(head), portion_limit(budget, 1)), budget);
-      running_.push_back(std::move(waiting_.front()));
-      waiting_.pop_front();
+      pool_.admit(next);   // pages for all its tokens; prefix hits move num_computed forward
+      if (next.admitted < 0) next.admitted = now;
+      next.in_prompt = true;
+      tally_.admissions += 1;
+      tally_.prefill_tokens_saved += next.cached_tokens;
+      const int open = uncomputed(next), cap = portion_limit(tokens_left_, 1);
+      take(next, open < cap ? open : cap);
+      active_.push_back(pop_queue());
     }
-    return false;
+    return Held::No;
   }
 
-  KVManager& kv_;
-  SchedulerConfig cfg_;
-  std::deque<std::unique_ptr<Sequence>> waiting_;
-  std::deque<std::unique_ptr<Sequence>> running_;  // admission order, back = youngest
-  std::vector<std::unique_ptr<Sequence>> finished_;
-  std::vector<ScheduledSeq> plan_;
-  SchedulerCounters ctr_;
+  Owned pop_queue() {
+    Owned front = std::move(queue_.front());
+    queue_.pop_front();
+    return front;
+  }
+
+  // Requests whose `finished` time is set leave the active list (order kept) and give their pages back.
+  void retire_ended() {
+    size_t kept = 0;
+    for (size_t i = 0; i < active_.size(); ++i) {
+      if (active_[i]->finished >= 0) {
+        pool_.release(*active_[i]);
+        retired_.push_back(std::move(active_[i]));
+      } else {
+        if (kept != i) active_[kept] = std::move(active_[i]);
+        ++kept;
+      }
+    }
+    active_.resize(kept);
+  }
+
+  KVManager& pool_;
+  SchedulerConfig limits_;
+  std::deque<Owned> queue_;      // arrival order; a preempted request goes to the front
+  std::vector<Owned> active_;    // admission order, back = youngest
+  std::vector<Owned> retired_;
+  std::vector<PlannedRun> runs_;
+  int tokens_left_ = 0;
+  SchedulerCounters tally_;
 };
 
 }  // namespace kvcm
