@@ -142,7 +142,9 @@ def main():
                          "choice (the engine's default), the fastest of its choices, or the fastest of all; timed at a "
                          "shape's first use, before anything is measured (tens of milliseconds per shape: worth it "
                          "for shapes that run thousands of times, as a benchmark's do)")
-    ap.add_argument("--context-limit", type=int, default=2048, help="most tokens a request may hold; sizes the cache pool")
+    ap.add_argument("--context-limit", type=int, default=0,
+                    help="most tokens a request may hold; sizes the cache pool (default: 2,048, or what --prompt-len, "
+                         "--warmup and --steps need if that is more)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
@@ -151,9 +153,10 @@ def main():
         print("bench.py: this engine runs on one GPU; --gpus N with N > 1 is not supported")
         sys.exit(2)
 
-    limit = args.context_limit
     budget = max(4096, args.prompt_len + args.batch)     # a whole prompt fits a step beside the decoding requests
-    if args.prompt_len + args.warmup + args.steps + 24 + prompt_step_count(args.batch, args.prompt_len, budget) > limit:
+    needed = args.prompt_len + args.warmup + args.steps + 24 + prompt_step_count(args.batch, args.prompt_len, budget)
+    limit = args.context_limit or max(2048, -(-needed // 64) * 64)
+    if needed > limit:
         print("bench.py: --prompt-len %d plus the decoded tokens does not fit --context-limit %d" % (args.prompt_len, limit))
         sys.exit(2)
 
