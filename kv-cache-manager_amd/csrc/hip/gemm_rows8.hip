@@ -452,7 +452,14 @@ int kvcm_gemm8(const void* X, int ldx, const void* W, int ldw, int M, int N, int
     return launch_status("gemm8_swiglu");
   }
   // two row groups per workgroup once a single one would give more than about four workgroups per CU
-  if (N % (2 * kCols) == 0 && N / kCols > 1024) {
+  // (measured in whole decode steps: the head and the QKV product of a 7B model), and also where that leaves no CU
+  // with more columns than it has with one (TinyLlama's QKV product: 320 tiles are two workgroups on 64 of the
+  // 256 CUs either way, and 160 workgroups of two groups start and end faster: batch 8 1.027 -> 1.008 ms; at 768
+  // tiles, a width of 4,096 with 8 KV heads, two groups give some CUs four tiles instead of three and are slower)
+  constexpr int kCUs = 256;
+  const int tiles = N / kCols;
+  const bool two_fit = tiles > kCUs && 2 * ((tiles / 2 + kCUs - 1) / kCUs) <= (tiles + kCUs - 1) / kCUs;
+  if (N % (2 * kCols) == 0 && (tiles > 1024 || two_fit)) {
     const dim3 grid(N / (2 * kCols));
     if (out_dtype == kBF16) { if (scaled) KVCM_G8(2, 2, true, kStore, bf16_t); else KVCM_G8(2, 2, false, kStore, bf16_t); }
     else { if (scaled) KVCM_G8(2, 2, true, kStore, float); else KVCM_G8(2, 2, false, kStore, float); }
