@@ -204,8 +204,15 @@ def main():
         return {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
                 "frac": round(flops / sec / PEAK_FLOPS[key], 4)}
 
+    def tuning_log():   # which shapes were tuned, the first choice's and the kept algorithm's microseconds
+        if os.environ.get("KVCM_BENCH_TUNING_LOG"):
+            from kvcm_amd import ops
+            for row in ops.library_tuning_log:
+                print("tuned M=%d N=%d K=%d: %.1f -> %.1f us (%d candidates)" % row, file=sys.stderr)
+
     if args.only_prefill:
         print(json.dumps({"prefill": prefill_record()}), flush=True)
+        tuning_log()
         return
 
     seconds, ctx = decode_run(eng, args.batch, args.prompt_len, args.steps, args.warmup, V)
@@ -235,10 +242,7 @@ def main():
         # beside the published peaks the fractions above are taken against: what this GPU reached in this run
         out["measured"] = measured_peaks()
     print(json.dumps(out), flush=True)
-    if os.environ.get("KVCM_BENCH_TUNING_LOG"):       # which shapes were tuned, the first choice's and the kept algorithm's microseconds
-        from kvcm_amd import ops
-        for row in ops.library_tuning_log:
-            print("tuned M=%d N=%d K=%d: %.1f -> %.1f us (%d candidates)" % row, file=sys.stderr)
+    tuning_log()
 
 
 if __name__ == "__main__":
