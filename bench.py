@@ -28,7 +28,7 @@ SIZES = dict(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_hid
              rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
 
 
-def build_engine(cfg, dtype, max_num_seqs, max_batched_tokens, tensors, context_limit=2048, tune_products="heuristic"):
+def build_engine(cfg, dtype, max_num_seqs, max_batched_tokens, tensors, context_limit=2048, tune_products="off"):
     from kvcm_amd.config.engine_config import EngineConfig
     from kvcm_amd.engine.engine import Engine
     ec = EngineConfig(block_size=16, max_seq_len=context_limit, num_blocks=max_num_seqs * context_limit // 16,
@@ -137,11 +137,11 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--sizes", default="tinyllama-1.1b", help="layer sizes by name (tinyllama-1.1b, llama-2-7b, llama-3-8b)")
-    ap.add_argument("--tune-products", default="heuristic", choices=["off", "heuristic", "all"],
+    ap.add_argument("--tune-products", default="off", choices=["off", "heuristic", "all"],
                     help="which of the vendor library's algorithms the many-row products of prompt steps run: its first "
-                         "choice (the engine's default), the fastest of its choices, or the fastest of all; timed at a "
-                         "shape's first use, before anything is measured (tens of milliseconds per shape: worth it "
-                         "for shapes that run thousands of times, as a benchmark's do)")
+                         "choice (the engine's default, and this program's: the figures are a default engine's), the "
+                         "fastest of its choices, or the fastest of all; timed at a shape's first use, before anything "
+                         "is measured (tens of milliseconds per shape: worth it for shapes that run thousands of times)")
     ap.add_argument("--context-limit", type=int, default=0,
                     help="most tokens a request may hold; sizes the cache pool (default: 2,048, or what --prompt-len, "
                          "--warmup and --steps need if that is more)")
@@ -176,16 +176,13 @@ def main():
     cfg = LlamaConfig.from_dict(sizes)
     dt = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     tensors = random_tensors("LlamaForCausalLM", cfg, seed=0, dtype=dt, device="cuda:0")
-    esize = 2 if args.dtype == "bfloat16" else 4
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
     H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
-    layer_params = cfg.qkv_dim * H + H * cfg.q_dim + 3 * I * H + 2 * H
-    kv_bytes_per_token = 2 * L * cfg.kv_dim * esize
 
     def roofline(batch, seconds_per_step, ctx):
-        weights = (L * layer_params + H + V * H + batch * H) * esize
-        cache = batch * ctx * kv_bytes_per_token
-        achieved = (weights + cache) / seconds_per_step / 1e9
+        # the bytes are the loaded model's and its cache storages' own count (every weight the step uses once,
+        # the embedding rows of its tokens, the keys and values of the live requests), not a formula of sizes
+        achieved = eng.runner.step_bytes([ctx] * batch) / seconds_per_step / 1e9
         return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_GBS, 4)}
 
@@ -199,8 +196,7 @@ def main():
     def prefill_record():
         T = 2048
         sec = prefill_run(eng, T, V)
-        flops = (2.0 * T * (L * (layer_params - 2 * H)) + 2.0 * V * H
-                 + L * 4.0 * (T * (T + 1) / 2) * cfg.head_dim * cfg.num_attention_heads)
+        flops = eng.model.step_flops(T, 1, T * (T + 1) // 2)      # the parts' own count: products, and q.k and p.v
         return {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
                 "frac": round(flops / sec / PEAK_FLOPS[key], 4)}
 

@@ -46,6 +46,12 @@ class KVStorage:
     def total_bytes(self) -> int:
         return self.data.numel() * self.data.element_size()
 
+    def bytes_read(self, context: int) -> int:
+        """Bytes a request with ``context`` tokens has a step read from this group: the keys and values of
+        every layer, of the window's tokens where there is a window."""
+        tokens = min(context, self.need.window) if self.need.window > 0 else context
+        return tokens * (self.bytes_per_block // self.block_size)
+
 
 class StateStorage:
     def __init__(self, group: int, need: StateNeed, num_layers: int, num_slots: int, device):
@@ -55,6 +61,10 @@ class StateStorage:
 
     def slots(self, layer: int) -> torch.Tensor:
         return self.data[layer]
+
+    def bytes_read(self, context: int) -> int:
+        """One slot of every layer, whatever the context."""
+        return self.num_layers * (self.data[0, 0].numel() * self.data.element_size())
 
     @property
     def total_bytes(self) -> int:

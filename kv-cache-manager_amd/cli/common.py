@@ -27,7 +27,8 @@ def engine_config_from_args(a, **overrides) -> EngineConfig:
     """Flag names and defaults of the reference's kvbench (src/main_bench.cpp:24-43), plus
     --dtype, --prefill-chunk, --eos-id, --no-graphs (no decode steps as HIP graphs), --no-programs
     (no steps replayed from recorded launch lists: every step through the model's parts) and
-    --tune-products off|heuristic|all (which of the library's algorithms a many-row product runs)."""
+    --tune-products off|heuristic|all (which of the library's algorithms a many-row product runs) and
+    --no-fold-norms (every RMS norm a launch of its own, rounding where the reference does)."""
     ec = EngineConfig(
         policy=a.str("policy", "paged"), block_size=a.i32("block-size", 16), max_seq_len=a.i32("max-seq-len", 2048),
         prefix_caching=a.flag("prefix"), num_blocks=a.i32("num-blocks", 0), watermark_blocks=a.i32("watermark", -1),
@@ -35,7 +36,7 @@ def engine_config_from_args(a, **overrides) -> EngineConfig:
         max_batched_tokens=a.i32("max-batched-tokens", 4096), attn=a.str("attn", "auto"),
         dtype=a.str("dtype", "bfloat16"), prefill_chunk=a.i32("prefill-chunk", 0), eos_id=a.i32("eos-id", -1),
         use_graphs=not a.flag("no-graphs"), use_programs=not a.flag("no-programs"),
-        tune_products=a.str("tune-products", "off"))
+        tune_products=a.str("tune-products", "off"), fold_norms=not a.flag("no-fold-norms"))
     for k, v in overrides.items():
         setattr(ec, k, v)
     return ec.validate()

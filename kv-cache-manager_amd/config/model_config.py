@@ -15,6 +15,11 @@ class ConfigError(ValueError):
     pass
 
 
+# What the attention kernels take (csrc/hip/attention_generic.hip refuses anything else): 16-byte pieces of a
+# head's row, and a head that fits a wave's registers.
+MAX_HEAD_DIM = 256
+
+
 def read_config_json(model_dir):
     path = os.path.join(model_dir, "config.json")
     if not os.path.isfile(path):
@@ -65,8 +70,9 @@ class LlamaConfig:
             hd = raw["hidden_size"] // nh
         if not isinstance(nkv, int) or nkv <= 0 or nh % nkv:
             problems.append(f"num_attention_heads {nh} must be a multiple of num_key_value_heads {nkv!r}")
-        if not isinstance(hd, int) or hd <= 0 or hd % 2:
-            problems.append(f"head_dim {hd!r} must be a positive even integer (rotary pairs)")
+        if not isinstance(hd, int) or hd <= 0 or hd % 8 or hd > MAX_HEAD_DIM:
+            problems.append(f"head_dim {hd!r} is not supported: the attention kernels take multiples of 8 up to "
+                            f"{MAX_HEAD_DIM} (hidden_size {raw['hidden_size']}, num_attention_heads {nh})")
         scaling = raw.get("rope_scaling")
         plain_rotary = scaling in (None, {}) or (isinstance(scaling, dict) and set(scaling) <= {"rope_type", "type"}
                                                  and all(v == "default" for v in scaling.values()))

@@ -134,16 +134,22 @@ int kvcm_gemm_library(const void* X, const void* W, void* out, int M, int N, int
   KVCM_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_library: bad sizes M=%d N=%d K=%d", M, N, K);
   KVCM_REQUIRE(ldx >= K && ldw >= K && ldo >= N, "gemm_library: leading dimensions too small");
   KVCM_REQUIRE(X != nullptr && W != nullptr && out != nullptr, "gemm_library: null operand");
+  // the plan's algorithm and workspace size are copied out under the lock: a tuning call on another
+  // thread replaces them under the same lock (the descriptors of a plan never change once made)
   Plan* plan = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t algo_workspace = 0;
   {
     std::lock_guard<std::mutex> hold(g_lock);
     if (int rc = plan_for(plan, M, N, K, ldx, ldw, ldo)) return rc;
+    algo = plan->algo;
+    algo_workspace = plan->workspace;
   }
-  KVCM_REQUIRE(static_cast<long long>(plan->workspace) <= workspace_bytes && (plan->workspace == 0 || workspace != nullptr),
-               "gemm_library: the algorithm needs %zu bytes of workspace, %lld were given", plan->workspace, workspace_bytes);
+  KVCM_REQUIRE(static_cast<long long>(algo_workspace) <= workspace_bytes && (algo_workspace == 0 || workspace != nullptr),
+               "gemm_library: the algorithm needs %zu bytes of workspace, %lld were given", algo_workspace, workspace_bytes);
   const float one = 1.0f, zero = 0.0f;
   KVCM_BLAS(hipblasLtMatmul(g_handle, plan->desc, &one, W, plan->a, X, plan->b, &zero, out, plan->c, out, plan->c,
-                            &plan->algo, workspace, plan->workspace, stream));
+                            &algo, workspace, algo_workspace, stream));
   return 0;
 }
 

@@ -97,7 +97,8 @@ def build_runner(model_dir: Optional[str] = None, engine_config: Optional[Engine
         max_logit_rows=ec.max_logit_rows if ec.max_logit_rows > 0 else max(ec.max_num_seqs, 512),
         max_blocks_per_seq=(ec.max_seq_len + ec.block_size - 1) // ec.block_size,
         max_context_len=ec.max_seq_len)
-    runner = ModelRunner(model, core, storages, limits, dtype, dev, attn=ec.attn)
+    runner = ModelRunner(model, core, storages, limits, dtype, dev, attn=ec.attn, fold_norms=ec.fold_norms,
+                         tune_products=ec.tune_products)
     runner.weight_bytes = weight_bytes
     runner.num_blocks = num_blocks
     runner.engine_config = ec

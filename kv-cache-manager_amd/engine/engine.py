@@ -35,10 +35,11 @@ class Engine:
         self.sampler = Sampler(self.runner.ops, self.runner.device, self.runner.limits.max_logit_rows)
         self._next_id = 0
         self._score_id = -1
-        self._forced, self._forced_logits = {}, {}       # request id -> forced tokens / logits kept for them
+        # teacher forcing: live request id -> its given tokens (dropped when the request finishes);
+        # request id -> [given tokens, vocab] logits kept for it until ``forced_logits`` hands them out
+        self._forced, self._forced_logits = {}, {}
         self._t0 = time.perf_counter()
         self.config = self.runner.engine_config      # as built (max_seq_len within the model's range)
-        self.runner.ops.LIBRARY_TUNING = self.config.tune_products      # process-wide, like the library's plans
         # Recorded steps replay a fixed launch sequence: only for models whose parts all declare that
         # their launches depend on the step's shape alone (Part.capturable).  use_programs: steps are
         # recorded per shape and replayed natively; use_graphs: decode-shaped ones also as HIP graphs.
@@ -85,7 +86,8 @@ class Engine:
             if not forced or min(forced) < 0 or max(forced) >= V:
                 raise ValueError("forced tokens must be a non-empty list of ids inside the vocabulary")
             max_new_tokens = len(forced)
-            self._forced[request_id], self._forced_logits[request_id] = forced, {}
+            self._forced[request_id] = forced
+            self._forced_logits[request_id] = np.full((len(forced), V), np.nan, dtype=np.float32)
         self.core.sched_add(request_id, toks, int(max_new_tokens), float(temperature), int(seed),
                             self.now() if arrival is None else arrival)
         return request_id
@@ -96,7 +98,10 @@ class Engine:
         return self.core.idle()
 
     def take_finished(self) -> List[Finished]:
-        return self.core.take_finished()
+        done = self.core.take_finished()
+        for f in done:
+            self._forced.pop(f.id, None)       # nothing of a finished request stays behind but the logits it asked for
+        return done
 
     # ------------------------------------------------------------------------------- step
     def step(self) -> StepInfo:
@@ -153,19 +158,18 @@ class Engine:
                 continue
             given = self._forced.get(p.id)
             if given is not None:
-                self._forced_logits[p.id][p.gen_index] = rows[k].copy()
+                self._forced_logits[p.id][p.gen_index] = rows[k]
                 out[k] = given[p.gen_index]
             k += 1
         return out
 
     def forced_logits(self, request_id: int) -> np.ndarray:
         """Of a request added with ``forced``: the logits each of its forced tokens was to be sampled
-        from, [len(forced), vocab] (a row of NaN where none has been computed yet)."""
-        n, V = len(self._forced[request_id]), self.model.spec.vocab_size
-        out = np.full((n, V), np.nan, dtype=np.float32)
-        for k, row in self._forced_logits[request_id].items():
-            out[k] = row
-        return out
+        from, [len(forced), vocab] (a row of NaN where none has been computed yet).  A finished
+        request's logits are handed out once: the engine keeps nothing of it afterwards."""
+        if request_id in self._forced:
+            return self._forced_logits[request_id].copy()
+        return self._forced_logits.pop(request_id)
 
     def run_until_idle(self, max_steps: int = 1 << 30) -> List[Finished]:
         done = []

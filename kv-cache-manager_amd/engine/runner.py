@@ -90,6 +90,7 @@ class StepContext(StepView):
     def __init__(self, runner, layout: BatchLayout):
         self.runner, self.layout = runner, layout
         self.limits, self.attention_mode = runner.limits, runner.attn
+        self.fold_norms, self.tune_products = runner.fold_norms, runner.tune_products
         self.recording = False
         L = layout
         self.rows, self.real_rows = L.rows_padded, L.rows
@@ -160,9 +161,11 @@ class StepContext(StepView):
 
 
 class ModelRunner:
-    def __init__(self, model: Model, core: HostCore, storages, limits: ModelLimits, dtype, device, attn="auto"):
+    def __init__(self, model: Model, core: HostCore, storages, limits: ModelLimits, dtype, device, attn="auto",
+                 fold_norms=True, tune_products="off"):
         self.model, self.core, self.storages, self.limits = model, core, storages, limits
         self.dtype, self.device, self.attn = dtype, device, attn
+        self.fold_norms, self.tune_products = bool(fold_norms), tune_products
         self.ops = model.ctx.ops
         self.workspace = Workspace(device, dtype, limits, self.ops)
         G = core.num_groups
@@ -245,6 +248,15 @@ class ModelRunner:
             logits = self.model.head_logits(step, x, pending, step.logit_row_index[lo:hi])
             out[lo:hi] = logits.cpu().numpy()
         return out
+
+    # ------------------------------------------------------------------------------- cost
+    def step_bytes(self, contexts, rows=None, logit_rows=None) -> int:
+        """Bytes a step has to read, as the loaded model and the cache storages count them: every weight it
+        uses once, and the cache of the live requests (``contexts``: their lengths; one row and one wanted
+        row per request unless said otherwise)."""
+        n = len(contexts)
+        weights = self.model.step_bytes(n if rows is None else rows, n if logit_rows is None else logit_rows)
+        return weights + sum(s.bytes_read(c) for s in self.storages for c in contexts)
 
     def run_entries(self, entries, **pad) -> Optional[torch.Tensor]:
         """entries: (sequence id, start, count, want) as HostCore.build_batch takes them."""

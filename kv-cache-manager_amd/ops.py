@@ -461,7 +461,7 @@ def skinny_splits(M, N, K):
     return lib().kvcm_gemm_skinny_splits(M, N, K)
 
 
-def gemm(x, w, out, scratch=None, keep_partial=False):
+def gemm(x, w, out, scratch=None, keep_partial=False, tuning=None):
     """out[M, N] = x[M, K] @ w[N, K]^T.  float32 x float32 -> float32 (plain FMA, fixed k order), or
     bfloat16 x bfloat16 -> bfloat16 | float32 (MFMA, 32-bit accumulation).
 
@@ -469,6 +469,9 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
     while the library is switched off: inside a captured graph); when they split K they need
     ``scratch`` (float32, at least splits*M*N elements).  With ``keep_partial``
     the un-added partial sums are returned as PartialSums (for a fused consumer) instead of ``out``.
+    ``tuning``: which of the library's algorithms a many-row product runs ("off" | "heuristic" | "all";
+    None: this module's LIBRARY_TUNING); an engine passes its own option, so that two engines in one
+    process do not change each other's.
     """
     if isinstance(x, NormedRows):
         M, K = x.shape
@@ -508,7 +511,7 @@ def gemm(x, w, out, scratch=None, keep_partial=False):
         return partial if keep_partial else partial.materialize()
     if library:
         ws = _library_workspace(out.device)
-        mode = _TUNING_MODES[LIBRARY_TUNING]
+        mode = _TUNING_MODES[LIBRARY_TUNING if tuning is None else tuning]
         shape = (M, N, K, x.stride(0), w.stride(0), out.stride(0))
         if mode and lib().kvcm_gemm_library_tuned(*shape) < mode:
             # not a recorded launch: it runs here, once, whoever is recording

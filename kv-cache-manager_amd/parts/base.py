@@ -25,12 +25,15 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: an arrangement (block kind) of named parts.  ``cache_from`` names another layer
-    whose cache this layer's mixer reads instead of owning one."""
+    """One layer: an arrangement (block kind) of named parts.  Every part that reports a cache need
+    (``cache_need()``) owns a cache of its own, whatever its name and however many the layer has.
+    ``cache_from`` makes parts read another part's cache instead: a string for every cache-using part
+    of the layer (a layer's name: the part of the same name there; or ``layer.part``), or a dict from
+    this layer's part names to such strings (parts it does not list keep their own)."""
     name: str
     block: str
     parts: Dict[str, PartSpec]
-    cache_from: Optional[str] = None
+    cache_from: Optional[object] = None
 
 
 @dataclass(frozen=True)
@@ -109,6 +112,10 @@ class StepView:
       attention_mode               "auto" | "v1" | "v2" (the engine option of that name)
       recording                    True while the step is being recorded for replay: a part may then
                                    call nothing but this package's kernels (ctx.ops) on device arrays
+      fold_norms                   the engine option of that name: False keeps every norm a launch of its
+                                   own, rounding exactly where the reference does
+      tune_products                the engine option of that name ("off" | "heuristic" | "all"), handed to
+                                   ops.gemm as ``tuning``
 
     Device arrays (int32, this step's metadata; all a capturable part may read):
       tokens[rows] positions[rows] ctx_lens[rows] row_seq[rows]
@@ -134,6 +141,8 @@ class StepView:
 
     recording = False
     attention_mode = "auto"
+    fold_norms = True
+    tune_products = None
     max_run = 1
     limits = None
 
@@ -193,6 +202,28 @@ class Part:
     def bind(self, tensors: Dict[str, torch.Tensor]):
         self.w = dict(tensors)
 
+    # What a step costs, for rooflines: a measurement asks the model, and the model asks its parts.
+    def bytes_read(self, rows: int) -> int:
+        """Bytes of its tensors a step of ``rows`` rows has to read: every tensor once, unless the part
+        knows better (a table of which only ``rows`` rows are touched, experts that no row was routed to)."""
+        return sum(t.numel() * t.element_size() for t in self.w.values())
+
+    def flops(self, rows: int, attended: int = 0) -> float:
+        """Floating-point operations of a step of ``rows`` rows: two per row and matrix element, unless the
+        part knows better.  ``attended``: (row, key) pairs the step's rows see in all, for parts that attend."""
+        return 2.0 * rows * sum(t.numel() for t in self.w.values() if t.dim() == 2)
+
+    # A part of a layer that keeps something per request between steps says what (a mixer usually does;
+    # any part of a layer may, and a layer may have several).
+    def cache_need(self):
+        """KVCacheNeed, StateNeed or None."""
+        return None
+
+    def attach_cache(self, storage, index: int, owner: bool = True):
+        """storage: the group's device storage; index: this part's place in it; owner False: the
+        cache belongs to another part and is only read."""
+        self.cache, self.cache_index, self.cache_owner = storage, index, owner
+
 
 class Norm(Part):
     # True: ``add`` may be a Deferred (un-added split-K sums, a product that has not run yet), which
@@ -234,15 +265,6 @@ class PositionEncoding(Part):
 class Mixer(Part):
     # True: ``h`` may be a Deferred (ops.NormedRows) that the mixer's first product consumes as it is.
     accepts_normed_rows = False
-
-    def cache_need(self):
-        """KVCacheNeed, StateNeed or None."""
-        return None
-
-    def attach_cache(self, storage, index: int, owner: bool = True):
-        """storage: the group's device storage; index: this layer's place in it; owner False: the
-        cache belongs to another layer and is only read."""
-        self.cache, self.cache_index, self.cache_owner = storage, index, owner
 
     def forward(self, step, h):
         """h: normed hidden states [rows, H] in the compute dtype -> the mixer's output [rows, H]."""

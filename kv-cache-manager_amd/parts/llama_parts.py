@@ -18,7 +18,8 @@ def _linear(ctx, step, x, w, name, keep_partial=False, dtype=None):
     un-added split-K sums (ops.PartialSums) for a consumer that adds them up itself."""
     out = step.ws(name, (x.shape[0], w.shape[0]), dtype)
     scratch = step.scratch(name, x.shape[0], w.shape[0], w.shape[1])
-    return ctx.ops.gemm(x, w, out, scratch=scratch, keep_partial=keep_partial and scratch is not None)
+    return ctx.ops.gemm(x, w, out, scratch=scratch, keep_partial=keep_partial and scratch is not None,
+                        tuning=step.tune_products)
 
 
 def _to_residual(ctx, step, x, w, name):
@@ -26,7 +27,8 @@ def _to_residual(ctx, step, x, w, name):
     rows it is handed on unrun (ops.PendingProduct): the norm that follows runs it with the addition
     and its own preparation in the epilogue.  Otherwise it runs here, split sums left un-added."""
     ops = ctx.ops
-    if x.dtype == torch.bfloat16 and x.shape[0] <= ops.FUSED_NORM_MAX_ROWS and ops.gemm8_supported(x.shape[0], w.shape[0], w.shape[1]):
+    if (step.fold_norms and x.dtype == torch.bfloat16 and x.shape[0] <= ops.FUSED_NORM_MAX_ROWS
+            and ops.gemm8_supported(x.shape[0], w.shape[0], w.shape[1])):
         out = step.ws(name, (x.shape[0], w.shape[0]))
         return ops.PendingProduct(x, w, out, step.scratch(name, x.shape[0], w.shape[0], w.shape[1]))
     return _linear(ctx, step, x, w, name, keep_partial=True)
@@ -138,6 +140,12 @@ class GQAAttention(Mixer):
         super().__init__(params, prefix, ctx)
         p = params
         self.nh, self.nkv, self.hd = p["num_heads"], p["num_kv_heads"], p["head_dim"]
+        # refused where the model is built, not at the first step's launch
+        if self.hd <= 0 or self.hd % 8 or self.hd > 256:
+            raise ValueError(f"gqa_attention {prefix!r}: head_dim {self.hd} is not supported (the attention kernels take "
+                             f"multiples of 8 up to 256; num_heads {self.nh}, num_kv_heads {self.nkv})")
+        if self.nkv <= 0 or self.nh % self.nkv:
+            raise ValueError(f"gqa_attention {prefix!r}: num_heads {self.nh} is not a multiple of num_kv_heads {self.nkv}")
         self.scale = p.get("scale", 1.0 / math.sqrt(self.hd))
         self.window = p.get("window", 0)
         pos = p["position"]
@@ -155,6 +163,10 @@ class GQAAttention(Mixer):
 
     def cache_need(self):
         return KVCacheNeed(self.nkv, self.hd, self.window)
+
+    def flops(self, rows, attended=0):
+        # the two projections, and q.k and p.v over every (row, key) pair of every query head
+        return super().flops(rows) + 4.0 * attended * self.hd * self.nh
 
     def forward(self, step, h):
         ops = self.ctx.ops
@@ -220,6 +232,13 @@ class TokenEmbedding(Embedding):
         self.ctx.ops.embed(step.tokens, self.w["table"], out)
         return out
 
+    def bytes_read(self, rows):
+        table = self.w["table"]
+        return rows * table.shape[1] * table.element_size()      # only the rows of the step's tokens
+
+    def flops(self, rows, attended=0):
+        return 0.0
+
 
 @HEADS.register("linear_head")
 class LinearHead(Head):
@@ -239,7 +258,7 @@ class LinearHead(Head):
         return (self.prefix + "weight",) if self.params.get("tied") else ()
 
     def forward(self, step, h, out):
-        self.ctx.ops.gemm(h, self.w["table"], out)
+        self.ctx.ops.gemm(h, self.w["table"], out, tuning=step.tune_products)
         return out
 
 

@@ -7,7 +7,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, Registry
-from .base import BuildContext, KVCacheNeed, Mixer, ModelSpec, Part, StateNeed, as_tensor
+from .base import BuildContext, KVCacheNeed, ModelSpec, Part, StateNeed, as_tensor
 
 # registries by the names a block arrangement may use in ``part_registries``
 _REGISTRY_NAMES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "ffn": FEED_FORWARDS, "norm": NORMS,
@@ -40,7 +40,7 @@ def _registry_for(slot, block_class=None):
 class CacheGroupPlan:
     """Layers whose caches have the same shape and rule share one group (and one page table)."""
     need: object                 # KVCacheNeed or StateNeed
-    layers: List[str]            # names of the layers that own a cache in this group, in order
+    layers: List[Tuple[str, str]]   # (layer name, part name) of every cache owner in this group, in order
 
 
 class Model:
@@ -93,48 +93,109 @@ class Model:
         names += [type(b).__name__ for b in self.blocks if not b.capturable]
         return sorted(set(names))
 
+    # --------------------------------------------------------------------------------- cost
+    def _layer_parts_with_their_own(self) -> List[Part]:
+        out, todo = [], [p for parts in self.layer_parts for p in parts.values()]
+        while todo:
+            p = todo.pop()
+            out.append(p)
+            todo.extend(p.sub_parts())
+        return out
+
+    def step_bytes(self, rows: int, logit_rows: int) -> int:
+        """Bytes of weights a step of ``rows`` rows with ``logit_rows`` wanted rows has to read: every
+        part's own answer (Part.bytes_read), every tensor once however often the schedule runs a layer."""
+        parts = self._layer_parts_with_their_own() + [self.final_norm]
+        return (self.embedding.bytes_read(rows) + sum(p.bytes_read(rows) for p in parts)
+                + self.head.bytes_read(logit_rows))
+
+    def step_flops(self, rows: int, logit_rows: int, attended: int) -> float:
+        """Floating-point operations of such a step (Part.flops); a layer the schedule runs twice counts twice."""
+        total = self.head.flops(logit_rows)
+        for i in self.spec.schedule:
+            todo = list(self.layer_parts[i].values())
+            while todo:
+                p = todo.pop()
+                total += p.flops(rows, attended)
+                todo.extend(p.sub_parts())
+        return total
+
     def finish_binding(self):
         """Called by the loader after every part got its tensors: shares tied tables."""
         if self.spec.head.params.get("tied"):
             self.head.bind({"table": self.embedding.w["table"]})
 
     # -------------------------------------------------------------------------------- cache
+    @staticmethod
+    def _cache_need_of(part):
+        """What a part of a layer says it needs of the cache manager: anything with a ``cache_need``
+        method may own a cache (a Mixer is the usual case), whatever name the layer gives it."""
+        ask = getattr(part, "cache_need", None)
+        return ask() if callable(ask) else None
+
+    def _resolve_cache_source(self, layer, slot) -> Optional[Tuple[str, str]]:
+        """The (layer name, part name) whose cache the part ``slot`` of ``layer`` reads instead of owning
+        one, or None when it owns its own.  ``LayerSpec.cache_from`` is a string that holds for every
+        cache-using part of the layer, or a dict from part names to such strings; a string is a layer's
+        name (then the part of the same name there is meant) or ``layer.part``."""
+        src = layer.cache_from
+        if isinstance(src, dict):
+            src = src.get(slot)
+        if src is None:
+            return None
+        if src in self.layer_names:
+            return (src, slot)
+        head, _, tail = src.rpartition(".")
+        if head in self.layer_names:
+            return (head, tail)
+        raise ValueError(f"layer {layer.name}: cache_from {src!r} names no layer (a layer's name, or layer.part)")
+
     def _plan_cache_groups(self) -> List[CacheGroupPlan]:
         groups: List[CacheGroupPlan] = []
-        self._cache_of: Dict[str, Tuple[int, int]] = {}    # owner layer name -> (group, index)
+        self._cache_of: Dict[Tuple[str, str], Tuple[int, int]] = {}    # owner (layer, part) -> (group, index)
+        self._cache_source: Dict[Tuple[str, str], Tuple[str, str]] = {}  # reader (layer, part) -> owner (layer, part)
         for layer, parts in zip(self.spec.layers, self.layer_parts):
-            mixer = parts.get("mixer")
-            if mixer is None or layer.cache_from is not None:
-                continue
-            need = mixer.cache_need()
-            if need is None:
-                continue
-            if not isinstance(need, (KVCacheNeed, StateNeed)):
-                raise TypeError(f"layer {layer.name}: cache_need() must give a KVCacheNeed or a StateNeed")
-            for g, plan in enumerate(groups):
-                if plan.need == need:
-                    self._cache_of[layer.name] = (g, len(plan.layers))
-                    plan.layers.append(layer.name)
-                    break
-            else:
-                self._cache_of[layer.name] = (len(groups), 0)
-                groups.append(CacheGroupPlan(need, [layer.name]))
-        for layer in self.spec.layers:
-            if layer.cache_from is not None and layer.cache_from not in self._cache_of:
-                raise ValueError(f"layer {layer.name} reads the cache of {layer.cache_from!r}, which owns none")
+            if isinstance(layer.cache_from, dict):
+                unknown = sorted(set(layer.cache_from) - set(parts))
+                if unknown:
+                    raise ValueError(f"layer {layer.name}: cache_from names parts the layer does not have: {unknown}")
+            for slot, part in parts.items():
+                need = self._cache_need_of(part)
+                if need is None:
+                    continue
+                if not isinstance(need, (KVCacheNeed, StateNeed)):
+                    raise TypeError(f"layer {layer.name}, part {slot}: cache_need() must give a KVCacheNeed or a StateNeed")
+                source = self._resolve_cache_source(layer, slot)
+                if source is not None:
+                    self._cache_source[(layer.name, slot)] = source
+                    continue
+                key = (layer.name, slot)
+                for g, plan in enumerate(groups):
+                    if plan.need == need:
+                        self._cache_of[key] = (g, len(plan.layers))
+                        plan.layers.append(key)
+                        break
+                else:
+                    self._cache_of[key] = (len(groups), 0)
+                    groups.append(CacheGroupPlan(need, [key]))
+        for reader, owner in self._cache_source.items():
+            if owner not in self._cache_of:
+                raise ValueError(f"layer {reader[0]}, part {reader[1]} reads the cache of {owner[0]}.{owner[1]}, which owns none")
         return groups
 
     def attach_caches(self, storages):
-        """storages[g]: device storage of group g (see cache.storage)."""
+        """storages[g]: device storage of group g (see cache.storage).  Every part that reported a
+        cache need gets its place (or its owner's, read-only)."""
         for layer, parts in zip(self.spec.layers, self.layer_parts):
-            mixer = parts.get("mixer")
-            if not isinstance(mixer, Mixer):
-                continue
-            owner_name = layer.cache_from or layer.name
-            if owner_name not in self._cache_of:
-                continue
-            g, idx = self._cache_of[owner_name]
-            mixer.attach_cache(storages[g], idx, owner=layer.cache_from is None)
+            for slot, part in parts.items():
+                key = (layer.name, slot)
+                owner = self._cache_source.get(key, key)
+                if owner not in self._cache_of:
+                    if self._cache_need_of(part) is not None:
+                        raise RuntimeError(f"layer {layer.name}, part {slot} needs a cache that was not planned")
+                    continue
+                g, idx = self._cache_of[owner]
+                part.attach_cache(storages[g], idx, owner=owner == key)
 
     # --------------------------------------------------------------------------------- step
     def run_layers(self, step):

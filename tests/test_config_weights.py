@@ -63,9 +63,9 @@ def test_config_reads_its_keys_and_defaults():
     assert (c.q_dim, c.kv_dim, c.qkv_dim) == (64, 32, 128)
     assert c.num_parameters() == 125248
     assert LlamaConfig.from_dict(H.TINY_B).num_parameters() == 332448
-    minimal = dict(vocab_size=10, hidden_size=12, intermediate_size=20, num_hidden_layers=1, num_attention_heads=3)
+    minimal = dict(vocab_size=10, hidden_size=24, intermediate_size=20, num_hidden_layers=1, num_attention_heads=3)
     m = LlamaConfig.from_dict(minimal)
-    assert m.num_key_value_heads == 3 and m.head_dim == 4                  # defaults derived
+    assert m.num_key_value_heads == 3 and m.head_dim == 8                  # defaults derived
     assert m.rope_theta == 10000.0 and m.rms_norm_eps == 1e-5 and m.max_position_embeddings == 2048
     # head_dim may differ from hidden/heads
     assert LlamaConfig.from_dict(H.TINY_C).head_dim == 48
@@ -77,7 +77,10 @@ def test_config_reads_its_keys_and_defaults():
 
 @pytest.mark.parametrize("patch,fragment", [
     ({"num_key_value_heads": 3}, "multiple of num_key_value_heads"),
-    ({"head_dim": 15}, "even"),
+    ({"head_dim": 15}, "head_dim 15 is not supported"),
+    ({"head_dim": 12}, "multiples of 8 up to 256"),           # even, but not what the kernels take
+    ({"head_dim": 264}, "head_dim 264"),
+    ({"hidden_size": 40, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": None}, "head_dim 10"),       # derived
     ({"rope_scaling": {"type": "linear", "factor": 2.0}}, "rope_scaling"),
     ({"attention_bias": True}, "attention_bias"),
     ({"mlp_bias": True}, "mlp_bias"),
@@ -140,7 +143,7 @@ def test_llama_spec_is_data_over_registered_parts():
     assert spec.layers[0].parts["norm_ffn"].params == {"size": 96, "eps": 1e-6}
     assert spec.head.params["tied"] is True
     assert len(model.groups) == 1 and model.groups[0].need == KVCacheNeed(1, 32, 0)
-    assert model.groups[0].layers == ["layers.0", "layers.1", "layers.2"]
+    assert model.groups[0].layers == [("layers.0", "mixer"), ("layers.1", "mixer"), ("layers.2", "mixer")]
 
 
 def test_expected_tensor_names_follow_the_checkpoint_layout():

@@ -11,7 +11,7 @@ from kvcm_amd import architectures  # noqa: F401
 from kvcm_amd.config.engine_config import EngineConfig
 from kvcm_amd.config.model_config import LlamaConfig
 from kvcm_amd.engine.build import within_max_position
-from kvcm_amd.parts.base import Block, BuildContext, FeedForward, LayerSpec, Mixer, ModelSpec, PartSpec, StateNeed
+from kvcm_amd.parts.base import Block, BuildContext, FeedForward, KVCacheNeed, LayerSpec, Mixer, ModelSpec, PartSpec, StateNeed
 from kvcm_amd.parts.model import Model, _registry_for
 from kvcm_amd.registry import ARCHITECTURES, BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, Registry
 
@@ -146,3 +146,79 @@ def test_max_seq_len_is_cut_down_to_the_models_max_position(capsys):
     assert within_max_position(EngineConfig(max_seq_len=2048), 0).max_seq_len == 2048           # the architecture states none
     assert within_max_position(EngineConfig(max_seq_len=2048, beyond_max_position=True), 128).max_seq_len == 2048
     assert capsys.readouterr().err == ""
+
+
+# ------------------------------------------------------------- refusals where the model is built
+def test_attention_refuses_a_head_size_its_kernels_do_not_take_when_it_is_built():
+    """Not at the first step's launch: a configuration that reaches the part some other way than
+    through LlamaConfig (another architecture's description) is refused with the sizes named."""
+    from kvcm_amd.parts.llama_parts import GQAAttention
+    position = PartSpec("none", {})
+    for hd in (12, 20, 264):
+        with pytest.raises(ValueError, match=f"head_dim {hd} is not supported"):
+            GQAAttention({"num_heads": 4, "num_kv_heads": 2, "head_dim": hd, "position": position}, "a.", _ctx(64))
+    with pytest.raises(ValueError, match="not a multiple of num_kv_heads"):
+        GQAAttention({"num_heads": 4, "num_kv_heads": 3, "head_dim": 16, "position": position}, "a.", _ctx(64))
+    GQAAttention({"num_heads": 4, "num_kv_heads": 2, "head_dim": 8, "position": position}, "a.", _ctx(64))
+    GQAAttention({"num_heads": 4, "num_kv_heads": 2, "head_dim": 256, "position": position}, "a.", _ctx(64))
+
+
+# --------------------------------------------------------------- several cache owners in a layer
+def test_every_part_of_a_layer_that_needs_a_cache_gets_one_under_any_name():
+    """An attention beside a state mixer in one layer, under names the package does not know; a
+    second layer whose parts read the first layer's caches, one by a layer name, one by layer.part."""
+    class Keys(Mixer):
+        def cache_need(self):
+            return KVCacheNeed(2, 16, 0)
+
+    class State(Mixer):
+        def cache_need(self):
+            return StateNeed((4,), torch.float32)
+
+    class Gate(FeedForward):            # not a mixer, and it keeps something per request all the same
+        def cache_need(self):
+            return StateNeed((2,), torch.float32)
+
+    class Pair(Block):
+        part_registries = {"look": "mixer", "remember": "mixer", "gate": "feed_forward"}
+
+    MIXERS.register("keys_for_owner_test", Keys)
+    MIXERS.register("state_for_owner_test", State)
+    FEED_FORWARDS.register("gate_for_owner_test", Gate)
+    BLOCKS.register("pair_for_owner_test", Pair)
+
+    def layer(name, cache_from=None):
+        return LayerSpec(name, "pair_for_owner_test", {
+            "look": PartSpec("keys_for_owner_test", {}, name + ".k."), "remember": PartSpec("state_for_owner_test", {}, name + ".s."),
+            "gate": PartSpec("gate_for_owner_test", {}, name + ".g.")}, cache_from)
+
+    def model(layers):
+        spec = ModelSpec("Probe", 8, 11, PartSpec("token_embedding", {"vocab_size": 11}, "e."), tuple(layers), tuple(range(len(layers))),
+                         PartSpec("rmsnorm", {"size": 8, "eps": 1e-5}, "f."), PartSpec("linear_head", {"vocab_size": 11, "tied": True}, "h."))
+        return Model(spec, _ctx(8))
+
+    m = model([layer("a"), layer("b"), layer("c", {"look": "a", "remember": "b.remember"})])
+    assert [(type(g.need).__name__, g.layers) for g in m.groups] == [
+        ("KVCacheNeed", [("a", "look"), ("b", "look")]),
+        ("StateNeed", [("a", "remember"), ("b", "remember")]),
+        ("StateNeed", [("a", "gate"), ("b", "gate"), ("c", "gate")])]          # c's gate is not listed: it keeps its own
+
+    class Store:
+        def __init__(self, g):
+            self.group = g
+
+    m.attach_caches([Store(0), Store(1), Store(2)])
+    got = {(l.name, slot): (p.cache.group, p.cache_index, p.cache_owner)
+           for l, parts in zip(m.spec.layers, m.layer_parts) for slot, p in parts.items()}
+    assert got == {("a", "look"): (0, 0, True), ("a", "remember"): (1, 0, True), ("a", "gate"): (2, 0, True),
+                   ("b", "look"): (0, 1, True), ("b", "remember"): (1, 1, True), ("b", "gate"): (2, 1, True),
+                   ("c", "look"): (0, 0, False), ("c", "remember"): (1, 1, False), ("c", "gate"): (2, 2, True)}
+    # one string for the whole layer: every cache-using part reads the part of its own name there
+    whole = model([layer("a"), layer("r", "a")])
+    assert [g.layers for g in whole.groups] == [[("a", "look")], [("a", "remember")], [("a", "gate")]]
+    with pytest.raises(ValueError, match="names no layer"):
+        model([layer("a"), layer("r", "nowhere")])
+    with pytest.raises(ValueError, match="which owns none"):
+        model([layer("a"), layer("r", {"look": "a.remember2"})])
+    with pytest.raises(ValueError, match="does not have"):
+        model([layer("a"), layer("r", {"lok": "a"})])

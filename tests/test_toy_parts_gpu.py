@@ -224,7 +224,7 @@ def test_layer_list_may_repeat_a_layer_and_share_a_cache(tmp_path):
     ref = plain.rms_norm(x, t["norm.weight"], 1e-5) @ t["head.weight"].T
 
     rp = TraceReplayer(d, "float32", max_tokens=64)
-    assert len(rp.model.groups) == 1 and rp.model.groups[0].layers == ["first"]       # one cache, one owner
+    assert len(rp.model.groups) == 1 and rp.model.groups[0].layers == [("first", "mixer")]       # one cache, one owner
     assert rp.runner.storages[0].num_layers == 1
     a = rp.step({"step": 0, "entries": [{"id": "s", "tokens": toks[:20], "want": list(range(20))}], "end": []})
     b = rp.step({"step": 1, "entries": [{"id": "s", "tokens": toks[20:22], "want": [0, 1]}], "end": []})
@@ -374,7 +374,7 @@ def test_full_and_windowed_layers_routed_ffn_and_another_position_encoding(tmp_p
     rp = TraceReplayer(d, "float32", max_tokens=192)
     kinds = [(g.kind, g.window) for g in rp.core.groups]
     assert kinds == [("full", 0), ("window", 20), ("window", 9)]
-    assert [p.layers for p in rp.model.groups] == [["b0", "b3", "b4"], ["b1"], ["b2"]]
+    assert [[name for name, _ in p.layers] for p in rp.model.groups] == [["b0", "b3", "b4"], ["b1"], ["b2"]]
     steps = [[("a", 0, 30), ("b", 0, 2)], [("a", 30, 33), ("b", 2, 41)], [("a", 33, 34), ("c", 0, 17)],
              [("a", 34, 70), ("c", 17, 18)], [("c", 18, 57)], [("a", 70, 72)]] + [[("a", k, k + 1)] for k in range(72, 90)]
     got = {k: [] for k in reqs}
