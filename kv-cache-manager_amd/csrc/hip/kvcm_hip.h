@@ -139,6 +139,37 @@ int kvcm_program_add(void* program, const char* entry, const uint64_t* args, int
 int kvcm_program_size(void* program);
 int kvcm_program_run(void* program, hipStream_t stream);
 
+
+// ---- the engine's step loop (native_engine.hip) ---------------------------------------------------
+// The reference's Engine (src/engine/engine.h:29-52: add, step, idle, take_finished) as an object a native
+// caller holds.  It is made over a host core (scheduler, cache manager, batch builder: libkvcm_host.so,
+// reached through the addresses of nine of its C functions: kvcm_sched_schedule_summary,
+// kvcm_build_batch_from_plan_shaped, kvcm_sched_update_sampled, kvcm_last_error, kvcm_sched_add,
+// kvcm_sched_idle, kvcm_sched_collect_finished, kvcm_finished_get, kvcm_finished_clear), the pinned and the
+// device metadata buffers of the model's step function, the sampler's device and pinned id buffers, the
+// engine's limits and a stream of its own.  A step runs here from schedule to update when its canonical
+// shape has a recorded program (kvcm_program_*); the first step of a shape is recorded by whoever holds the
+// model's parts (they decide the launches), and handed over with kvcm_engine_register.
+void* kvcm_engine_new(void* core, const uint64_t* host_functions, int32_t* meta_host, int32_t* meta_dev, long long meta_ints,
+                      int32_t* sampled_dev, int32_t* sampled_host, int max_sampled, int num_groups, int block_size,
+                      int max_context, int max_tokens, int max_seqs, int max_logit_rows, int graph_rows, hipStream_t stream);
+void kvcm_engine_delete(void* engine);
+int kvcm_engine_add(void* engine, long long id, const int32_t* tokens, int n, int max_new_tokens, float temperature,
+                    uint64_t sampler_seed, double arrival);
+int kvcm_engine_idle(void* engine);
+// 1: a step ran; 2: nothing was planned; 0: the planned step's shape has no program yet (record and register it).
+int kvcm_engine_step(void* engine, double now, int64_t* info);
+int kvcm_engine_take_finished(void* engine);
+int kvcm_engine_finished_get(void* engine, int i, int64_t* info, double* times, int32_t* tokens, int cap);
+void kvcm_engine_finished_clear(void* engine);
+// The two halves of kvcm_engine_step, for callers that look at the plan first (out: 20 values, see
+// native_engine.hip) or keep the scheduler's update to themselves (defer_update: teacher forcing).
+int kvcm_engine_plan(void* engine, double now, int64_t* out);
+int kvcm_engine_last_plan(void* engine, int64_t* out);      // the same report again, the scheduler not run
+int kvcm_engine_run(void* engine, double now, int defer_update, int64_t* info);
+int kvcm_engine_register(void* engine, void* program, int as_graph);
+void kvcm_engine_stats(void* engine, int64_t* out);
+
 #ifdef __cplusplus
 }
 #endif

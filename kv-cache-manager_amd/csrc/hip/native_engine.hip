@@ -4,10 +4,12 @@
 // (step_program.hip); decode-shaped shapes are additionally captured into a HIP graph.
 //
 // The scheduler, the cache manager and the batch builder live in the host core, a library of its
-// own without any GPU dependency; this file reaches them through the addresses of four of its C
+// own without any GPU dependency; this file reaches them through the addresses of nine of its C
 // functions, handed over when the engine is made.  A step of a shape that has no program yet is
 // not run here: the caller runs it once through the model's parts while recording, and registers
-// the program.
+// the program.  Requests come in and finished ones go out through this object too (add, idle,
+// take_finished as in src/engine/engine.h:29-52), so that a native caller serves without the
+// interpreter for as long as the steps it meets have recorded shapes.
 //
 // Shapes.  A step is brought to a canonical shape so that programs are reused: its leading
 // single-token runs (the scheduler puts decoding requests first) are padded to a bucket D with
@@ -31,6 +33,12 @@ struct HostApi {
                                       int pad_leading, int32_t* out, int64_t cap, int32_t* desc);
   int (*update_sampled)(void* core, const int32_t* ids, int n, double now);
   const char* (*last_error)();
+  int (*add)(void* core, int64_t id, const int32_t* tokens, int n, int max_new_tokens, float temperature,
+             uint64_t sampler_seed, double arrival);
+  int (*idle)(void* core);
+  int (*collect_finished)(void* core);
+  int (*finished_get)(void* core, int i, int64_t* info, double* times, int32_t* tokens, int cap);
+  void (*finished_clear)(void* core);
 };
 
 struct Shape {
@@ -77,6 +85,8 @@ struct Engine {
   std::map<decltype(Shape().key()), std::unique_ptr<Recorded>> recorded;
   std::vector<int32_t> desc;
   int64_t summary[10] = {};
+  int64_t last_plan[20] = {};   // what kvcm_engine_plan last reported
+  int last_plan_entries = 0;
   Shape shape;   // of the current plan
   bool planned = false;
   long long steps_replayed = 0, steps_as_graph = 0;
@@ -124,7 +134,8 @@ bool canonical(const Engine& e, const int64_t* s, Shape& out) {
 extern "C" {
 
 // host_functions: addresses of kvcm_sched_schedule_summary, kvcm_build_batch_from_plan_shaped,
-// kvcm_sched_update_sampled and kvcm_last_error of the host core library, in this order.
+// kvcm_sched_update_sampled, kvcm_last_error, kvcm_sched_add, kvcm_sched_idle, kvcm_sched_collect_finished,
+// kvcm_finished_get and kvcm_finished_clear of the host core library, in this order.
 void* kvcm_engine_new(void* core, const uint64_t* host_functions, int32_t* meta_host, int32_t* meta_dev, long long meta_ints,
                       int32_t* sampled_dev, int32_t* sampled_host, int max_sampled, int num_groups, int block_size,
                       int max_context, int max_tokens, int max_seqs, int max_logit_rows, int graph_rows, hipStream_t stream) {
@@ -138,6 +149,16 @@ void* kvcm_engine_new(void* core, const uint64_t* host_functions, int32_t* meta_
   e->host.build_batch_from_plan_shaped = reinterpret_cast<decltype(HostApi::build_batch_from_plan_shaped)>(host_functions[1]);
   e->host.update_sampled = reinterpret_cast<decltype(HostApi::update_sampled)>(host_functions[2]);
   e->host.last_error = reinterpret_cast<decltype(HostApi::last_error)>(host_functions[3]);
+  e->host.add = reinterpret_cast<decltype(HostApi::add)>(host_functions[4]);
+  e->host.idle = reinterpret_cast<decltype(HostApi::idle)>(host_functions[5]);
+  e->host.collect_finished = reinterpret_cast<decltype(HostApi::collect_finished)>(host_functions[6]);
+  e->host.finished_get = reinterpret_cast<decltype(HostApi::finished_get)>(host_functions[7]);
+  e->host.finished_clear = reinterpret_cast<decltype(HostApi::finished_clear)>(host_functions[8]);
+  for (int i = 0; i < 9; ++i)
+    if (!host_functions[i]) {
+      kvcm::set_error("engine_new: host function %d is null", i);
+      return nullptr;
+    }
   e->meta_host = meta_host; e->meta_dev = meta_dev; e->meta_ints = meta_ints;
   e->sampled_dev = sampled_dev; e->sampled_host = sampled_host; e->max_sampled = max_sampled;
   e->block_size = block_size; e->max_context = max_context; e->max_tokens = max_tokens; e->max_seqs = max_seqs;
@@ -167,9 +188,8 @@ int kvcm_engine_plan(void* engine, double now, int64_t* out) {
   }
   std::memcpy(out, e->summary, sizeof(e->summary));
   for (int i = 10; i < 20; ++i) out[i] = 0;
-  if (n == 0) return 0;
   Shape sh;
-  if (canonical(*e, e->summary, sh)) {
+  if (n > 0 && canonical(*e, e->summary, sh)) {
     e->shape = sh;
     e->planned = true;
     out[10] = 1; out[11] = sh.rows; out[12] = sh.seqs; out[13] = sh.leading; out[14] = sh.logit_rows;
@@ -177,7 +197,18 @@ int kvcm_engine_plan(void* engine, double now, int64_t* out) {
     out[18] = e->recorded.count(sh.key()) ? 1 : 0;
     out[19] = (e->summary[4] != 0 && sh.rows <= e->graph_rows) ? 1 : 0;
   }
+  std::memcpy(e->last_plan, out, sizeof(e->last_plan));
+  e->last_plan_entries = n;
   return n;
+}
+
+// What the last kvcm_engine_plan (or kvcm_engine_step) reported, again, without running the scheduler:
+// for the caller that records a step kvcm_engine_step could not run.  Returns that plan's entries.
+int kvcm_engine_last_plan(void* engine, int64_t* out) {
+  auto* e = static_cast<Engine*>(engine);
+  std::memcpy(out, e->last_plan, sizeof(e->last_plan));
+  if (e->planned) out[18] = e->recorded.count(e->shape.key()) ? 1 : 0;
+  return e->last_plan_entries;
 }
 
 // Hands a recorded program for the current plan's shape to the engine (which owns it from now on).
@@ -253,6 +284,61 @@ int kvcm_engine_run(void* engine, double now, int defer_update, int64_t* info) {
   info[0] = e->desc[0]; info[1] = e->desc[1]; info[2] = sampling; info[3] = rec.exec ? 1 : 0;
   info[4] = static_cast<int64_t>(issued * 1e6);
   return 1;
+}
+
+// ---- requests in, finished requests out (src/engine/engine.h:29-52: add, idle, step, take_finished) ----
+// A request: its prompt's token ids, how many tokens it may generate, its sampling temperature (0:
+// greedy) and seed, and its arrival time on the caller's clock (the clock of `now` in plan / run / step).
+int kvcm_engine_add(void* engine, long long id, const int32_t* tokens, int n, int max_new_tokens, float temperature,
+                    uint64_t sampler_seed, double arrival) {
+  auto* e = static_cast<Engine*>(engine);
+  KVCM_REQUIRE(e != nullptr && tokens != nullptr && n > 0, "engine_add: a request needs at least one token");
+  if (e->host.add(e->core, id, tokens, n, max_new_tokens, temperature, sampler_seed, arrival) < 0) {
+    kvcm::set_error("engine_add: %s", e->host.last_error());
+    return -1;
+  }
+  return 0;
+}
+
+// 1 when no request waits or runs.
+int kvcm_engine_idle(void* engine) {
+  auto* e = static_cast<Engine*>(engine);
+  return e->host.idle(e->core);
+}
+
+// One step: plan, then run from the shape's recorded program.  Returns 1 when a step ran (info as
+// kvcm_engine_run fills it), 2 when the scheduler planned nothing (idle, or every waiting request
+// was rejected), 0 when the planned step's shape has no program yet: the plan stands, nothing ran,
+// and the caller has the step recorded (the model's parts decide its launches) and registers it
+// with kvcm_engine_register before it goes on.  Negative on failure.
+int kvcm_engine_step(void* engine, double now, int64_t* info) {
+  int64_t plan[20];
+  const int n = kvcm_engine_plan(engine, now, plan);
+  if (n < 0) return n;
+  if (n == 0) return 2;
+  return kvcm_engine_run(engine, now, 0, info);
+}
+
+// Moves what finished since the last call into a holding area and says how many requests wait there;
+// kvcm_engine_finished_get reads entry i of it (info: id, prompt length, tokens in all, preemptions,
+// prompt tokens computed, prompt tokens served from the prefix cache; times: arrival, admission, first
+// token, finish; tokens: prompt and generated ids, at most cap of them; returns the number of tokens),
+// kvcm_engine_finished_clear empties it.
+int kvcm_engine_take_finished(void* engine) {
+  auto* e = static_cast<Engine*>(engine);
+  const int n = e->host.collect_finished(e->core);
+  if (n < 0) kvcm::set_error("engine_take_finished: %s", e->host.last_error());
+  return n;
+}
+int kvcm_engine_finished_get(void* engine, int i, int64_t* info, double* times, int32_t* tokens, int cap) {
+  auto* e = static_cast<Engine*>(engine);
+  const int n = e->host.finished_get(e->core, i, info, times, tokens, cap);
+  if (n < 0) kvcm::set_error("engine_finished_get: %s", e->host.last_error());
+  return n;
+}
+void kvcm_engine_finished_clear(void* engine) {
+  auto* e = static_cast<Engine*>(engine);
+  e->host.finished_clear(e->core);
 }
 
 // out: programs recorded, of them graphs, steps replayed, of them as graphs.

@@ -104,17 +104,22 @@ class Engine:
         return done
 
     # ------------------------------------------------------------------------------- step
-    def step(self) -> StepInfo:
+    def step(self, planned_natively=False) -> StepInfo:
+        """One step.  ``planned_natively``: a native caller's kvcm_engine_step has run the scheduler already
+        and found no program for the plan's shape; the scheduler is not run again, the planned step runs
+        through the parts and is recorded."""
         info = StepInfo()
         t_start = self.now()
         rec, forcing = self.recorded, bool(self._forced)
+        if planned_natively and rec is None:
+            raise RuntimeError("step(planned_natively=True) needs recorded steps (a capturable model, use_programs or use_graphs)")
         ids = None
         if rec is None:
             n, info.prefill_tokens, info.decode_seqs, sampling, _ = self.core.schedule_summary(t_start)
             if n:
                 ids = self._step_direct(info, sampling)
         else:
-            n, info.prefill_tokens, info.decode_seqs, sampling = rec.plan(t_start)
+            n, info.prefill_tokens, info.decode_seqs, sampling = rec.plan(t_start, again=planned_natively)
             if n:
                 # (with use_programs off only the decode-shaped steps that become graphs are recorded)
                 wanted = rec.shape is not None and (self.config.use_programs or rec.wants_graph)

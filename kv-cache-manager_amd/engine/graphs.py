@@ -81,8 +81,9 @@ class RecordedSteps:
         lim = self.runner.limits
         self.stream = torch.cuda.Stream()          # default priority; every step of this engine runs on it
         names = ("kvcm_sched_schedule_summary", "kvcm_build_batch_from_plan_shaped", "kvcm_sched_update_sampled",
-                 "kvcm_last_error")
-        fns = (C.c_uint64 * 4)(*[self.core.native_function(n) for n in names])
+                 "kvcm_last_error", "kvcm_sched_add", "kvcm_sched_idle", "kvcm_sched_collect_finished",
+                 "kvcm_finished_get", "kvcm_finished_clear")
+        fns = (C.c_uint64 * len(names))(*[self.core.native_function(n) for n in names])
         s = self.sampler
         self._h = self.lib.kvcm_engine_new(
             self.core.handle, fns, self.runner._pinned.data_ptr(), self.runner.meta_dev.data_ptr(), self.runner.meta_dev.numel(),
@@ -104,11 +105,13 @@ class RecordedSteps:
             self._h = None
 
     # ------------------------------------------------------------------------------- one step
-    def plan(self, now: float):
+    def plan(self, now: float, again=False):
         """Runs the scheduler.  -> (entries, prompt tokens, decoding sequences, sampling entries); sets
-        ``shape`` (None when the plan fits no canonical shape), ``has_program`` and ``wants_graph``."""
+        ``shape`` (None when the plan fits no canonical shape), ``has_program`` and ``wants_graph``.
+        ``again``: the scheduler is not run; the plan a native caller's kvcm_engine_step made and could
+        not run (its shape has no program yet) is taken up."""
         o = self._out
-        n = self.lib.kvcm_engine_plan(self._h, float(now), o)
+        n = self.lib.kvcm_engine_last_plan(self._h, o) if again else self.lib.kvcm_engine_plan(self._h, float(now), o)
         if n < 0:
             raise self.ops.KernelError(self.lib.kvcm_hip_last_error().decode())
         self.core.plan_max_context, self.core.plan_rows, self.core.plan_leading, self.core.plan_max_run = o[5], o[6], o[7], o[8]
@@ -161,6 +164,13 @@ class RecordedSteps:
                 raise ops.KernelError(self.lib.kvcm_hip_last_error().decode())
             self.recorded_shapes[shape] = "graph" if self.wants_graph else "program"
         return layout, sampled
+
+    @property
+    def native_handle(self):
+        """The native engine object (csrc/hip/kvcm_hip.h: kvcm_engine_add / step / idle / take_finished):
+        what a native caller holds to serve requests without the interpreter once the shapes it meets
+        are recorded."""
+        return self._h
 
     # ---------------------------------------------------------------------------------- info
     def stats(self) -> dict:

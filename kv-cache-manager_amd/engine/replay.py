@@ -40,6 +40,12 @@ class TraceReplayer:
         self._next = 0
         self._computed = {}     # integer id -> tokens already run
 
+    def tables(self):
+        """Page tables of the live requests, per cache group: {request: [[page ids of group 0], ...]}
+        (-1: a page a window has passed and given back)."""
+        return {json.loads(key): [self.core.seq_table(sid, g) for g in range(self.core.num_groups)]
+                for key, sid in self._ids.items()}
+
     def _sid(self, ext, create):
         key = json.dumps(ext)
         if key not in self._ids:
@@ -96,7 +102,7 @@ class TraceReplayer:
         return logits
 
 
-def scheduled_replay(engine, requests, arrivals=None, max_steps=1 << 20):
+def scheduled_replay(engine, requests, arrivals=None, max_steps=1 << 20, on_step=None):
     """The second way to replay given tokens: through the engine's own scheduler.  Each request is
     (prompt tokens, continuation tokens): it is admitted, cut into portions, preempted and served
     from prefix hits as the engine's options decide, and wherever a token would be sampled the next
@@ -106,7 +112,8 @@ def scheduled_replay(engine, requests, arrivals=None, max_steps=1 << 20):
     The reference scores given tokens one whole sequence at a time (src/main_correct.cpp:194-222)
     and generates through add/step/take_finished (main_correct.cpp:61-80); this does both at once.
 
-    arrivals[i]: the step before which request i is added (default: all before the first step)."""
+    arrivals[i]: the step before which request i is added (default: all before the first step).
+    on_step(step number, StepInfo, {request index: engine id}): called after every step."""
     arrivals = list(arrivals) if arrivals is not None else [0] * len(requests)
     order = sorted(range(len(requests)), key=lambda i: (arrivals[i], i))
     ids, nxt, steps = {}, 0, 0
@@ -116,7 +123,9 @@ def scheduled_replay(engine, requests, arrivals=None, max_steps=1 << 20):
             prompt, continuation = requests[i]
             ids[i] = engine.add_request(prompt, len(continuation), forced=continuation)
             nxt += 1
-        engine.step()
+        info = engine.step()
+        if on_step is not None:
+            on_step(steps, info, ids)
         engine.take_finished()
         steps += 1
         if steps > max_steps:
@@ -124,9 +133,18 @@ def scheduled_replay(engine, requests, arrivals=None, max_steps=1 << 20):
     return [engine.forced_logits(ids[i]) for i in range(len(requests))]
 
 
+def _write_tables(out_dir, step, tables):
+    with open(os.path.join(out_dir, f"{step}.tables.json"), "w") as f:
+        json.dump({"step": step, "tables": [{"id": k, "groups": v} for k, v in tables.items()]}, f)
+
+
 def main(argv=None):
+    argv = list(sys.argv[1:] if argv is None else argv)
+    if "--scheduled" in argv:
+        return scheduled_main(argv)
     import argparse
-    ap = argparse.ArgumentParser(prog="trace_run", description="replay given token ids step by step and write logits")
+    ap = argparse.ArgumentParser(prog="trace_run", description="replay given token ids step by step and write logits "
+                                 "(--scheduled: through the engine's own scheduler, one request per input line)")
     ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
@@ -134,6 +152,8 @@ def main(argv=None):
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--attn", default="auto", choices=["v1", "v2", "auto"])
+    ap.add_argument("--dump-tables", action="store_true",
+                    help="also write <step>.tables.json: the live requests' page tables after the step, per cache group")
     args = ap.parse_args(argv)
     os.makedirs(args.out, exist_ok=True)
     print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
@@ -147,7 +167,13 @@ def main(argv=None):
             record = json.loads(line)
             if not isinstance(record, dict) or "step" not in record:
                 raise ReplayError('a step is a JSON object {"step": .., "entries": [..], "end": [..]}')
-            logits = rp.step(record)
+            if args.dump_tables:      # before the step's ``end`` gives the pages back
+                ended, record = record.get("end", []), dict(record, end=[])
+                logits = rp.step(record)
+                _write_tables(args.out, record["step"], rp.tables())
+                rp.step({"step": record["step"], "entries": [], "end": ended})
+            else:
+                logits = rp.step(record)
         except (ReplayError, ValueError, KeyError, TypeError) as e:      # what the input can get wrong: one line, exit 1
             what = f"missing key {e}" if isinstance(e, KeyError) else str(e)
             print(f"trace_run: input line {number}: {what}", file=sys.stderr, flush=True)
@@ -155,4 +181,82 @@ def main(argv=None):
         if logits is not None:
             np.ascontiguousarray(logits, dtype="<f4").tofile(os.path.join(args.out, f"{record['step']}.f32"))
         print(f"done {record['step']}", flush=True)
+    return 0
+
+
+def scheduled_main(argv):
+    """trace_run --scheduled: the second way to replay given tokens.  Standard input holds one request a
+    line, {"id": .., "prompt": [..], "forced": [..], "arrival": k}: the request joins before step k
+    (default 0) and goes through the engine's own scheduler under the engine flags the serving tools
+    take (--block-size, --num-blocks | --pool-gb, --max-seq-len, --max-num-seqs, --max-batched-tokens,
+    --prefill-chunk, --prefix, --watermark, --policy, --attn, --no-graphs, --no-programs, --no-fold-norms);
+    every token it would sample is replaced by the next of ``forced``.  <id>.f32 in --out receives the
+    logits those tokens were to be sampled from, [len(forced), vocab] little-endian 32-bit floats, and
+    ``done <id>`` is printed per request.  --dump-tables writes <step>.tables.json after every step.
+    The reference's pieces of this: generation through add / step / take_finished
+    (src/main_correct.cpp:61-80) and teacher-forced scoring of given tokens (main_correct.cpp:194-222)."""
+    from ..cli.args import Args
+    from ..cli.common import engine_config_from_args
+    from .engine import Engine
+    try:
+        a = Args([x for x in argv if x != "--scheduled"])
+        model, out = a.str("model", ""), a.str("out", "")
+        if not model or not out:
+            raise ValueError("give --model DIR and --out DIR")
+        dtype = a.str("dtype", "bfloat16")
+        dump = a.flag("dump-tables")
+        ec = engine_config_from_args(a, dtype=dtype, beyond_max_position=True)       # a trace's lengths are given
+        a.warn_unused()
+    except ValueError as e:
+        print(f"trace_run: {e}", file=sys.stderr, flush=True)
+        return 2
+    os.makedirs(out, exist_ok=True)
+    requests, names, arrivals = [], [], []
+    for number, line in enumerate(sys.stdin, 1):
+        line = line.strip()
+        if not line:
+            continue
+        try:
+            r = json.loads(line)
+            if not isinstance(r, dict):
+                raise ReplayError('a request is a JSON object {"id": .., "prompt": [..], "forced": [..], "arrival": k}')
+            prompt, forced = [int(t) for t in r["prompt"]], [int(t) for t in r["forced"]]
+            if not prompt or not forced:
+                raise ReplayError(f"request {r['id']!r}: prompt and forced need at least one token each")
+            if json.dumps(r["id"]) in {json.dumps(n) for n in names}:
+                raise ReplayError(f"request {r['id']!r} appears twice")
+            names.append(r["id"])
+            requests.append((prompt, forced))
+            arrivals.append(int(r.get("arrival", 0)))
+        except (ReplayError, ValueError, KeyError, TypeError) as e:
+            what = f"missing key {e}" if isinstance(e, KeyError) else str(e)
+            print(f"trace_run: input line {number}: {what}", file=sys.stderr, flush=True)
+            return 1
+    print(f"[trace_run] loading {model} ({dtype}); {len(requests)} requests through the scheduler", file=sys.stderr, flush=True)
+    eng = Engine(model, ec)
+    print("[trace_run] ready", file=sys.stderr, flush=True)
+
+    def after_step(step, info, ids):
+        if dump:
+            live = {}
+            for i, rid in ids.items():
+                try:
+                    groups = [eng.core.seq_table(rid, g) for g in range(eng.core.num_groups)]
+                except Exception:        # finished and collected already
+                    continue
+                if any(groups):          # a waiting or finished request holds no page
+                    live[json.dumps(names[i])] = groups
+            _write_tables(out, step, {json.loads(k): v for k, v in live.items()})
+
+    try:
+        logits = scheduled_replay(eng, requests, arrivals, on_step=after_step)
+    except (ReplayError, ValueError) as e:
+        print(f"trace_run: {e}", file=sys.stderr, flush=True)
+        return 1
+    for name, rows in zip(names, logits):
+        np.ascontiguousarray(rows, dtype="<f4").tofile(os.path.join(out, f"{name}.f32"))
+        print(f"done {name}", flush=True)
+    k = eng.core.counters()
+    print(f"[trace_run] {k['steps']} steps, {k['preemptions']} preemptions, {k['rejected']} rejected, "
+          f"{k['prefill_tokens_saved']} prompt tokens served from the prefix cache", file=sys.stderr, flush=True)
     return 0

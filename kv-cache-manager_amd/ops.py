@@ -92,8 +92,16 @@ def _declare(lib):
     lib.kvcm_engine_delete.restype = None
     lib.kvcm_engine_delete.argtypes = [vp]
     fn("kvcm_engine_plan", vp, C.c_double, C.POINTER(C.c_int64))
+    fn("kvcm_engine_last_plan", vp, C.POINTER(C.c_int64))
     fn("kvcm_engine_register", vp, vp, i)
     fn("kvcm_engine_run", vp, C.c_double, i, C.POINTER(C.c_int64))
+    fn("kvcm_engine_add", vp, C.c_longlong, C.POINTER(C.c_int32), i, i, f, C.c_uint64, C.c_double)
+    fn("kvcm_engine_idle", vp)
+    fn("kvcm_engine_step", vp, C.c_double, C.POINTER(C.c_int64))
+    fn("kvcm_engine_take_finished", vp)
+    fn("kvcm_engine_finished_get", vp, i, C.POINTER(C.c_int64), C.POINTER(C.c_double), C.POINTER(C.c_int32), i)
+    lib.kvcm_engine_finished_clear.restype = None
+    lib.kvcm_engine_finished_clear.argtypes = [vp]
     lib.kvcm_engine_stats.restype = None
     lib.kvcm_engine_stats.argtypes = [vp, C.POINTER(C.c_int64)]
 

@@ -58,3 +58,41 @@ def test_kvcorrect_passes_on_a_tiny_model(tmp_path):
     assert p.returncode == 0 and os.path.getsize(refs) > 16, p.stdout + p.stderr
     p = _run("kvcorrect", "--model", d, "--dtype", "bf16", "--max-seq-len", "128", "--num-blocks", "64", "--refs", refs)
     assert p.returncode == 0 and "8 reference prompts, 8 steps" in p.stdout, p.stdout + p.stderr
+
+
+def test_kvgen_prints_the_generated_ids_of_given_prompts(tmp_path):
+    """A model folder and prompts as token ids in, one line of generated ids per prompt out: the same ids
+    the plain implementation generates (up to near ties of its two best scores)."""
+    import plain_llama as plain
+    d = str(tmp_path / "m")
+    H.make_model_dir(d, H.CONFIGS["A"], H.WEIGHT_SEED["A"], torch.float32)
+    prompts = [[5, 17, 3, 200, 41], [9, 9, 1], [100]]
+    (tmp_path / "more.txt").write_text("7 8 9 10\n")
+    p = _run("kvgen", "--model", d, "--dtype", "fp32", "--prompt-ids", "5,17,3,200,41", "--prompt-ids=9,9,1", "--prompt-ids", "100",
+             "--prompts-file", str(tmp_path / "more.txt"), "--max-new-tokens", "6", "--max-seq-len", "64", "--num-blocks", "16",
+             "--dump-tables")
+    assert p.returncode == 0, p.stderr
+    lines = p.stdout.strip("\n").split("\n")
+    assert len(lines) == 4
+    pm = plain.load_model_dir(d, None)
+    for prompt, line in zip(prompts + [[7, 8, 9, 10]], lines):
+        got = [int(t) for t in line.split()]
+        want, margins = pm.generate(prompt, 6)
+        first = next((k for k in range(6) if got[k] != want[k]), None)
+        assert len(got) == 6 and (first is None or margins[first] < 1e-4), (prompt, got, want)
+    import json
+    dumps = [json.loads(l) for l in p.stderr.split("\n") if l.startswith("{")]
+    assert dumps and dumps[0]["step"] == 0 and set(dumps[0]["tables"]) == {"0", "1", "2", "3"}
+    assert all(len(g) == 1 and len(g[0]) == 1 for g in dumps[0]["tables"].values())       # one group, one page each
+    # temperature sampling with a seed is reproducible, and differs from greedy somewhere
+    a = _run("kvgen", "--model", d, "--dtype", "fp32", "--prompt-ids", "5,17,3", "--max-new-tokens", "12", "--temperature", "1.5",
+             "--sampler-seed", "7", "--max-seq-len", "64", "--num-blocks", "16")
+    b = _run("kvgen", "--model", d, "--dtype", "fp32", "--prompt-ids", "5,17,3", "--max-new-tokens", "12", "--temperature", "1.5",
+             "--sampler-seed", "7", "--max-seq-len", "64", "--num-blocks", "16")
+    g = _run("kvgen", "--model", d, "--dtype", "fp32", "--prompt-ids", "5,17,3", "--max-new-tokens", "12", "--max-seq-len", "64",
+             "--num-blocks", "16")
+    assert a.returncode == b.returncode == g.returncode == 0 and a.stdout == b.stdout != g.stdout
+    # what it cannot run: one line, exit code 1
+    bad = _run("kvgen", "--model", d, "--prompt-ids", "5,99999")
+    assert bad.returncode == 1 and "outside the vocabulary" in bad.stderr
+    assert _run("kvgen", "--model", d).returncode == 1

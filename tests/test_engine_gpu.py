@@ -48,6 +48,60 @@ def _same_up_to_near_ties(got, want, margins, tie):
 
 
 # ------------------------------------------------------------------------------ generation
+def _serve_natively(eng, prompts, new_tokens, first_id):
+    """Serves the prompts through the native engine object alone (csrc/hip/kvcm_hip.h: kvcm_engine_add /
+    step / idle / take_finished), as a C caller would; the interpreter is entered only for a step whose
+    shape has no program yet.  -> (generated ids per prompt, steps run natively, steps recorded)."""
+    import ctypes as C
+    lib, h = eng.runner.ops.lib(), eng.recorded.native_handle
+    for k, p in enumerate(prompts):
+        arr = (C.c_int32 * len(p))(*p)
+        assert lib.kvcm_engine_add(h, first_id + k, arr, len(p), new_tokens, 0.0, 0, eng.now()) == 0
+    info, native, recorded, out = (C.c_int64 * 8)(), 0, 0, {}
+    for _ in range(10000):
+        if lib.kvcm_engine_idle(h):
+            break
+        rc = lib.kvcm_engine_step(h, eng.now(), info)
+        assert rc >= 0, lib.kvcm_hip_last_error().decode()
+        if rc == 1:
+            native += 1
+        elif rc == 0:                       # a shape the engine has not met: the parts run it once, recording
+            eng.step(planned_natively=True)
+            recorded += 1
+        n = lib.kvcm_engine_take_finished(h)
+        meta, times = (C.c_int64 * 6)(), (C.c_double * 4)()
+        for i in range(n):
+            size = lib.kvcm_engine_finished_get(h, i, meta, times, None, 0)
+            toks = (C.c_int32 * size)()
+            assert lib.kvcm_engine_finished_get(h, i, meta, times, toks, size) == size
+            out[int(meta[0])] = list(toks)[int(meta[1]):]
+        lib.kvcm_engine_finished_clear(h)
+    assert lib.kvcm_engine_idle(h)
+    return [out[first_id + k] for k in range(len(prompts))], native, recorded
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_native_caller_serves_through_the_engine_object(models, dtype):
+    """Requests in, steps, finished requests out through the C entry points alone: once the step shapes of a
+    workload are recorded no step enters the interpreter, and the tokens are those of the Python engine; a
+    workload with shapes not met before falls back to recording, step by step, and goes on natively."""
+    d, pm = models[("A", dtype)]
+    prompts = _prompts(H.TINY_A, [7, 13, 5, 30], seed=21)
+    eng = _engine(d, dtype=dtype)
+    want = eng.generate(prompts, max_new_tokens=9)              # records the shapes this workload meets
+    got, native, recorded = _serve_natively(eng, prompts, 9, first_id=100)
+    assert got == want
+    assert recorded == 0 and native >= 9, (native, recorded)
+    assert eng.core.blocks_in_use() == 0
+    # other prompt lengths and another number of requests: new shapes turn up mid-run
+    others = _prompts(H.TINY_A, [40, 3, 3, 19, 8, 11], seed=22)
+    got, native, recorded = _serve_natively(eng, others, 6, first_id=200)
+    assert recorded >= 1 and native >= 1, (native, recorded)
+    fresh = _engine(d, dtype=dtype, use_graphs=False).generate(others, max_new_tokens=6)
+    assert got == fresh
+    assert eng.core.blocks_in_use() == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_config_a(models, dtype):
     """Tiny A: three requests with prompts of 7, 13 and 5 ids, 8 greedy tokens each."""

@@ -231,3 +231,45 @@ def test_trace_run_reports_bad_input_and_stops(setups, tmp_path):
                            capture_output=True, text=True, env=dict(os.environ, HOME=str(tmp_path)), timeout=300)
         assert p.returncode == 1 and p.stdout.strip() == "done 0", (p.returncode, p.stdout, p.stderr[-500:])
         assert "trace_run: input line 2" in p.stderr and message in p.stderr, p.stderr[-500:]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_scheduled_program(setups, dtype, tmp_path):
+    """bin/trace_run --scheduled: requests with given continuations go through the engine's own scheduler
+    (portions of 16, a pool small enough that pages are used again, arrivals at different steps) and
+    <id>.f32 holds the logits each given token was to be sampled from."""
+    d, reqs, ref, _ = setups[("A", dtype)]
+    names = ["r1", "r2", "r3", "r6", "r0"]
+    lines, cut = [], {}
+    for k, rid in enumerate(names):
+        toks = reqs[rid]
+        n = max(1, min(6, len(toks) - 1))
+        cut[rid] = len(toks) - n
+        lines.append(json.dumps({"id": rid, "prompt": toks[:cut[rid]], "forced": toks[cut[rid]:], "arrival": 2 * k}))
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--scheduled", "--model", d, "--dtype", dtype,
+                        "--out", str(out), "--max-seq-len", "128", "--num-blocks", "12", "--max-num-seqs", "3",
+                        "--prefill-chunk", "16", "--max-batched-tokens", "40", "--dump-tables"],
+                       input="\n".join(lines) + "\n", capture_output=True, text=True,
+                       env=dict(os.environ, HOME=str(tmp_path)), timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert p.stdout.split() == [w for rid in names for w in ("done", rid)]
+    V = H.TINY_A["vocab_size"]
+    tol = tolerance(dtype, ref)
+    for rid in names:
+        toks = reqs[rid]
+        got = np.fromfile(out / f"{rid}.f32", dtype="<f4").reshape(len(toks) - cut[rid], V)
+        want = ref[rid][cut[rid] - 1:len(toks) - 1]
+        err = np.abs(got.astype(np.float64) - want).max()
+        assert err <= tol, f"request {rid}: error {err:.3g}"
+    tables = json.loads((out / "0.tables.json").read_text())
+    assert tables["step"] == 0 and [t["id"] for t in tables["tables"]] == ["r1"]
+    # the plain replay writes the same kind of dump
+    steps = H.schedule_whole({"r1": reqs["r1"]})
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", dtype, "--out", str(out),
+                        "--max-tokens", "128", "--dump-tables"], input=json.dumps(steps[0]) + "\n", capture_output=True,
+                       text=True, env=dict(os.environ, HOME=str(tmp_path)), timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    dump = json.loads((out / "0.tables.json").read_text())
+    pages = -(-len(reqs["r1"]) // 16)
+    assert dump["tables"][0]["id"] == "r1" and len(dump["tables"][0]["groups"][0]) == pages
