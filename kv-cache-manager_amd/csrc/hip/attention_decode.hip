@@ -140,21 +140,31 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
   }
   __syncthreads();
 
-  // ---- pass 3: out[head][dim] += P[head][token] * V[token][dim]; P rounded to bfloat16 as the A operand
+  // ---- pass 3: out[head][dim] += P[head][token] * V[token][dim].  The probabilities stay 32-bit values as in the
+  // reference (src/cuda/paged_attention.cu:150-183); a matrix instruction takes bfloat16 operands, so p goes in as two
+  // of them, p rounded and what the rounding took away, and the product runs twice.
   f32x4 o[DT];
 #pragma unroll
   for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int j = 0; j < VSTEPS; ++j) {
-    Frag8 pf;
+    Frag8 pf, pl;
     pf.u = uint4{0u, 0u, 0u, 0u};
+    pl.u = uint4{0u, 0u, 0u, 0u};
     if (n16 < GROUP) {
       const float* pr = &scores[n16][(wave * VSTEPS + j) * 32 + kq * 8];
       const float4 a = *reinterpret_cast<const float4*>(pr), b = *reinterpret_cast<const float4*>(pr + 4);
-      pf.u.x = float_to_bf16_bits(a.x) | (uint32_t(float_to_bf16_bits(a.y)) << 16);
-      pf.u.y = float_to_bf16_bits(a.z) | (uint32_t(float_to_bf16_bits(a.w)) << 16);
-      pf.u.z = float_to_bf16_bits(b.x) | (uint32_t(float_to_bf16_bits(b.y)) << 16);
-      pf.u.w = float_to_bf16_bits(b.z) | (uint32_t(float_to_bf16_bits(b.w)) << 16);
+      const float p[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      uint32_t hi[4], lo[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t h0 = float_to_bf16_bits(p[2 * e]), h1 = float_to_bf16_bits(p[2 * e + 1]);
+        hi[e] = h0 | (h1 << 16);
+        lo[e] = uint32_t(float_to_bf16_bits(p[2 * e] - __uint_as_float(h0 << 16))) |
+                (uint32_t(float_to_bf16_bits(p[2 * e + 1] - __uint_as_float(h1 << 16))) << 16);
+      }
+      pf.u = uint4{hi[0], hi[1], hi[2], hi[3]};
+      pl.u = uint4{lo[0], lo[1], lo[2], lo[3]};
     }
     // value slots past the context's end hold stale data, which zero probabilities do not cancel if it is Inf or NaN
     const int left = end - (start + (wave * VSTEPS + j) * 32 + kq * 8);
@@ -163,6 +173,7 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
       Frag8 v = vf[j][d];
       if (left < 8) v.u = keep_first_bf16(v.u, left);
       o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, v.v, o[d], 0, 0, 0);
+      o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl.v, v.v, o[d], 0, 0, 0);
     }
   }
   // accumulator: column = dim n16 of tile d, rows = heads 4*kq..+3

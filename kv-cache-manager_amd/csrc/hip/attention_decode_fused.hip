@@ -284,16 +284,27 @@ __global__ void __launch_bounds__(WAVES* kWave, HD == 64 ? 8 / WAVES : 1)
     const float alpha = exp2f(m_run - m_new);
     m_run = m_new;
     float sum = 0.f;
-    FragF pf[2];
+    // The probabilities stay 32-bit values as in the reference (src/cuda/paged_attention.cu:150-183 multiplies
+    // 32-bit probabilities with the stored values): a matrix instruction takes bfloat16 operands, so p goes in
+    // as two of them, p rounded and what the rounding took away (16 bits of mantissa in all), and the product
+    // with the values runs twice.  The instruction count of a decode row does not show in its time.
+    FragF pf[2], pl[2];
 #pragma unroll
     for (int g = 0; g < 2; ++g) {
       float p[8];
+      uint32_t hi[4], lo[4];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         p[j] = s[g][j] > 0.5f * kFusNone ? exp2f(s[g][j] - m_new) : 0.f;
         sum += p[j];
       }
-      pf[g].u = uint4{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3]), pack2_bf16(p[4], p[5]), pack2_bf16(p[6], p[7])};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        hi[j] = pack2_bf16(p[2 * j], p[2 * j + 1]);
+        lo[j] = pack2_bf16(p[2 * j] - __uint_as_float(hi[j] << 16), p[2 * j + 1] - __uint_as_float(hi[j] & 0xffff0000u));
+      }
+      pf[g].u = uint4{hi[0], hi[1], hi[2], hi[3]};
+      pl[g].u = uint4{lo[0], lo[1], lo[2], lo[3]};
     }
     l_run = l_run * alpha + sum;
     // this lane's 8 value slots of a group that reach past the context hold stale data: cut them
@@ -308,6 +319,7 @@ __global__ void __launch_bounds__(WAVES* kWave, HD == 64 ? 8 / WAVES : 1)
         FragF vf = ch.v[g][d];
         if (cut) vf.u = keep_first_bf16(vf.u, ctx - (base + g * 32));
         o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[g].v, o[d], 0, 0, 0);
+        o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl[g].v, o[d], 0, 0, 0);
       }
     }
   };

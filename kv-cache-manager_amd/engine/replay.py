@@ -24,21 +24,70 @@ class ReplayError(RuntimeError):
 
 class TraceReplayer:
     def __init__(self, model_dir, dtype="bfloat16", max_tokens=4096, block_size=16, device="cuda:0",
-                 max_live=8, attn="auto", architecture=None, model_config=None, tensors=None):
+                 max_live=8, attn="auto", architecture=None, model_config=None, tensors=None, use_programs=False,
+                 fold_norms=True):
         """``model_dir``: a model folder; or None with architecture + model_config + tensors (checkpoint
-        names -> tensors in memory), as build_runner takes them."""
+        names -> tensors in memory), as build_runner takes them.  ``use_programs``: steps run as generation
+        runs them by default, from launch lists recorded once per step shape (a step's rows and wanted rows
+        padded to multiples of 64) and replayed with only the step's metadata changed; a model with a part
+        that is not capturable, and steps that want more rows than one head launch takes, run launch by
+        launch all the same."""
         pages = (max_tokens + block_size - 1) // block_size
         span = max(pages * block_size, block_size)
         ec = EngineConfig(policy="paged", block_size=block_size, max_seq_len=span, num_blocks=max(pages, 1),
                           watermark_blocks=0, max_num_seqs=max_live, max_batched_tokens=span,
-                          max_logit_rows=min(span, 1024), dtype=dtype, attn=attn, use_graphs=False,
-                          beyond_max_position=True)     # a trace's lengths are given, not generated
+                          max_logit_rows=min(-(-span // 64) * 64, 1024), dtype=dtype, attn=attn, use_graphs=False,
+                          fold_norms=fold_norms, beyond_max_position=True)     # a trace's lengths are given, not generated
         self.runner, self.core, self.model, self.model_config = build_runner(
             model_dir, ec, device=device, architecture=architecture, model_config=model_config, tensors=tensors)
         self.vocab_size = self.model.spec.vocab_size
         self._ids = {}          # external id -> integer id
         self._next = 0
         self._computed = {}     # integer id -> tokens already run
+        self.programs = {} if (use_programs and self.model.capturable) else None      # StepShape -> ops.StepProgram
+        self.steps_replayed = 0
+
+    # -------------------------------------------------------------------- recorded step shapes
+    def _shape_of(self, entries):
+        """The shape a step of these entries is recorded and replayed in, or None when it takes the
+        direct path (more wanted rows, or more rows, than the buffers of one launch hold)."""
+        from .graphs import StepShape
+        lim = self.runner.limits
+        rows = sum(e[2] for e in entries)
+        wanted = sum(len(e[3]) for e in entries)
+        leading = 0
+        while leading < len(entries) and entries[leading][2] == 1:
+            leading += 1
+        run = max(e[2] for e in entries)
+        shape = StepShape(rows=-(-rows // 64) * 64, seqs=len(entries), leading=leading, logit_rows=-(-wanted // 64) * 64,
+                          max_run=1 if run == 1 else -(-run // 64) * 64, context_bound=lim.max_context_len,
+                          table_stride=lim.max_blocks_per_seq)
+        if wanted == 0 or shape.rows > lim.max_tokens or shape.logit_rows > lim.max_logit_rows:
+            return None
+        return shape
+
+    def _run_recorded(self, entries, shape):
+        """One step in its recorded shape: the first of a shape runs through the parts while its launches
+        are recorded, later ones replay the list.  -> float32 logits [wanted, vocab] on the host."""
+        import torch
+        from .graphs import RecordedStepContext
+        runner, ops = self.runner, self.runner.ops
+        layout = self.core.build_batch(entries, runner.host_buffer(), pad_rows=shape.rows, pad_seqs=shape.seqs,
+                                       pad_logit_rows=shape.logit_rows, table_stride=shape.table_stride)
+        runner._check(layout)
+        runner.upload(layout)
+        program = self.programs.get(shape)
+        if program is None:
+            step = RecordedStepContext(runner, layout, shape)
+            program = ops.StepProgram()
+            with ops.recording(program):
+                logits = runner.model.forward(step)
+            self.programs[shape] = program
+        else:
+            program.run()
+            self.steps_replayed += 1
+            logits = runner.workspace.get("logits", (shape.logit_rows, self.vocab_size), torch.float32)
+        return logits[:layout.logit_rows].cpu().numpy()
 
     def tables(self):
         """Page tables of the live requests, per cache group: {request: [[page ids of group 0], ...]}
@@ -87,8 +136,12 @@ class TraceReplayer:
             entries.append((sid, self._computed[sid], len(tokens), want))
         logits = None
         if entries:
-            layout = self.core.build_batch(entries, self.runner.host_buffer())
-            logits = self.runner.execute_to_host(layout)
+            shape = self._shape_of(entries) if self.programs is not None else None
+            if shape is not None:
+                logits = self._run_recorded(entries, shape)
+            else:
+                layout = self.core.build_batch(entries, self.runner.host_buffer())
+                logits = self.runner.execute_to_host(layout)
             for sid, start, count, _ in entries:
                 self._computed[sid] = start + count
                 self.core.set_computed(sid, start + count)
@@ -152,12 +205,14 @@ def main(argv=None):
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--attn", default="auto", choices=["v1", "v2", "auto"])
+    ap.add_argument("--recorded", action="store_true",
+                    help="run steps as generation does by default: from launch lists recorded once per step shape")
     ap.add_argument("--dump-tables", action="store_true",
                     help="also write <step>.tables.json: the live requests' page tables after the step, per cache group")
     args = ap.parse_args(argv)
     os.makedirs(args.out, exist_ok=True)
     print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
-    rp = TraceReplayer(args.model, args.dtype, args.max_tokens, args.block_size, attn=args.attn)
+    rp = TraceReplayer(args.model, args.dtype, args.max_tokens, args.block_size, attn=args.attn, use_programs=args.recorded)
     print("[trace_run] ready", file=sys.stderr, flush=True)
     for number, line in enumerate(sys.stdin, 1):
         line = line.strip()

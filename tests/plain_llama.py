@@ -21,10 +21,11 @@ import numpy as np
 def round_bf16(a):
     """Round-to-nearest-even to bfloat16, returned as float64."""
     f = np.ascontiguousarray(np.asarray(a, dtype=np.float32))
-    u = f.view(np.uint32).astype(np.uint64)
-    lsb = (u >> 16) & 1
-    u = ((u + 0x7FFF + lsb) >> 16) << 16
-    return u.astype(np.uint32).view(np.float32).astype(np.float64).reshape(f.shape)
+    u = f.view(np.uint32)
+    # add half a step of the 16 bits that go (0x7FFF, and the kept part's last bit to break ties to even),
+    # then drop them; 32-bit unsigned arithmetic, which wraps only for NaN patterns
+    kept = (u + (np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1)))) & np.uint32(0xFFFF0000)
+    return kept.view(np.float32).astype(np.float64).reshape(f.shape)
 
 
 def _ident(a):
@@ -236,16 +237,49 @@ class PlainLlama:
         x = x + linear(swiglu(gu, r), t[p + "mlp.down_proj.weight"], r)
         return x
 
-    def logits(self, tokens):
-        """Logits [T, V] at every position of one whole sequence.  src/model/llama.cpp:84-128"""
+    def logits(self, tokens, rows=None):
+        """Logits [T, V] at every position of one whole sequence (``rows``: at these positions only;
+        the final norm and the head work row by row).  src/model/llama.cpp:84-128"""
         t, r = self.t, self.r16
         positions = np.arange(len(tokens))
         x = embedding(t["model.embed_tokens.weight"], tokens)
         for l in range(self.L):
             x = self.layer(l, x, positions)
+        if rows is not None:
+            x = x[np.asarray(rows, dtype=np.int64)]
         h = rms_norm(x, t["model.norm.weight"], self.eps, r)
         head = t["model.embed_tokens.weight"] if self.tied else t["lm_head.weight"]
         return np.asarray(h, dtype=np.float64) @ head.T  # logits stay wide
+
+    def logits_of_many(self, sequences, rows):
+        """``logits(sequences[i], rows[i])`` for many whole sequences at once, for tests with hundreds of
+        requests at real widths: everything that works row by row (norms, projections, rotation by each
+        row's own position, SwiGLU, head) runs on the sequences' rows stacked, attention runs per sequence
+        as in ``layer``.  Still no cache and no batching of attention; the same part functions."""
+        t, r = self.t, self.r16
+        lens = [len(s) for s in sequences]
+        starts = np.concatenate([[0], np.cumsum(lens)])
+        positions = np.concatenate([np.arange(n) for n in lens])
+        x = embedding(t["model.embed_tokens.weight"], np.concatenate([np.asarray(s, dtype=np.int64) for s in sequences]))
+        T = x.shape[0]
+        for l in range(self.L):
+            p = f"model.layers.{l}."
+            h = rms_norm(x, t[p + "input_layernorm.weight"], self.eps, r)
+            q = rotary(linear(h, t[p + "self_attn.q_proj.weight"], r).reshape(T, self.nh, self.hd), positions, self.theta, r)
+            k = rotary(linear(h, t[p + "self_attn.k_proj.weight"], r).reshape(T, self.nkv, self.hd), positions, self.theta, r)
+            v = linear(h, t[p + "self_attn.v_proj.weight"], r).reshape(T, self.nkv, self.hd)
+            a = np.concatenate([attention(q[lo:hi], k[lo:hi], v[lo:hi], positions[lo:hi], positions[lo:hi],
+                                          1.0 / math.sqrt(self.hd), 0, r) for lo, hi in zip(starts[:-1], starts[1:])])
+            x = x + linear(a.reshape(T, self.nh * self.hd), t[p + "self_attn.o_proj.weight"], r)
+            h = rms_norm(x, t[p + "post_attention_layernorm.weight"], self.eps, r)
+            gu = np.concatenate([linear(h, t[p + "mlp.gate_proj.weight"], r), linear(h, t[p + "mlp.up_proj.weight"], r)], axis=-1)
+            x = x + linear(swiglu(gu, r), t[p + "mlp.down_proj.weight"], r)
+        head = t["model.embed_tokens.weight"] if self.tied else t["lm_head.weight"]
+        out = []
+        for lo, want in zip(starts[:-1], rows):
+            h = rms_norm(x[lo + np.asarray(want, dtype=np.int64)], t["model.norm.weight"], self.eps, r)
+            out.append(np.asarray(h, dtype=np.float64) @ head.T)
+        return out
 
     def generate(self, prompt, max_new_tokens, temperature=0.0, seed=0, request_id=0):
         toks = list(prompt)

@@ -425,6 +425,19 @@ def test_plain_model_cuts_agree_with_itself():
     full = pm.logits(toks)
     np.testing.assert_allclose(pm.logits(toks[:11]), full[:11], atol=1e-12)
     assert full.shape == (20, 256)
+    np.testing.assert_allclose(pm.logits(toks, rows=[3, 19]), full[[3, 19]], atol=1e-12)
+    # many sequences stacked (the form the tests with hundreds of requests use) give each sequence's own logits
+    seqs = [toks, toks[:7], list(np.random.default_rng(4).integers(0, 256, size=33)), [5]]
+    rows = [[0, 19], [6], list(range(33)), [0]]
+    for r16 in (None, plain.round_bf16):
+        pm.r16 = r16
+        many = pm.logits_of_many(seqs, rows)
+        for s, want, got in zip(seqs, rows, many):
+            one = pm.logits(s, rows=want)
+            assert got.shape == one.shape
+            # (a product over stacked rows may add in another order: a rounding to 16 bits can fall the other way, rarely)
+            close = np.abs(got - one) <= (1e-11 if r16 is None else 1e-2 * np.abs(one).max())
+            assert close.all() and (np.abs(got - one) <= 1e-11).mean() > (0.999 if r16 is None else 0.9)
 
 
 def test_kvmodel_writes_a_folder_that_loads(tmp_path):

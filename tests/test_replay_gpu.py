@@ -273,3 +273,25 @@ def test_trace_run_scheduled_program(setups, dtype, tmp_path):
     dump = json.loads((out / "0.tables.json").read_text())
     pages = -(-len(reqs["r1"]) // 16)
     assert dump["tables"][0]["id"] == "r1" and len(dump["tables"][0]["groups"][0]) == pages
+
+
+@pytest.mark.parametrize("case", [("A", "float32"), ("B", "bfloat16"), ("D", "bfloat16"), ("D", "float32"), ("E", "bfloat16")])
+def test_replay_through_recorded_step_programs(setups, case):
+    """The same schedules with every step run the way generation runs it by default: from the launch list
+    recorded at the first step of its shape, replayed with nothing but the step's metadata changed.  Every
+    position's logits are fetched, so a value that a recording took from its own step instead of the
+    metadata (a position, a page, a row count) shows at the first replay that differs in it."""
+    from kvcm_amd.engine.replay import TraceReplayer
+    d, reqs, ref, _ = setups[case]
+    name, dtype = case
+    rp = TraceReplayer(d, dtype, max_tokens=H.tokens_needed(reqs), block_size=H.BLOCK_SIZE[name], use_programs=True)
+    assert rp.programs is not None
+    for steps in (H.schedule_portions(reqs), H.schedule_mixed(reqs, seed=3), H.schedule_tail_singly(reqs, 32)):
+        got = H.replay(rp, steps, reqs)
+        assert all(not np.isnan(g).any() for g in got.values())
+        bad = H.first_difference(got, ref, tolerance(dtype, ref))
+        assert bad is None, f"first wrong logits at request {bad[0]} position {bad[1]}: error {bad[2]:.3g}"
+        assert rp.core.blocks_in_use() == 0
+    assert rp.steps_replayed > 3 * len(rp.programs) > 0, (rp.steps_replayed, len(rp.programs))
+    shapes = set(rp.programs)
+    assert any(s.max_run > 1 and s.seqs > 1 for s in shapes) and any(s.max_run == 1 for s in shapes)
