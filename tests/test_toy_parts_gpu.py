@@ -520,3 +520,126 @@ def test_toy_norm_and_parallel_block_arrangement(tmp_path):
     b = rp.step({"step": 1, "entries": [{"id": "s", "tokens": toks[17:19], "want": [0, 1]}], "end": []})
     c = rp.step({"step": 2, "entries": [{"id": "s", "tokens": toks[19:], "want": list(range(22))}], "end": ["s"]})
     np.testing.assert_allclose(np.concatenate([a, b, c]), ref, atol=2e-4)
+
+
+# ----------------------------------------- two cache owners in one layer, under names of their own
+def test_a_layer_with_an_attention_and_a_state_mixer_side_by_side(tmp_path):
+    """A block arrangement defined here holds two parts that each keep something per request: an attention
+    over paged keys and values ("look") and the toy mixer with a state slot ("remember"); a second layer of
+    the same kind whose attention reads the first layer's pages.  Both get their caches from the model's
+    planner (one paged group, one state group), are stepped in portions beside other requests with pages
+    used again, and equal a plain toy."""
+    _register_toy()
+    from kvcm_amd.engine.replay import TraceReplayer
+    from kvcm_amd.parts.base import Block, LayerSpec, ModelSpec, PartSpec, as_tensor
+    from kvcm_amd.registry import ARCHITECTURES, BLOCKS, Architecture
+    from kvcm_amd.weights.random_init import write_model_dir
+
+    if "toy_two_memories" not in BLOCKS:
+        @BLOCKS.register("toy_two_memories")
+        class TwoMemories(Block):
+            """x += look(n(x)) + remember(n(x)); x += ffn(n2(x))."""
+            part_registries = {"look": "mixer", "remember": "mixer"}
+
+            def forward(self, step, x, pending):
+                h = step.ws("normed", (step.rows, x.shape[1]))
+                self.parts["norm_in"].forward(x, h, add=as_tensor(pending))
+                both = step.ws("both", (step.rows, x.shape[1]), torch.float32)
+                both.copy_(as_tensor(self.parts["look"].forward(step, h)).float())     # (the two mixers use one work buffer)
+                both += self.parts["remember"].forward(step, h).float()
+                self.parts["norm_ffn"].forward(x, h, add=both)
+                return as_tensor(self.parts["ffn"].forward(step, h))
+
+    @dataclass(frozen=True)
+    class Cfg:
+        vocab_size: int
+        width: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        inner: int
+        state_size: int
+        decay: float
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("vocab_size", "width", "heads", "kv_heads", "head_dim", "inner", "state_size",
+                                              "decay", "eps")})
+
+        def to_dict(self):
+            return asdict(self)
+
+    def spec(cfg):
+        def layer(name, prefix, cache_from=None):
+            attn = {"num_heads": cfg.heads, "num_kv_heads": cfg.kv_heads, "head_dim": cfg.head_dim, "scale": cfg.head_dim ** -0.5,
+                    "window": 0, "position": PartSpec("rotary", {"theta": 5000.0, "dim": cfg.head_dim})}
+            return LayerSpec(name, "toy_two_memories", {
+                "norm_in": PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, prefix + "n1."),
+                "look": PartSpec("gqa_attention", attn, prefix + "attn."),
+                "remember": PartSpec("toy_decay_state", {"state_size": cfg.state_size, "decay": cfg.decay}, prefix + "mix."),
+                "norm_ffn": PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, prefix + "n2."),
+                "ffn": PartSpec("swiglu", {"intermediate_size": cfg.inner}, prefix + "mlp.")}, cache_from)
+        # the second layer's attention reads the first layer's keys and values; its state mixer keeps a state of its own
+        layers = (layer("first", "l0."), layer("second", "l1.", {"look": "first.look"}))
+        return ModelSpec("ToyTwoMemoriesForCausalLM", cfg.width, cfg.vocab_size,
+                         PartSpec("token_embedding", {"vocab_size": cfg.vocab_size}, "emb."), layers, (0, 1),
+                         PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, "out_norm."),
+                         PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "tied": True}, "head."))
+
+    ARCHITECTURES.register("ToyTwoMemoriesForCausalLM", Architecture("ToyTwoMemoriesForCausalLM", Cfg, spec))
+    raw = dict(architectures=["ToyTwoMemoriesForCausalLM"], vocab_size=83, width=48, heads=4, kv_heads=2, head_dim=16, inner=64,
+               state_size=12, decay=0.8, eps=1e-5)
+    cfg = Cfg.from_dict(raw)
+    d = write_model_dir(str(tmp_path / "two"), "ToyTwoMemoriesForCausalLM", cfg, seed=21, dtype=torch.float32, std=0.25, norm_jitter=0.1)
+    t = plain.read_safetensors(os.path.join(d, "model.safetensors"))
+    # (the second layer's attention has no k and v projections of its own to read: the loader asks for them all the same,
+    # they are simply not used for the cache it reads)
+
+    def plain_logits(tokens):
+        n, pos = len(tokens), np.arange(len(tokens))
+        x = plain.embedding(t["emb.weight"], tokens)
+        first_kv = None
+        for l, p in enumerate(("l0.", "l1.")):
+            h = plain.rms_norm(x, t[p + "n1.weight"], raw["eps"])
+            q = plain.rotary(plain.linear(h, t[p + "attn.q_proj.weight"]).reshape(n, 4, 16), pos, 5000.0)
+            if l == 0:
+                k = plain.rotary(plain.linear(h, t[p + "attn.k_proj.weight"]).reshape(n, 2, 16), pos, 5000.0)
+                v = plain.linear(h, t[p + "attn.v_proj.weight"]).reshape(n, 2, 16)
+                first_kv = (k, v)
+            k, v = first_kv
+            a = plain.linear(plain.attention(q, k, v, pos, pos, 0.25).reshape(n, 64), t[p + "attn.o_proj.weight"])
+            u = h @ t[p + "mix.in_proj.weight"].T
+            state, b = np.zeros(raw["state_size"]), np.zeros_like(x)
+            for r in range(n):
+                state = raw["decay"] * state + u[r]
+                b[r] = t[p + "mix.out_proj.weight"] @ state
+            x = x + a + b
+            h = plain.rms_norm(x, t[p + "n2.weight"], raw["eps"])
+            gu = np.concatenate([plain.linear(h, t[p + "mlp.gate_proj.weight"]), plain.linear(h, t[p + "mlp.up_proj.weight"])], -1)
+            x = x + plain.linear(plain.swiglu(gu), t[p + "mlp.down_proj.weight"])
+        return plain.rms_norm(x, t["out_norm.weight"], raw["eps"]) @ t["emb.weight"].T
+
+    rng = np.random.default_rng(8)
+    reqs = {"x": rng.integers(0, 83, size=37).tolist(), "y": rng.integers(0, 83, size=9).tolist(),
+            "z": rng.integers(0, 83, size=50).tolist(), "w": rng.integers(0, 83, size=21).tolist()}
+    ref = {k: plain_logits(v) for k, v in reqs.items()}
+    rp = TraceReplayer(d, "float32", max_tokens=128, max_live=3)         # 8 pages: x, y and z fill them, w runs on pages given back
+    assert [(g.kind, [name for name, _ in plan.layers]) for g, plan in zip(rp.core.groups, rp.model.groups)] == \
+        [("full", ["first"]), ("state", ["first", "second"])]
+    assert [part for _, part in rp.model.groups[0].layers] == ["look"] and [part for _, part in rp.model.groups[1].layers] == ["remember"] * 2
+    steps = [[("x", 0, 11), ("y", 0, 2)], [("x", 11, 12), ("y", 2, 9), ("z", 0, 30)], [("x", 12, 37), ("z", 30, 31)],
+             [("z", 31, 50), ("w", 0, 3)], [("w", 3, 21)]]
+    got = {k: [] for k in reqs}
+    for k, entries in enumerate(steps):
+        ended = [rid for rid, lo, hi in entries if hi == len(reqs[rid])]
+        out = rp.step({"step": k, "entries": [{"id": rid, "tokens": reqs[rid][lo:hi], "want": list(range(hi - lo))}
+                                              for rid, lo, hi in entries], "end": ended})
+        row = 0
+        for rid, lo, hi in entries:
+            got[rid].append(out[row:row + hi - lo])
+            row += hi - lo
+    for rid in reqs:
+        err = np.abs(np.concatenate(got[rid]) - ref[rid]).max()
+        assert err < 2e-4, (rid, err)
+    assert rp.core.blocks_in_use(0) == 0 and rp.core.state_slots_free() == 3
