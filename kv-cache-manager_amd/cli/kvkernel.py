@@ -32,6 +32,14 @@ as one captured HIP graph: an empty kernel (1 and 1,024 workgroups), a kernel th
 before it wrote (64 KB, 1 MB), and kernels that stream 8, 23 and 46 MB each from a 2 GiB buffer (the
 sizes of a TinyLlama layer's weight matrices; consecutive launches read consecutive regions, so that
 the bytes come from HBM and not from a cache).
+
+  --sync [--layers 22]                           (not in the reference)
+
+times what it costs the workgroups of ONE launch to depend on one another, the alternative to a chain of
+launches: a barrier across the launch (data handed over by stores and loads past the caches, or by fences),
+split sums added up by the last workgroup of a tile to arrive against a second launch that adds them, and the
+bytes of a whole decode step (``--layers`` layers of five phases at TinyLlama sizes) read by one launch whose
+phases wait for one another against one launch per phase.  Every wait inside these kernels is bounded.
 """
 import sys
 
@@ -108,6 +116,83 @@ def _floor(nodes):
     return 0
 
 
+def _sync(layers):
+    """What it costs workgroups of one launch to depend on one another, against what launches cost:
+    a barrier across the launch, split sums added by the last workgroup to arrive or by a second launch,
+    and a decode step's bytes read by one launch of dependent phases or by one launch per phase."""
+    import torch
+    from .. import ops
+    ops.lib()
+    dev = torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    flags = torch.zeros(2, dtype=torch.int32, device=dev)
+    stream = torch.cuda.Stream()
+
+    def timed(fn, reps=20, calls=1):
+        """Microseconds per call of fn; ``calls`` calls in a row make one captured graph, which is replayed."""
+        with torch.cuda.stream(stream):
+            fn()
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for _ in range(calls):
+                    fn()
+            for _ in range(2):
+                graph.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            stream.synchronize()
+            e0.record()
+            for _ in range(reps):
+                graph.replay()
+            e1.record()
+            e1.synchronize()
+        return 1e3 * e0.elapsed_time(e1) / (reps * calls)
+
+    print(f"{cus} CUs.  A barrier across the workgroups of one launch (microseconds per barrier, from 1 and 101 rounds):")
+    data = torch.zeros(2 * 1024 * 256, dtype=torch.float32, device=dev)
+    counter = torch.zeros(1, dtype=torch.int32, device=dev)
+    print("%-44s %12s %12s" % ("data handed over by", "64 workgroups", f"{cus} workgroups"))
+    for fences, label in ((False, "stores and loads past the caches"), (True, "release and acquire fences")):
+        row = []
+        for G in (64, cus):
+            def go(rounds):
+                return timed(lambda: (counter.zero_(), ops.probe_barrier(data, counter, flags, G, rounds, fences=fences)))
+            row.append((go(101) - go(1)) / 100.0)
+        print("%-44s %12.2f %12.2f" % (label, *row))
+    print()
+    print("Split sums (4 KB per workgroup) added up by the tile's last workgroup to arrive, or by a second launch (microseconds):")
+    print("%8s %8s %16s %16s %16s" % ("splits", "tiles", "last arriver", "two launches", "an empty launch"))
+    partials = torch.zeros(8 * 512 * 1024, dtype=torch.float32, device=dev)
+    out = torch.zeros(512 * 1024, dtype=torch.float32, device=dev)
+    counters = torch.zeros(512, dtype=torch.int32, device=dev)
+    for S in (4, 8):
+        for tiles in (32, 128, 512):
+            a = timed(lambda: ops.probe_sums(partials, counters, out, S, tiles, True, flags), 20, calls=40)
+            b = timed(lambda: ops.probe_sums(partials, counters, out, S, tiles, False, flags), 20, calls=40)
+            c = timed(lambda: ops.probe_empty(tiles * S, 256), 20, calls=40)
+            print("%8d %8d %16.2f %16.2f %16.2f" % (S, tiles, a, b, c))
+    print()
+    # a layer of TinyLlama-1.1B sizes: QKV, the cache of eight requests, O, gate and up, down
+    H, I, QKV = 2048, 5632, 2560
+    phases = [QKV * H * 2, 1 << 20, H * H * 2, 2 * I * H * 2, H * I * 2]
+    layer = sum(phases)
+    weights = torch.zeros(4 * layer // 4, dtype=torch.int32, device=dev)
+    act = torch.zeros(8192, dtype=torch.float32, device=dev)
+    sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+    cnt = torch.zeros(layers * len(phases) * 17, dtype=torch.int32, device=dev)
+    total = layer * layers
+    print(f"A decode step's bytes ({layers} layers of {len(phases)} phases, {total / 1e9:.2f} GB) read by:")
+    one = timed(lambda: (cnt.zero_(), ops.probe_phases(weights, phases, layers, True, cus, cnt, act, flags, sink)), 10)
+    chain = timed(lambda: ops.probe_phases(weights, phases, layers, False, sink=sink), 10)
+    whole = timed(lambda: ops.probe_read(weights, sink, grid=2048), 10) * total / (4 * layer)
+    print("%-64s %10.1f us %8.2f TB/s" % (f"one launch of {cus} workgroups, a phase waits for the one before", one, total / one / 1e6))
+    print("%-64s %10.1f us %8.2f TB/s" % (f"one launch per phase ({layers * len(phases)} graph nodes)", chain, total / chain / 1e6))
+    print("%-64s %10.1f us %8.2f TB/s" % ("one launch that depends on nothing (scaled from four layers)", whole, total / whole / 1e6))
+    gave_up, wrong = [int(v) for v in flags.cpu()]
+    print(f"workgroups that gave up waiting: {gave_up}; wrong values read: {wrong}")
+    return 1 if (gave_up or wrong) else 0
+
+
 def _ints(s):
     return [int(x) for x in s.split(",") if x]
 
@@ -120,11 +205,14 @@ def main(argv=None):
     use_graph = a.flag("graph")
     prefill, seqs = a.str("prefill", ""), a.i32("seqs", 1)
     floor, nodes = a.flag("floor"), a.i32("nodes", 156)
+    sync, layers = a.flag("sync"), a.i32("layers", 22)
     a.warn_unused()
     if prefill:
         return _prefill(prefill, seqs, blocks, heads, kvh, hd, iters, out_csv, use_graph)
     if floor:
         return _floor(nodes)
+    if sync:
+        return _sync(layers)
 
     import torch
     from .. import ops

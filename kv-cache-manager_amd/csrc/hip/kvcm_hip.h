@@ -123,6 +123,14 @@ int kvcm_probe_empty(int grid, int block, hipStream_t s);
 int kvcm_probe_copy(const void* src, void* dst, long long bytes, int grid, hipStream_t s);      // moves 2 * bytes
 int kvcm_probe_read(const void* src, long long bytes, void* sink, int grid, hipStream_t s);
 int kvcm_probe_mfma(int iters, void* sink, int grid, hipStream_t s);   // grid * 4 waves * iters * 4 * 32768 flops
+// What it costs workgroups of one launch to depend on one another (every wait inside is bounded: flags[0] counts
+// workgroups that gave up, flags[1] wrong values): a barrier across G workgroups, `rounds` times; S sums per tile
+// added by the tile's last workgroup to arrive, or by a second launch; a step of layers x phases as one launch of
+// dependent phases, or as one launch per phase.
+int kvcm_probe_barrier(float* data, unsigned* counter, unsigned* flags, int G, int rounds, int spin_cap, int fences, hipStream_t s);
+int kvcm_probe_sums(float* partials, unsigned* counters, float* out, int S, int tiles, int last_arriver, unsigned* flags, hipStream_t s);
+int kvcm_probe_phases(const void* weights, const long long* phase_bytes, int phases, int layers, int persistent, int G,
+                      unsigned* counters, float* act, unsigned* flags, void* sink, int spin_cap, hipStream_t s);
 
 // ---- recorded steps ---------------------------------------------------------------------------
 // A step program is the list of launches of one step, recorded once for a step shape and replayed

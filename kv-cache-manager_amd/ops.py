@@ -73,6 +73,9 @@ def _declare(lib):
     fn("kvcm_probe_copy", vp, vp, C.c_longlong, i, vp)
     fn("kvcm_probe_read", vp, C.c_longlong, vp, i, vp)
     fn("kvcm_probe_mfma", i, vp, i, vp)
+    fn("kvcm_probe_barrier", vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_probe_sums", vp, vp, vp, i, i, i, vp, vp)
+    fn("kvcm_probe_phases", vp, C.POINTER(C.c_longlong), i, i, i, i, vp, vp, vp, vp, i, vp)
     fn("kvcm_fill_normal", vp, i, C.c_longlong, C.c_uint64, f, f, vp)
     fn("kvcm_fill_index", vp, C.c_longlong, C.c_uint64, i, vp)
     fn("kvcm_gemm8_supported", i, i, i)
@@ -784,6 +787,36 @@ def probe_mfma(iters, sink, grid=2048):
     _need(sink.numel() * sink.element_size() >= 1024, "probe_mfma needs a sink of 1 KiB")
     _check(lib().kvcm_probe_mfma(int(iters), _ptr(sink), int(grid), _stream()))
     return int(grid) * 4 * int(iters) * 4 * 32768
+
+
+def probe_barrier(data, counter, flags, workgroups, rounds, spin_cap=1 << 16, fences=False):
+    """``rounds`` barriers across ``workgroups`` workgroups of one launch (counter: zero before the launch)."""
+    _dev(data, counter, flags)
+    _need(data.numel() >= 2 * workgroups * 256 and data.dtype == torch.float32 and counter.dtype == flags.dtype == torch.int32
+          and flags.numel() >= 2, "probe_barrier: data float32 [2, workgroups, 256], counter int32 [1], flags int32 [2]")
+    _check(lib().kvcm_probe_barrier(_ptr(data), _ptr(counter), _ptr(flags), int(workgroups), int(rounds), int(spin_cap), int(fences), _stream()))
+
+
+def probe_sums(partials, counters, out, splits, tiles, last_arriver, flags):
+    _dev(partials, counters, out, flags)
+    _need(partials.numel() >= splits * tiles * 1024 and out.numel() >= tiles * 1024 and counters.numel() >= tiles
+          and partials.dtype == out.dtype == torch.float32 and counters.dtype == flags.dtype == torch.int32 and flags.numel() >= 2,
+          "probe_sums: partials float32 [tiles, splits, 1024], out float32 [tiles, 1024], counters int32 [tiles], flags int32 [2]")
+    _check(lib().kvcm_probe_sums(_ptr(partials), _ptr(counters), _ptr(out), int(splits), int(tiles), int(last_arriver), _ptr(flags), _stream()))
+
+
+def probe_phases(weights, phase_bytes, layers, persistent, workgroups=256, counters=None, act=None, flags=None, sink=None, spin_cap=1 << 18):
+    """A step of ``layers`` x len(phase_bytes) dependent phases over ``weights`` (four layers' bytes): as one
+    launch (``persistent``) or as one launch per phase."""
+    _dev(weights, counters, act, flags, sink)
+    layer = sum(phase_bytes)
+    _need(weights.numel() * weights.element_size() >= 4 * layer, "probe_phases: weights must hold four layers' bytes")
+    if persistent:
+        _need(counters is not None and counters.numel() >= layers * len(phase_bytes) * 17 and act is not None and act.numel() >= 8192
+              and flags is not None and flags.numel() >= 2, "probe_phases: counters int32 [layers * phases * 17], act float32 [8192], flags int32 [2]")
+    arr = (C.c_longlong * len(phase_bytes))(*[int(b) for b in phase_bytes])
+    _check(lib().kvcm_probe_phases(_ptr(weights), arr, len(phase_bytes), int(layers), int(bool(persistent)), int(workgroups), _ptr(counters),
+                                   _ptr(act), _ptr(flags), _ptr(sink), int(spin_cap), _stream()))
 
 
 def fill_normal(out, key, mean=0.0, std=1.0):
