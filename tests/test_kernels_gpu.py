@@ -1326,3 +1326,30 @@ def test_stale_values_past_a_context_do_not_reach_the_output(ops, nh, nkv, hd, B
     got = _run_prefill(ops, Pr, runs, nh, nkv, hd)
     assert np.isfinite(got).all()
     np.testing.assert_allclose(got, want, atol=1.5e-2, rtol=0)
+
+
+def test_dependencies_inside_one_launch_hand_data_over_and_every_wait_is_bounded(ops):
+    """The probe kernels behind ``kvkernel --sync``: workgroups of one launch meet at a counter and read what
+    the others left past the caches (no wrong value, nobody gives up); split sums added by the last
+    workgroup to arrive equal those a second launch adds; and a wait that does not end in time (the host
+    hands the kernel a spin limit of one poll) ends all the same: the workgroup raises the flag and leaves,
+    and so do those that then wait for it in vain."""
+    flags = torch.zeros(2, dtype=torch.int32, device=DEV)
+    data = torch.zeros(2 * 64 * 256, dtype=torch.float32, device=DEV)
+    counter = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ops.probe_barrier(data, counter, flags, 64, 5)
+    assert flags.tolist() == [0, 0] and int(counter) == 5 * 64
+    S, tiles = 8, 40
+    partials = torch.zeros(S * tiles * 1024, dtype=torch.float32, device=DEV)
+    counters = torch.zeros(tiles, dtype=torch.int32, device=DEV)
+    a, b = torch.zeros(tiles * 1024, dtype=torch.float32, device=DEV), torch.zeros(tiles * 1024, dtype=torch.float32, device=DEV)
+    ops.probe_sums(partials, counters, a, S, tiles, True, flags)
+    ops.probe_sums(partials, counters, a, S, tiles, True, flags)          # the counters were left at zero
+    ops.probe_sums(partials, counters, b, S, tiles, False, flags)
+    assert torch.equal(a, b) and float(a.view(tiles, 256, 4)[3, 0, 0]) == S * (S + 1) / 2 and flags.tolist() == [0, 0]
+    assert int(counters.abs().sum()) == 0
+    # one poll each: whoever polls before the last workgroup has counted gives up, the launch ends
+    counter.zero_()
+    ops.probe_barrier(data, counter, flags, 64, 3, spin_cap=1)
+    torch.cuda.synchronize()
+    assert 1 <= int(flags[0]) <= 64 and int(flags[1]) == 0
