@@ -152,18 +152,20 @@ __global__ void __launch_bounds__(kNormThreads)
     float a[VPT][4];
 #pragma unroll
     for (int k = 0; k < VPT; ++k) a[k][0] = a[k][1] = a[k][2] = a[k][3] = 0.f;
-    // four splits per trip, all their loads requested before the first sum; a split beyond S
-    // reads split S - 1 again and adds nothing, so the order of the sums is that of the splits
-    for (int s0 = 0; s0 < S; s0 += 4) {
-      float p[4][VPT][4];
+    // eight splits per trip (four for wide rows, whose pieces would not fit the registers), all their loads
+    // requested before the first sum; a split beyond S reads split S - 1 again and adds nothing, so the
+    // order of the sums is that of the splits
+    constexpr int TRIP = VPT <= 2 ? 8 : 4;
+    for (int s0 = 0; s0 < S; s0 += TRIP) {
+      float p[TRIP][VPT][4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < TRIP; ++j) {
         const int sj = s0 + j < S ? s0 + j : S - 1;
 #pragma unroll
         for (int k = 0; k < VPT; ++k) load4<float>(pr + sj * pstride + at[k], p[j][k]);
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < TRIP; ++j) {
         const bool keep = s0 + j < S;
 #pragma unroll
         for (int k = 0; k < VPT; ++k)
