@@ -148,14 +148,17 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
+    ap.add_argument("--prefill-tokens", type=int, default=2048,
+                    help="tokens of the prefill measurement (2,048 in the record; other lengths for sweeps)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N with N > 1 is not supported")
         sys.exit(2)
 
-    budget = max(4096, args.prompt_len + args.batch)     # a whole prompt fits a step beside the decoding requests
+    # a whole prompt fits a step beside the decoding requests
+    budget = max(4096, args.prompt_len + args.batch, args.prefill_tokens + 64)
     needed = args.prompt_len + args.warmup + args.steps + 24 + prompt_step_count(args.batch, args.prompt_len, budget)
-    limit = args.context_limit or max(2048, -(-needed // 64) * 64)
+    limit = args.context_limit or max(2048, -(-needed // 64) * 64, -(-args.prefill_tokens // 64) * 64)
     if needed > limit:
         print("bench.py: --prompt-len %d plus the decoded tokens does not fit --context-limit %d" % (args.prompt_len, limit))
         sys.exit(2)
@@ -194,7 +197,7 @@ def main():
     torch.cuda.empty_cache()
 
     def prefill_record():
-        T = 2048
+        T = args.prefill_tokens
         sec = prefill_run(eng, T, V)
         flops = eng.model.step_flops(T, 1, T * (T + 1) // 2)      # the parts' own count: products, and q.k and p.v
         return {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
