@@ -1,7 +1,8 @@
 """Decode and prefill throughput of the engine at TinyLlama-1.1B sizes with random weights.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512] [--layers L]
-                  [--sizes tinyllama-1.1b|llama-2-7b|llama-3-8b] [--context-limit 2048]
+                  [--sizes tinyllama-1.1b|llama-2-7b|llama-3-8b] [--context-limit 2048] [--prefill-tokens 2048]
+                  [--tune-products off|heuristic|all] [--no-points] [--only-prefill]
 
 A "step" is one decode step of the whole engine (schedule, batch metadata, upload, model step on
 the GPU, sampling, download, update).  W untimed steps, then exactly K timed steps between two

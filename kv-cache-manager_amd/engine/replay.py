@@ -278,7 +278,10 @@ def scheduled_main(argv):
             prompt, forced = [int(t) for t in r["prompt"]], [int(t) for t in r["forced"]]
             if not prompt or not forced:
                 raise ReplayError(f"request {r['id']!r}: prompt and forced need at least one token each")
-            if json.dumps(r["id"]) in {json.dumps(n) for n in names}:
+            if not isinstance(r["id"], (str, int)) or isinstance(r["id"], bool) or any(c in str(r["id"]) for c in "/\\\0") \
+                    or str(r["id"]) in ("", ".", ".."):
+                raise ReplayError(f"request id {r['id']!r} must be a number or a string that can name a file (<id>.f32)")
+            if str(r["id"]) in {str(n) for n in names}:
                 raise ReplayError(f"request {r['id']!r} appears twice")
             names.append(r["id"])
             requests.append((prompt, forced))

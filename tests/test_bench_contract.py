@@ -50,3 +50,21 @@ def test_one_json_line_with_the_agreed_fields():
     assert d["roofline"]["bound"] == "hbm" and d["roofline"]["peak"] == 8000.0
     assert abs(d["roofline"]["frac"] - d["roofline"]["achieved"] / d["roofline"]["peak"]) < 1e-3
     assert {"decode_b1", "decode_b64"} <= set(d["points"])
+
+
+def test_trace_run_scheduled_refuses_bad_requests_before_it_loads_a_model(tmp_path):
+    """The second mode of bin/trace_run reads every request first: what a line gets wrong ends the program with
+    one line on stderr and exit code 1, with no model loaded (so this runs without a GPU)."""
+    tool = os.path.join(ROOT, "bin", "trace_run")
+    good = '{"id": "a", "prompt": [1, 2], "forced": [3]}'
+    for lines, what in (([good, '{"id": "a", "prompt": [4], "forced": [5]}'], "appears twice"),
+                        (['{"id": "x/y", "prompt": [1], "forced": [2]}'], "name a file"),
+                        (['{"id": "b", "prompt": [], "forced": [2]}'], "at least one token"),
+                        (['{"id": "b", "prompt": [1]}'], "missing key"),
+                        (["not json"], "line 1")):
+        r = subprocess.run([sys.executable, tool, "--scheduled", "--model", str(tmp_path / "none"), "--out", str(tmp_path / "o")],
+                           input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=120)
+        assert r.returncode == 1 and "trace_run: input line" in r.stderr and what in r.stderr, (lines, r.returncode, r.stderr[-300:])
+        assert len([l for l in r.stderr.splitlines() if l.startswith("trace_run:")]) == 1
+    r = subprocess.run([sys.executable, tool, "--scheduled", "--out", str(tmp_path / "o")], input="", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "give --model DIR and --out DIR" in r.stderr
