@@ -127,7 +127,7 @@ int kvcm_probe_mfma(int iters, void* sink, int grid, hipStream_t s);   // grid *
 // workgroups that gave up, flags[1] wrong values): a barrier across G workgroups, `rounds` times; S sums per tile
 // added by the tile's last workgroup to arrive, or by a second launch; a step of layers x phases as one launch of
 // dependent phases, or as one launch per phase.
-int kvcm_probe_barrier(float* data, unsigned* counter, unsigned* flags, int G, int rounds, int spin_cap, int fences, hipStream_t s);
+int kvcm_probe_barrier(float* data, unsigned* counter, unsigned* flags, int G, int rounds, int spin_cap, int fences, int awaited, hipStream_t s);
 int kvcm_probe_sums(float* partials, unsigned* counters, float* out, int S, int tiles, int last_arriver, unsigned* flags, hipStream_t s);
 int kvcm_probe_phases(const void* weights, const long long* phase_bytes, int phases, int layers, int persistent, int G,
                       unsigned* counters, float* act, unsigned* flags, void* sink, int spin_cap, hipStream_t s);

@@ -70,8 +70,9 @@ __device__ __forceinline__ bool wait_for(const unsigned* counter, unsigned targe
 
 // `rounds` times: every workgroup writes 1 KB, all meet at a counter, every workgroup reads another one's 1 KB
 // and checks it (flags[1] counts wrong values).  fences: ordinary stores and loads with a release and an
-// acquire fence of agent scope instead of stores and loads past the caches.
-__global__ void __launch_bounds__(256) probe_barrier_kernel(float* data, unsigned* counter, unsigned* flags, int rounds, int spin_cap, int fences) {
+// acquire fence of agent scope instead of stores and loads past the caches.  awaited: how many arrivals a round
+// waits for (the launch's workgroups; a test of the bounded wait names one more, who never comes).
+__global__ void __launch_bounds__(256) probe_barrier_kernel(float* data, unsigned* counter, unsigned* flags, int rounds, int spin_cap, int fences, int awaited) {
   const int G = gridDim.x, b = blockIdx.x, t = threadIdx.x;
   __shared__ int ok;
   unsigned errors = 0;
@@ -87,7 +88,7 @@ __global__ void __launch_bounds__(256) probe_barrier_kernel(float* data, unsigne
     __syncthreads();
     if (t == 0) {
       __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      ok = wait_for(counter, unsigned(r + 1) * G, spin_cap);
+      ok = wait_for(counter, unsigned(r) * G + awaited, spin_cap);
     }
     __syncthreads();
     if (!ok) {
@@ -244,9 +245,10 @@ int kvcm_probe_mfma(int iters, void* sink, int grid, hipStream_t s) {
 // Every workgroup must be resident at once for a wait to end: the callers keep G at the number of CUs (a
 // workgroup that waits too long gives up, so a larger G costs time, not the GPU).  counter(s): zeroed by the
 // caller before every launch; flags: [0] workgroups that gave up, [1] wrong values read.
-int kvcm_probe_barrier(float* data, unsigned* counter, unsigned* flags, int G, int rounds, int spin_cap, int fences, hipStream_t s) {
-  KVCM_REQUIRE(data && counter && flags && G > 0 && G <= 1024 && rounds > 0 && spin_cap > 0, "probe_barrier: bad arguments");
-  probe_barrier_kernel<<<G, 256, 0, s>>>(data, counter, flags, rounds, spin_cap, fences);
+// awaited: arrivals a round waits for, G in every measurement; G + 1 makes every wait run into its limit.
+int kvcm_probe_barrier(float* data, unsigned* counter, unsigned* flags, int G, int rounds, int spin_cap, int fences, int awaited, hipStream_t s) {
+  KVCM_REQUIRE(data && counter && flags && G > 0 && G <= 1024 && rounds > 0 && spin_cap > 0 && awaited >= G, "probe_barrier: bad arguments");
+  probe_barrier_kernel<<<G, 256, 0, s>>>(data, counter, flags, rounds, spin_cap, fences, awaited);
   return launch_status("probe_barrier");
 }
 

@@ -73,7 +73,7 @@ def _declare(lib):
     fn("kvcm_probe_copy", vp, vp, C.c_longlong, i, vp)
     fn("kvcm_probe_read", vp, C.c_longlong, vp, i, vp)
     fn("kvcm_probe_mfma", i, vp, i, vp)
-    fn("kvcm_probe_barrier", vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_probe_barrier", vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_probe_sums", vp, vp, vp, i, i, i, vp, vp)
     fn("kvcm_probe_phases", vp, C.POINTER(C.c_longlong), i, i, i, i, vp, vp, vp, vp, i, vp)
     fn("kvcm_fill_normal", vp, i, C.c_longlong, C.c_uint64, f, f, vp)
@@ -789,12 +789,15 @@ def probe_mfma(iters, sink, grid=2048):
     return int(grid) * 4 * int(iters) * 4 * 32768
 
 
-def probe_barrier(data, counter, flags, workgroups, rounds, spin_cap=1 << 16, fences=False):
-    """``rounds`` barriers across ``workgroups`` workgroups of one launch (counter: zero before the launch)."""
+def probe_barrier(data, counter, flags, workgroups, rounds, spin_cap=1 << 16, fences=False, awaited=None):
+    """``rounds`` barriers across ``workgroups`` workgroups of one launch (counter: zero before the launch).
+    ``awaited``: the arrivals a barrier waits for, the launch's workgroups unless a test of the bounded wait
+    names one more (who never comes: every workgroup then polls ``spin_cap`` times, raises flags[0] and leaves)."""
     _dev(data, counter, flags)
     _need(data.numel() >= 2 * workgroups * 256 and data.dtype == torch.float32 and counter.dtype == flags.dtype == torch.int32
           and flags.numel() >= 2, "probe_barrier: data float32 [2, workgroups, 256], counter int32 [1], flags int32 [2]")
-    _check(lib().kvcm_probe_barrier(_ptr(data), _ptr(counter), _ptr(flags), int(workgroups), int(rounds), int(spin_cap), int(fences), _stream()))
+    _check(lib().kvcm_probe_barrier(_ptr(data), _ptr(counter), _ptr(flags), int(workgroups), int(rounds), int(spin_cap), int(fences),
+                                    int(workgroups if awaited is None else awaited), _stream()))
 
 
 def probe_sums(partials, counters, out, splits, tiles, last_arriver, flags):

@@ -1331,9 +1331,9 @@ def test_stale_values_past_a_context_do_not_reach_the_output(ops, nh, nkv, hd, B
 def test_dependencies_inside_one_launch_hand_data_over_and_every_wait_is_bounded(ops):
     """The probe kernels behind ``kvkernel --sync``: workgroups of one launch meet at a counter and read what
     the others left past the caches (no wrong value, nobody gives up); split sums added by the last
-    workgroup to arrive equal those a second launch adds; and a wait that does not end in time (the host
-    hands the kernel a spin limit of one poll) ends all the same: the workgroup raises the flag and leaves,
-    and so do those that then wait for it in vain."""
+    workgroup to arrive equal those a second launch adds; and a wait that cannot end (the host
+    names one arrival more than the launch has workgroups, and a limit of eight polls) ends all the same: every
+    workgroup raises the flag and leaves."""
     flags = torch.zeros(2, dtype=torch.int32, device=DEV)
     data = torch.zeros(2 * 64 * 256, dtype=torch.float32, device=DEV)
     counter = torch.zeros(1, dtype=torch.int32, device=DEV)
@@ -1348,8 +1348,9 @@ def test_dependencies_inside_one_launch_hand_data_over_and_every_wait_is_bounded
     ops.probe_sums(partials, counters, b, S, tiles, False, flags)
     assert torch.equal(a, b) and float(a.view(tiles, 256, 4)[3, 0, 0]) == S * (S + 1) / 2 and flags.tolist() == [0, 0]
     assert int(counters.abs().sum()) == 0
-    # one poll each: whoever polls before the last workgroup has counted gives up, the launch ends
+    # the barrier waits for one arrival more than the launch has workgroups: every workgroup polls eight
+    # times, gives up in the first round, and the launch ends
     counter.zero_()
-    ops.probe_barrier(data, counter, flags, 64, 3, spin_cap=1)
+    ops.probe_barrier(data, counter, flags, 64, 3, spin_cap=8, awaited=65)
     torch.cuda.synchronize()
-    assert 1 <= int(flags[0]) <= 64 and int(flags[1]) == 0
+    assert flags.tolist() == [64, 0] and int(counter) == 64
