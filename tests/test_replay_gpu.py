@@ -116,6 +116,32 @@ def test_first_tokens_of_a_sequence(setups, case):
     assert rp.core.blocks_in_use() == 0
 
 
+def _config(V, H_, I, L, nh, nkv, hd, theta=10000.0, eps=1e-5, tied=False):
+    return dict(architectures=["LlamaForCausalLM"], vocab_size=V, hidden_size=H_, intermediate_size=I, num_hidden_layers=L,
+                num_attention_heads=nh, num_key_value_heads=nkv, head_dim=hd, max_position_embeddings=1024, rope_theta=theta,
+                rms_norm_eps=eps, tie_word_embeddings=tied)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("raw", [_config(301, 72, 104, 2, 6, 2, 24, theta=5e5, eps=1e-6), _config(500, 80, 112, 1, 5, 1, 40, tied=True),
+                                 _config(259, 128, 192, 1, 4, 2, 120), _config(263, 96, 136, 1, 2, 2, 248)],
+                         ids=["hd24", "hd40", "hd120", "hd248"])
+def test_head_sizes_that_are_multiples_of_8_only(raw, dtype, tmp_path):
+    """The configuration takes head sizes in steps of 8 up to 256; those that are no multiple of 16 run through
+    the general kernels, whole and mixed with reused pages like every other size."""
+    from kvcm_amd.engine.replay import TraceReplayer
+    d = str(tmp_path)
+    H.make_model_dir(d, raw, 3, torch.float32 if dtype == "float32" else torch.bfloat16, sharpen=6.0)
+    reqs = H.requests_for(raw, [40, 3, 300, 17], seed=4)
+    ref, _ = H.plain_logits(d, reqs, bf16=dtype == "bfloat16")
+    rp = TraceReplayer(d, dtype, max_tokens=H.tokens_needed(reqs), block_size=16)
+    for steps in (H.schedule_whole(reqs), H.schedule_tail_singly(reqs, 32), H.schedule_mixed(reqs, seed=1)):
+        got = H.replay(rp, steps, reqs)
+        bad = H.first_difference(got, ref, tolerance(dtype, ref))
+        assert bad is None, f"first wrong logits at request {bad[0]} position {bad[1]}: error {bad[2]:.3g}"
+    assert rp.core.blocks_in_use() == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(setups, dtype):
     """One token at a time from the very first, across many page edges."""
