@@ -124,11 +124,13 @@ def _config(V, H_, I, L, nh, nkv, hd, theta=10000.0, eps=1e-5, tied=False):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("raw", [_config(301, 72, 104, 2, 6, 2, 24, theta=5e5, eps=1e-6), _config(500, 80, 112, 1, 5, 1, 40, tied=True),
-                                 _config(259, 128, 192, 1, 4, 2, 120), _config(263, 96, 136, 1, 2, 2, 248)],
-                         ids=["hd24", "hd40", "hd120", "hd248"])
-def test_head_sizes_that_are_multiples_of_8_only(raw, dtype, tmp_path):
+                                 _config(259, 128, 192, 1, 4, 2, 120), _config(263, 96, 136, 1, 2, 2, 248),
+                                 _config(101, 99, 77, 2, 3, 1, 32, theta=5e5, eps=1e-6)],
+                         ids=["hd24", "hd40", "hd120", "hd248", "odd_widths"])
+def test_head_sizes_in_steps_of_8_and_odd_widths(raw, dtype, tmp_path):
     """The configuration takes head sizes in steps of 8 up to 256; those that are no multiple of 16 run through
-    the general kernels, whole and mixed with reused pages like every other size."""
+    the general kernels, whole and mixed with reused pages like every other size.  So does a model whose width,
+    feed-forward width and vocabulary are odd numbers (no vector load fits a row)."""
     from kvcm_amd.engine.replay import TraceReplayer
     d = str(tmp_path)
     H.make_model_dir(d, raw, 3, torch.float32 if dtype == "float32" else torch.bfloat16, sharpen=6.0)
