@@ -165,40 +165,44 @@ __global__ void __launch_bounds__(256)
 
 // The same product for more than 16 rows.  With that many rows X is no longer small: every
 // 16-column tile needs all of it, and re-reading it from L2 per tile would cost several times the
-// weights' bytes.  Here a workgroup owns 64 columns (one 16-column tile per wave), up to 128 rows
-// and a slice of K, and its waves share X through LDS: per trip of DEPTH x 64 k the workgroup
-// stages X[rows][DEPTH * 64] once (double-buffered; the next trip's global loads are issued before
-// the current trip's products), every wave streams its own 16 weight rows from HBM and multiplies
-// them with the staged rows.  No reduction between waves; split-K partial sums as above.  More
-// than 128 rows run as row blocks of 128 (blockIdx.z), each streaming the weights again.
-// SWIGLU: a wave's tile is 8 gate + 8 up rows, the workgroup stores 32 activation columns.
+// weights' bytes.  Here a workgroup of NWV waves owns NWV column tiles (one 16-column tile per wave;
+// the last workgroup may have fewer tiles than waves), up to 128 rows and a slice of K, and its waves
+// share X through LDS: per trip of DEPTH x 64 k the workgroup stages X[rows][DEPTH * 64] once
+// (double-buffered; the next trip's global loads are issued before the current trip's products), every
+// wave streams its own 16 weight rows from HBM and multiplies them with the staged rows.  No reduction
+// between waves; split-K partial sums as above.  More than 128 rows run as row blocks of 128
+// (blockIdx.z), each streaming the weights again.
+// SWIGLU: a wave's tile is 8 gate + 8 up rows, it stores 8 activation columns.
 constexpr int kXPad = 8;    // bfloat16 of padding per staged row, so that rows spread over the banks
 constexpr int kRowBlock = 128;
 
-template <int MT, int DEPTH, class TO, bool SWIGLU>
-__global__ void __launch_bounds__(256)
+template <int MT, int DEPTH, class TO, bool SWIGLU, int NWV>
+__global__ void __launch_bounds__(NWV * kWave)
     gemm_rows_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ partials,
                      TO* __restrict__ out, int M, int N, int K, int ldx, int ldw, int ldo, int S) {
-  constexpr int RP = (MT * 16 + 63) / 64;   // staging passes: 256 threads move 64 rows x 64 k at a time
+  constexpr int kPassRows = NWV * kWave / 4;                      // rows the workgroup's threads stage at a time (x 64 k)
+  constexpr int RP = (MT * 16 + kPassRows - 1) / kPassRows;       // staging passes
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][DEPTH * kUnit + kXPad];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int r = lane % 16, kq = lane / 16;
   constexpr int kCols = SWIGLU ? 8 : 16;
-  const int c0 = blockIdx.x * (4 * kCols) + wave * kCols;   // this wave's first output column
+  const int c0 = blockIdx.x * (NWV * kCols) + wave * kCols;   // this wave's first output column
+  const bool col_on = c0 < N;                                   // the last workgroup may have fewer tiles than waves
   const int s = blockIdx.y;
   const int row_base = blockIdx.z * kRowBlock;
   const int units = K / kUnit;
   const int u_lo = int((long long)units * s / S), u_hi = int((long long)units * (s + 1) / S);
   const int trips = (u_hi - u_lo + DEPTH - 1) / DEPTH;
 
-  const uint16_t* wrow = W + size_t(SWIGLU ? (r < 8 ? c0 + r : N + c0 + r - 8) : c0 + r) * ldw + kq * 16;
-  // staging: thread -> (row tid / 4 + 64 p, 16 elements at (tid % 4) * 16 of every unit); rows
+  const int cw = col_on ? c0 : 0;   // a wave without a tile reads the first tile's rows and drops them
+  const uint16_t* wrow = W + size_t(SWIGLU ? (r < 8 ? cw + r : N + cw + r - 8) : cw + r) * ldw + kq * 16;
+  // staging: thread -> (row tid / 4 + kPassRows p, 16 elements at (tid % 4) * 16 of every unit); rows
   // beyond M read the block's first row and are dropped at the store
   const int srow = threadIdx.x / 4, sseg = (threadIdx.x % 4) * 16;
   const uint16_t* xsrc[RP];
 #pragma unroll
   for (int p = 0; p < RP; ++p) {
-    const int m = row_base + srow + 64 * p;
+    const int m = row_base + srow + kPassRows * p;
     xsrc[p] = X + size_t(m < M ? m : row_base) * ldx + sseg;
   }
 
@@ -236,11 +240,11 @@ __global__ void __launch_bounds__(256)
   auto stage = [&](int buf, const Trip& tr) {
 #pragma unroll
     for (int q = 0; q < RP; ++q) {
-      if (srow + 64 * q < MT * 16) {   // uniform per wave
+      if (srow + kPassRows * q < MT * 16) {   // uniform per wave
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
-          *reinterpret_cast<uint4*>(&xs[buf][srow + 64 * q][d * kUnit + sseg]) = tr.x[d][q][0];
-          *reinterpret_cast<uint4*>(&xs[buf][srow + 64 * q][d * kUnit + sseg + 8]) = tr.x[d][q][1];
+          *reinterpret_cast<uint4*>(&xs[buf][srow + kPassRows * q][d * kUnit + sseg]) = tr.x[d][q][0];
+          *reinterpret_cast<uint4*>(&xs[buf][srow + kPassRows * q][d * kUnit + sseg + 8]) = tr.x[d][q][1];
         }
       }
     }
@@ -278,6 +282,7 @@ __global__ void __launch_bounds__(256)
       multiply(1, j0 + DEPTH, tb);
     }
   }
+  if (!col_on) return;
   // accumulator: column = r of the wave's tile, rows = 4 kq + i
   if constexpr (SWIGLU) {
 #pragma unroll
@@ -328,14 +333,50 @@ constexpr int kMaxSharedRows = 512;
 static bool shares_rows(int M, int N) { return M > 16 && M <= kMaxSharedRows && N % 64 == 0; }
 static int row_blocks(int M) { return (M + kRowBlock - 1) / kRowBlock; }
 
+// Waves per workgroup (each takes one column tile) so that tiles x splits x row blocks make about one
+// workgroup per CU and none is left out: a CU has only so many requests for weights on their way, so what
+// a launch streams per microsecond grows with the CUs it covers, not with the waves on each (measured:
+// gate/up at TinyLlama sizes, 704 tiles, 32 rows: 176 workgroups of four waves 16.5 us, 235 of three
+// 13.2 us; at Llama-3-8B sizes, 1,792 tiles, 64 rows: 448 of four 63 us, 256 of seven 51 us).  One wave
+// more where that saves a staging pass (the workgroup's threads stage 16 rows per wave at a time: 64 rows
+// are two passes for three waves, one for four).
+constexpr int kRowsCUs = 256;
+static int rows_waves(long long units, int mt) {
+  const long long want = (units + kRowsCUs - 1) / kRowsCUs;
+  int w = want < 2 ? 2 : want > 8 ? 8 : static_cast<int>(want);
+  if (w < 8 && (mt + w) / (w + 1) < (mt + w - 1) / w) ++w;
+  return w;
+}
+static int rows_tiles_m(int M) { return M > kRowBlock ? kRowBlock / 16 : (M + 15) / 16; }
+
+// Splits of K of a plain shared-rows product: eight where there are few column tiles, or where K is long
+// against the rows (the partial sums, S*M*N floats that the next kernel reads, are small against the
+// weights then), else four; as long as every slice has a trip of its own and the partial sums stay below
+// the weights' bytes; halved while more than eight waves a workgroup would be needed to get down to one
+// workgroup per CU.  Measured at 17 to 128 rows over the projections of TinyLlama and Llama-3-8B sizes,
+// alone and in whole decode steps.
+static int rows_splits(int M, int N, int K) {
+  const long long tiles = static_cast<long long>(N / 16) * row_blocks(M);
+  const int units = K / kUnit;
+  if (tiles >= 4 * kRowsCUs) return 1;
+  int S = tiles <= 128 || (M > 48 && K >= 112 * M) ? 8 : 4;
+  const int trip = M <= 64 ? 4 : 2;   // units per trip (the launch's choice below)
+  const int cap = units / trip < K / (2 * M) ? units / trip : K / (2 * M);
+  while (S > 1 && S > cap) S >>= 1;
+  while (S > 1 && tiles * S > 8 * kRowsCUs) S >>= 1;
+  return S;
+}
+
 // One launch of the shared-rows kernel: MT row tiles per block (8 for every block when there are
 // several), two k-depths: four units per trip up to 64 rows, two beyond (LDS holds rows x depth).
-template <class TO, bool SWIGLU>
-static void launch_rows(dim3 grid, hipStream_t st, const uint16_t* x, const uint16_t* w, float* partials, TO* out, int M,
-                        int N, int K, int ldx, int ldw, int ldo, int S) {
-  const int mt = M > kRowBlock ? kRowBlock / 16 : (M + 15) / 16;
+template <class TO, bool SWIGLU, int NWV>
+static void launch_rows_n(hipStream_t st, const uint16_t* x, const uint16_t* w, float* partials, TO* out, int M, int N,
+                          int K, int ldx, int ldw, int ldo, int S) {
+  const int mt = rows_tiles_m(M);
+  const int tiles = N / (SWIGLU ? 8 : 16);
+  const dim3 grid((tiles + NWV - 1) / NWV, S, row_blocks(M));
 #define KVCM_ROWS(MT, DEPTH) \
-  gemm_rows_kernel<MT, DEPTH, TO, SWIGLU><<<grid, 256, 0, st>>>(x, w, partials, out, M, N, K, ldx, ldw, ldo, S)
+  gemm_rows_kernel<MT, DEPTH, TO, SWIGLU, NWV><<<grid, NWV * kWave, 0, st>>>(x, w, partials, out, M, N, K, ldx, ldw, ldo, S)
   switch (mt) {
     case 1: case 2: KVCM_ROWS(2, 4); break;
     case 3: KVCM_ROWS(3, 4); break;
@@ -346,30 +387,52 @@ static void launch_rows(dim3 grid, hipStream_t st, const uint16_t* x, const uint
 #undef KVCM_ROWS
 }
 
+// N: the result's width (SWIGLU: the activation's).  A 32-bit result (the head's logits, thousands of
+// tiles) keeps four waves.
+template <class TO, bool SWIGLU>
+static void launch_rows(hipStream_t st, const uint16_t* x, const uint16_t* w, float* partials, TO* out, int M, int N, int K,
+                        int ldx, int ldw, int ldo, int S) {
+  const long long units = static_cast<long long>(N / (SWIGLU ? 8 : 16)) * row_blocks(M) * S;
+  const int waves = sizeof(TO) == 4 || (S == 1 && !SWIGLU) ? 4 : rows_waves(units, rows_tiles_m(M));
+#define KVCM_WAVES(NWV) launch_rows_n<TO, SWIGLU, NWV>(st, x, w, partials, out, M, N, K, ldx, ldw, ldo, S)
+  if constexpr (sizeof(TO) == 4) {
+    KVCM_WAVES(4);
+  } else {
+    switch (waves) {
+      case 2: KVCM_WAVES(2); break;
+      case 3: KVCM_WAVES(3); break;
+      case 4: KVCM_WAVES(4); break;
+      case 5: KVCM_WAVES(5); break;
+      case 6: KVCM_WAVES(6); break;
+      case 7: KVCM_WAVES(7); break;
+      default: KVCM_WAVES(8); break;
+    }
+  }
+#undef KVCM_WAVES
+}
+
 
 extern "C" {
 
 // How many splits of K a launch of this shape uses (0: the shape is not supported by this kernel).
 int kvcm_gemm_skinny_splits(int M, int N, int K) {
   if (M <= 0 || N % 16 != 0 || K % kUnit != 0 || N <= 0 || K <= 0) return 0;
-  if (shares_rows(M, N)) {
-    // Measured over the projections of three model sizes at 32, 64 and 128 rows: powers of two
-    // only (a slice then is a whole number of trips), four slices, eight where there are few
-    // column groups; each slice at least one trip of four units, and partial sums (S*M*N floats)
-    // that stay below the weights' bytes.
-    const int cols = N / 64, units = K / kUnit;
-    if (cols * row_blocks(M) >= 256) return 1;
-    int S = cols <= 32 ? 8 : 4;
-    const int cap = units / 4 < K / (4 * M) ? units / 4 : K / (4 * M);
-    while (S > 1 && S > cap) S >>= 1;
-    return S;
-  }
+  if (shares_rows(M, N)) return rows_splits(M, N, K);
   if (M > 64) return 0;
   const int tiles = N / 16, units = K / kUnit;
   int S = (640 + tiles - 1) / tiles;           // aim at >= 640 workgroups (2.5 per CU) ...
   if (S >= 5) S = 8;                           // ... five to seven slices lose to eight in whole decode steps (measured)
   while (S > 1 && S > units / 2) --S;          // at least two units per slice
   return S;
+}
+
+// Waves per workgroup that the shared-rows kernel runs a bfloat16 product of this shape with (0: another
+// kernel takes the shape).  swiglu: N is the activation's width, S is 1.
+int kvcm_gemm_skinny_waves(int M, int N, int K, int S, int swiglu) {
+  if (swiglu ? !(M > 16 && M <= kMaxSharedRows && N % 32 == 0) : !shares_rows(M, N)) return 0;
+  if (K <= 0 || K % kUnit != 0 || S < 1) return 0;
+  if (!swiglu && S == 1) return 4;
+  return rows_waves(static_cast<long long>(N / (swiglu ? 8 : 16)) * row_blocks(M) * S, rows_tiles_m(M));
 }
 
 // S == 1: the result is stored to `out` (bfloat16 or float32).  S > 1: partial sums are written to
@@ -388,9 +451,8 @@ int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, i
   const uint16_t* w = static_cast<const uint16_t*>(W);
   const int mt = (M + 15) / 16;
   if (shares_rows(M, N)) {
-    const dim3 grid(N / 64, S, row_blocks(M));
-    if (out_dtype == kBF16) launch_rows<bf16_t, false>(grid, st, x, w, partials, static_cast<bf16_t*>(out), M, N, K, ldx, ldw, ldo, S);
-    else launch_rows<float, false>(grid, st, x, w, partials, static_cast<float*>(out), M, N, K, ldx, ldw, ldo, S);
+    if (out_dtype == kBF16) launch_rows<bf16_t, false>(st, x, w, partials, static_cast<bf16_t*>(out), M, N, K, ldx, ldw, ldo, S);
+    else launch_rows<float, false>(st, x, w, partials, static_cast<float*>(out), M, N, K, ldx, ldw, ldo, S);
     return launch_status("gemm_rows");
   }
   const dim3 grid(N / 16, S);
@@ -426,9 +488,8 @@ int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dty
   const uint16_t* w = static_cast<const uint16_t*>(W);
   const int mt = (M + 15) / 16;
   if (M > 16 && M <= kMaxSharedRows && I % 32 == 0) {
-    const dim3 grid(I / 32, 1, row_blocks(M));
-    if (out_dtype == kBF16) launch_rows<bf16_t, true>(grid, st, x, w, nullptr, static_cast<bf16_t*>(out), M, I, K, ldx, ldw, ldo, 1);
-    else launch_rows<float, true>(grid, st, x, w, nullptr, static_cast<float*>(out), M, I, K, ldx, ldw, ldo, 1);
+    if (out_dtype == kBF16) launch_rows<bf16_t, true>(st, x, w, nullptr, static_cast<bf16_t*>(out), M, I, K, ldx, ldw, ldo, 1);
+    else launch_rows<float, true>(st, x, w, nullptr, static_cast<float*>(out), M, I, K, ldx, ldw, ldo, 1);
     return launch_status("gemm_rows_swiglu");
   }
   const dim3 grid(I / 8, 1);

@@ -24,6 +24,9 @@ int kvcm_gemm_skinny_splits(int M, int N, int K);
 int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, int out_dtype, int M, int N, int K,
                      int ldx, int ldw, int ldo, int S, hipStream_t stream);
 int kvcm_reduce_store(const float* partials, void* out, int out_dtype, int M, int N, int ldo, int S, hipStream_t stream);
+// Waves per workgroup of the shared-rows kernel for a bfloat16 product of this shape (0: another kernel takes it):
+// chosen so that column tiles x splits x row blocks come to about one workgroup per CU.
+int kvcm_gemm_skinny_waves(int M, int N, int K, int S, int swiglu);
 
 // The same product, whole (split where kvcm_gemm_skinny_splits says so, partial sums added up in
 // split order, result in `out`), for callers that cannot allocate device memory: code under HIP

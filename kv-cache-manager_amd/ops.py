@@ -45,6 +45,7 @@ def _declare(lib):
     fn("kvcm_gemm_skinny_swiglu_supported", i, i, i)
     fn("kvcm_gemm_skinny_swiglu", vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_gemm_skinny_splits", i, i, i)
+    fn("kvcm_gemm_skinny_waves", i, i, i, i, i)
     fn("kvcm_gemm_skinny", vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp)
     fn("kvcm_reduce_store", vp, vp, i, i, i, i, i, vp)
     fn("kvcm_swiglu", vp, vp, i, i, i, vp)
@@ -465,6 +466,11 @@ def _library_workspace(device):
     if _library_ws is None:
         _library_ws = torch.empty(lib().kvcm_gemm_library_workspace_bytes(), dtype=torch.uint8, device=device)
     return _library_ws
+
+
+def skinny_waves(M, N, K, S=1, swiglu=False):
+    """Waves per workgroup the shared-rows kernel runs this bfloat16 product with (0: another kernel takes it)."""
+    return lib().kvcm_gemm_skinny_waves(int(M), int(N), int(K), int(S), int(bool(swiglu)))
 
 
 def skinny_splits(M, N, K):

@@ -594,6 +594,53 @@ def test_gemm_shared_rows_beyond_64_rows(ops, M, N, K):
         ops.LIBRARY_GEMM_MIN_ROWS = keep
 
 
+def test_gemm_shared_rows_with_every_number_of_waves(ops):
+    """The shared-rows kernel sizes its workgroups (two to eight waves, one column tile each) so that tiles x
+    splits come to about one workgroup per CU: every number of waves, plain and with the SwiGLU epilogue, with a
+    last workgroup that has fewer tiles than waves, against the 64-bit product."""
+    keep, ops.LIBRARY_GEMM_MIN_ROWS = ops.LIBRARY_GEMM_MIN_ROWS, 0
+    seen, seen_act = set(), set()
+    try:
+        for M, N, K in [(24, 1024, 2048), (32, 2560, 2048), (64, 2560, 2048), (64, 2560, 8192), (40, 6144, 1024),
+                        (100, 7168, 1024), (33, 8192, 1024), (96, 2048, 2048)]:
+            rng = np.random.default_rng(M + N + K)
+            x = _bf16_grid(rng.normal(size=(M, K)))
+            w = _bf16_grid(rng.normal(size=(N, K)) * 0.05)
+            ref = plain.linear(x, w)
+            S = ops.skinny_splits(M, N, K)
+            waves = ops.skinny_waves(M, N, K, S)
+            assert S > 1 and 2 <= waves <= 8 and (N // 16 + waves - 1) // waves * S <= 256 + 64, (M, N, K, S, waves)
+            seen.add(waves)
+            scratch = torch.zeros(S * M * N, dtype=torch.float32, device=DEV)
+            out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+            ops.gemm(_t(x, torch.bfloat16), _t(w, torch.bfloat16), out, scratch=scratch)
+            np.testing.assert_allclose(_np(out), ref, rtol=2 ** -7, atol=1e-3, err_msg=f"{M}x{N}x{K}: {waves} waves, {S} splits")
+        for M, I, K in [(32, 5120, 256), (64, 5632, 256), (24, 5632, 256), (48, 10240, 128), (96, 11008, 128),
+                        (17, 14336, 128), (128, 14336, 128), (20, 16384, 128)]:
+            rng = np.random.default_rng(M + I + K)
+            x = _bf16_grid(rng.normal(size=(M, K)))
+            w = _bf16_grid(rng.normal(size=(2 * I, K)) * 0.2)
+            waves = ops.skinny_waves(M, I, K, 1, swiglu=True)
+            assert 2 <= waves <= 8
+            seen_act.add(waves)
+            xt, wt = _t(x, torch.bfloat16), _t(w, torch.bfloat16)
+            act = torch.full((M, I), 7.0, dtype=torch.bfloat16, device=DEV)
+            assert ops.gemm_swiglu(xt, wt, act)
+            gu = torch.zeros(M, 2 * I, dtype=torch.bfloat16, device=DEV)
+            ops.gemm(xt, wt, gu)                                 # unsplit: no scratch given
+            want = torch.zeros_like(act)
+            ops.swiglu(gu, want)
+            a, b = _np(act), _np(want)
+            # the two launches walk K from different starting points: a sum may round to the neighbouring bfloat16
+            # (2^-7 relative), in the gate, in the up value, or in both, and SiLU below zero multiplies a step of
+            # its argument by up to four
+            assert np.mean(a == b) > 0.98, f"{M}x{I}x{K}: {waves} waves"
+            np.testing.assert_allclose(a, b, rtol=2 ** -5, atol=2e-3, err_msg=f"{M}x{I}x{K}: {waves} waves")
+    finally:
+        ops.LIBRARY_GEMM_MIN_ROWS = keep
+    assert seen == {2, 3, 4, 5, 6, 7, 8} and seen_act >= {3, 4, 5, 6, 7, 8}, (seen, seen_act)
+
+
 @pytest.mark.parametrize("mode", ["off", "heuristic", "all"])
 @pytest.mark.parametrize("M,N,K", [(96, 192, 320), (200, 2560, 512), (333, 328, 136)])
 def test_library_product_with_each_choice_of_algorithm(ops, mode, M, N, K):
