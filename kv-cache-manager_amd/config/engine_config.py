@@ -25,9 +25,10 @@ class EngineConfig:
     use_graphs: bool = True          # replay decode-only steps from captured HIP graphs (models whose parts are all capturable)
     use_programs: bool = True        # replay other step shapes from natively recorded launch lists (same condition)
     beyond_max_position: bool = False  # False: max_seq_len is cut down to the model's max_position_embeddings (with a notice)
-    fold_norms: bool = True            # bfloat16 decode steps of up to 16 rows fold their RMS norms into the products around
-                                       # them (two roundings at other places than the reference's, same size); False: every
-                                       # norm is a launch of its own and rounds exactly where the reference does
+    fold_norms: bool = True            # bfloat16 decode steps of a few rows (up to 8; fewer for wide models, where it stops
+                                       # paying earlier) fold their RMS norms into the products around them (two roundings at
+                                       # other places than the reference's, same size); False: every norm is a launch of its
+                                       # own and rounds exactly where the reference does
     tune_products: str = "off"         # which library algorithm a many-row product runs: "off" the library's first choice,
                                        # "heuristic" its choices timed at a shape's first use (tens of milliseconds per shape,
                                        # about 5 % of the product's time afterwards), "all" every algorithm (seconds per shape)

@@ -1,4 +1,4 @@
-// Products for decode steps of at most 16 rows, Y[M,N] = X[M,K] * W[N,K]^T (bfloat16), made so that a
+// Products for decode steps of at most 8 rows, Y[M,N] = X[M,K] * W[N,K]^T (bfloat16), made so that a
 // layer needs no launch of its own for its two RMS norms.  The reference runs norm, product,
 // residual add as separate kernels (src/model/llama.cpp:104-124, src/cuda/kernels.cu:34-49,84-88);
 // at these sizes a launch costs more than the bytes it moves, so here the norm is split in two and
@@ -24,10 +24,10 @@
 // asks for all its weight bytes of a trip at once (32 contiguous bytes per row and unit, four lanes
 // one 128-byte line), two trips in flight.  The waves' sums meet in LDS in a fixed order.
 //
-// 9 to 16 rows (gemm16_kernel): the same folding, without the trick of the two halves: a matrix
-// instruction's 16 operand rows are the 16 batch rows and 16 output columns, a workgroup owns 16 columns
-// per row group, its four waves a quarter of K each, and all 256 threads finish one element of the
-// 16 x 16 result.  Sums of squares are still left per 8-column tile, so both kernels read each other's.
+// More rows than 8 go through the shared-rows product with norms of their own (gemm_skinny.hip): every
+// workgroup here reads all of X, M x K per 8 or 16 output columns, from L2, which at 8 rows is as many
+// bytes as the weights themselves (a 16-row variant of this kernel lost to the shared-rows path at every
+// size measured: TinyLlama sizes batch 16 1.26 -> 1.17 ms, Llama-3-8B sizes 4.82 -> 4.05 ms).
 #include "common.h"
 #include "kvcm_hip.h"
 
@@ -236,162 +236,6 @@ __global__ void __launch_bounds__(NW * kWave) gemm8_kernel(const Gemm8Args a) {
   }
 }
 
-// ---- 9 to 16 rows ---------------------------------------------------------------------------
-constexpr int kCols16 = 16;   // output columns per row group of the 16-row kernel
-
-template <int RG, int UT>
-struct Trip16 {
-  Frag w[RG][UT][2];
-  Frag x[UT][2];
-};
-
-template <int RG, int UT, bool SCALED, int EPI, class TO>
-__global__ void __launch_bounds__(4 * kWave) gemm16_kernel(const Gemm8Args a) {
-  constexpr int NW = 4, kRowsPerWave = 16 / NW;
-  __shared__ f32x4 red[NW][RG][kWave];
-  __shared__ float rstd_s[16];
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int r = lane % 16, kq = lane / 16;
-  const int n0 = blockIdx.x * (kCols16 * RG);   // kSwiglu: N is the width of the result, RG == 2 means gate and up
-  const int units = a.K / kUnit;
-  const int u_lo = units * wave / NW, u_hi = units * (wave + 1) / NW;   // this wave's slice of K
-  const int cnt = u_hi - u_lo;
-
-  const uint16_t* wrow[RG];
-#pragma unroll
-  for (int g = 0; g < RG; ++g) {
-    const int row = EPI == kSwiglu ? (g == 0 ? n0 / 2 + r : a.N + n0 / 2 + r) : n0 + g * kCols16 + r;
-    wrow[g] = a.W + size_t(row) * a.ldw + kq * 16;
-  }
-  const uint16_t* xrow = a.X + size_t(r < a.M ? r : 0) * a.ldx + kq * 16;
-
-  f32x4 acc[RG];
-#pragma unroll
-  for (int g = 0; g < RG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  auto fetch = [&](int j0, Trip16<RG, UT>& t) {
-#pragma unroll
-    for (int d = 0; d < UT; ++d) {
-      int j = j0 + d;
-      j = j < cnt ? j : (cnt > 0 ? cnt - 1 : 0);   // beyond the slice: repeat its last unit, not multiplied
-      const size_t off = size_t(u_lo + j < units ? u_lo + j : 0) * kUnit;
-#pragma unroll
-      for (int g = 0; g < RG; ++g) {
-        t.w[g][d][0].u = *reinterpret_cast<const uint4*>(wrow[g] + off);
-        t.w[g][d][1].u = *reinterpret_cast<const uint4*>(wrow[g] + off + 8);
-      }
-      t.x[d][0].u = *reinterpret_cast<const uint4*>(xrow + off);
-      t.x[d][1].u = *reinterpret_cast<const uint4*>(xrow + off + 8);
-    }
-  };
-  auto multiply = [&](int j0, const Trip16<RG, UT>& t) {
-#pragma unroll
-    for (int d = 0; d < UT; ++d) {
-      if (j0 + d >= cnt) break;   // uniform over the wave
-#pragma unroll
-      for (int g = 0; g < RG; ++g) {
-        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.x[d][0].v, t.w[g][d][0].v, acc[g], 0, 0, 0);
-        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.x[d][1].v, t.w[g][d][1].v, acc[g], 0, 0, 0);
-      }
-    }
-  };
-  // what the epilogue needs from memory, asked for ahead of the weights: the tiles' sums of squares of
-  // four rows per wave (SCALED), and this thread's element of the residual stream and the norm's weight
-  constexpr int kSsRegs = 4;
-  float ssv[kRowsPerWave][kSsRegs];
-  float ss_more[kRowsPerWave] = {};
-  const int em = threadIdx.x / 16, en = threadIdx.x % 16;   // the epilogue's (row, column of a group)
-  float resid_in = 0.f, g_in = 0.f;
-  if constexpr (SCALED) {
-#pragma unroll
-    for (int i = 0; i < kRowsPerWave; ++i) {
-      const int m = wave + NW * i;
-      const float* p = a.ss_in + size_t(m < a.M ? m : 0) * a.tiles_in;
-#pragma unroll
-      for (int q = 0; q < kSsRegs; ++q) {
-        const int t = lane + q * kWave;
-        ssv[i][q] = p[t < a.tiles_in ? t : 0];
-      }
-      for (int t = lane + kSsRegs * kWave; t < a.tiles_in; t += kWave) ss_more[i] += p[t];
-    }
-  }
-  if constexpr (EPI == kResidualNorm) {
-    const int col = n0 + en;
-    resid_in = a.resid[size_t(em < a.M ? em : 0) * a.N + col];
-    g_in = a.g_f32 ? static_cast<const float*>(a.g)[col] : load_f(static_cast<const bf16_t*>(a.g) + col);
-  }
-  auto rstd_to_lds = [&]() {
-    if constexpr (SCALED) {
-#pragma unroll
-      for (int i = 0; i < kRowsPerWave; ++i) {
-        float part = ss_more[i];
-#pragma unroll
-        for (int q = 0; q < kSsRegs; ++q) part += (lane + q * kWave < a.tiles_in) ? ssv[i][q] : 0.f;
-        const float s = wave_sum(part);
-        if (lane == 0) rstd_s[wave + NW * i] = rsqrtf(s * a.inv_width + a.eps);
-      }
-    }
-  };
-  if (cnt > 0) {
-    Trip16<RG, UT> ta, tb;
-    fetch(0, ta);
-    if (UT < cnt) fetch(UT, tb);
-    rstd_to_lds();
-    for (int j0 = 0; j0 < cnt; j0 += 2 * UT) {
-      multiply(j0, ta);
-      if (j0 + UT >= cnt) break;
-      if (j0 + 2 * UT < cnt) fetch(j0 + 2 * UT, ta);
-      multiply(j0 + UT, tb);
-      if (j0 + 3 * UT < cnt) fetch(j0 + 3 * UT, tb);
-    }
-  } else {
-    rstd_to_lds();
-  }
-
-#pragma unroll
-  for (int g = 0; g < RG; ++g) red[wave][g][lane] = acc[g];
-  __syncthreads();
-
-  // thread -> (row m, column n of a group): the accumulator of lane (m / 4) * 16 + n holds it as element m % 4
-  const int m = em, n = en;
-  float v[RG];
-#pragma unroll
-  for (int g = 0; g < RG; ++g) {
-    float s = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) s += red[w][g][(m / 4) * 16 + n][m % 4];
-    v[g] = SCALED ? s * rstd_s[m] : s;
-  }
-  const bool live = m < a.M;
-  if constexpr (EPI == kStore) {
-    if (live) {
-#pragma unroll
-      for (int g = 0; g < RG; ++g) store_f(static_cast<TO*>(a.out) + size_t(m) * a.ldo + n0 + g * kCols16 + n, v[g]);
-    }
-  } else if constexpr (EPI == kSwiglu) {
-    static_assert(EPI != kSwiglu || RG == 2, "gate and up are the two row groups");
-    if (live) {
-      const float gate = round_to<TO>(v[0]);
-      const float act = silu<TO>(gate);
-      store_f(static_cast<TO*>(a.out) + size_t(m) * a.ldo + n0 / 2 + n, round_to<TO>(act) * round_to<TO>(v[RG - 1]));
-    }
-  } else {
-    static_assert(EPI != kResidualNorm || RG == 1, "one 16-column tile per workgroup leaves two sums of squares");
-    const int col = n0 + n;
-    float xn = 0.f;
-    if (live) {
-      xn = resid_in + round_to<bf16_t>(v[0]);
-      a.resid[size_t(m) * a.N + col] = xn;
-      a.xg[size_t(m) * a.N + col] = float_to_bf16_bits(g_in * round_to<bf16_t>(xn));
-    }
-    float sq = xn * xn;   // summed over the 8 columns of a tile: the same tiles as the 8-row kernel leaves
-    sq += __shfl_xor(sq, 1, kWave);
-    sq += __shfl_xor(sq, 2, kWave);
-    sq += __shfl_xor(sq, 4, kWave);
-    if (live && n % kCols == 0) a.ss_out[size_t(m) * (a.N / kCols) + blockIdx.x * 2 + n / kCols] = sq;
-  }
-}
-
 bool operands_ok(const Gemm8Args& a) {
   return a.ldx % 8 == 0 && a.ldw % 8 == 0 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(a.W) % 16 == 0 && a.ldx >= a.K && a.ldw >= a.K;
@@ -404,11 +248,9 @@ using namespace kvcm;
 
 extern "C" {
 
-// Shapes these kernels take: at most 8 rows with whole 8-column tiles, 9 to 16 rows with whole 16-column
-// tiles; whole 64-element units of K.
+// Shapes these kernels take: at most 8 rows with whole 8-column tiles; whole 64-element units of K.
 int kvcm_gemm8_supported(int M, int N, int K) {
-  if (!(M >= 1 && K >= kUnit && K % kUnit == 0)) return 0;
-  return M <= 8 ? (N >= 8 && N % 8 == 0) : (M <= 16 && N >= 16 && N % 16 == 0);
+  return M >= 1 && M <= 8 && K >= kUnit && K % kUnit == 0 && N >= 8 && N % 8 == 0;
 }
 
 // out[M, N] = (X * W^T) (* rstd per row when ss_in is given: X is then xg of a producer, ss_in its
@@ -426,19 +268,6 @@ int kvcm_gemm8(const void* X, int ldx, const void* W, int ldw, int M, int N, int
   a.inv_width = tiles_in > 0 ? 1.0f / float(tiles_in * kCols) : 0.f; a.eps = eps; a.out = out; a.ldo = ldo;
   KVCM_REQUIRE(operands_ok(a), "gemm8: operands must be 16-byte aligned with leading dimensions that are multiples of 8 and at least K");
   const bool scaled = ss_in != nullptr;
-  if (M > 8) {   // 9 to 16 rows: 16 columns per row group, a quarter of K per wave
-#define KVCM_G16(RG, UT, SC, EP, TO) gemm16_kernel<RG, UT, SC, EP, TO><<<grid, 256, 0, st>>>(a)
-    if (swiglu) {
-      const dim3 grid(N / kCols16);
-      if (out_dtype == kBF16) { if (scaled) KVCM_G16(2, 2, true, kSwiglu, bf16_t); else KVCM_G16(2, 2, false, kSwiglu, bf16_t); }
-      else { if (scaled) KVCM_G16(2, 2, true, kSwiglu, float); else KVCM_G16(2, 2, false, kSwiglu, float); }
-      return launch_status("gemm16_swiglu");
-    }
-    const dim3 grid(N / kCols16);
-    if (out_dtype == kBF16) { if (scaled) KVCM_G16(1, 4, true, kStore, bf16_t); else KVCM_G16(1, 4, false, kStore, bf16_t); }
-    else { if (scaled) KVCM_G16(1, 4, true, kStore, float); else KVCM_G16(1, 4, false, kStore, float); }
-    return launch_status("gemm16");
-  }
   // longer trips where two trips of UT units per half would not have a tile's whole K on its way at once
 #define KVCM_G8(RG, UT, SC, EP, TO)                                                         \
   do {                                                                                      \
@@ -483,15 +312,6 @@ int kvcm_gemm8_residual_norm(const void* X, int ldx, const void* W, int ldw, int
   a.M = M; a.N = N; a.K = K; a.resid = resid; a.g = g; a.g_f32 = g_dtype == kF32; a.xg = static_cast<uint16_t*>(xg);
   a.ss_out = ss_out;
   KVCM_REQUIRE(operands_ok(a), "gemm8_residual_norm: operands must be 16-byte aligned with leading dimensions that are multiples of 8 and at least K");
-  if (M > 8) {
-    const dim3 grid(N / kCols16);
-    // a wave's quarter of K in two trips where it fits the registers of a wave that has its SIMD to itself
-    // (N / 16 workgroups: fewer than CUs at the widths of a residual stream)
-    if (K / kUnit > 4 * 2 * 8) gemm16_kernel<1, 11, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);
-    else if (K / kUnit > 4 * 2 * 4) gemm16_kernel<1, 8, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);
-    else gemm16_kernel<1, 4, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);
-    return launch_status("gemm16_residual_norm");
-  }
   const dim3 grid(N / kCols);
   if (K / kUnit > 8 * 2 * 4) gemm8_kernel<4, 1, 6, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);
   else gemm8_kernel<4, 1, 4, false, kResidualNorm, bf16_t><<<grid, 256, 0, st>>>(a);

@@ -163,9 +163,10 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// The same product for more than 16 rows.  With that many rows X is no longer small: every
-// 16-column tile needs all of it, and re-reading it from L2 per tile would cost several times the
-// weights' bytes.  Here a workgroup of NWV waves owns NWV column tiles (one 16-column tile per wave;
+// The same product with the rows shared by a workgroup's waves: the kernel every unfolded product of up
+// to 512 rows takes when its width is a multiple of 64 (the one above serves the other widths).  X is
+// not small beside the weights: every 16-column tile needs all of it, and re-reading it from L2 per tile
+// costs as many bytes as the weights from 8 rows on.  Here a workgroup of NWV waves owns NWV column tiles (one 16-column tile per wave;
 // the last workgroup may have fewer tiles than waves), up to 128 rows and a slice of K, and its waves
 // share X through LDS: per trip of DEPTH x 64 k the workgroup stages X[rows][DEPTH * 64] once
 // (double-buffered; the next trip's global loads are issued before the current trip's products), every
@@ -329,9 +330,14 @@ using namespace kvcm;
 
 constexpr int kMaxSharedRows = 512;
 
-// More than 16 rows and whole groups of 64 columns: the kernel whose waves share X through LDS.
-static bool shares_rows(int M, int N) { return M > 16 && M <= kMaxSharedRows && N % 64 == 0; }
+// Whole groups of 64 columns: the kernel whose waves share X through LDS.
+static bool shares_rows(int M, int N) { return M > 0 && M <= kMaxSharedRows && N % 64 == 0; }
 static int row_blocks(int M) { return (M + kRowBlock - 1) / kRowBlock; }
+// The SwiGLU form (I: the activation's width) is unsplit: with too few workgroups a split product and a
+// launch for SwiGLU fill the chip better.
+static bool swiglu_shares_rows(int M, int I) {
+  return M > 0 && M <= kMaxSharedRows && I % 32 == 0 && (I / 32) * row_blocks(M) >= 160;
+}
 
 // Waves per workgroup (each takes one column tile) so that tiles x splits x row blocks make about one
 // workgroup per CU and none is left out: a CU has only so many requests for weights on their way, so what
@@ -378,7 +384,8 @@ static void launch_rows_n(hipStream_t st, const uint16_t* x, const uint16_t* w, 
 #define KVCM_ROWS(MT, DEPTH) \
   gemm_rows_kernel<MT, DEPTH, TO, SWIGLU, NWV><<<grid, NWV * kWave, 0, st>>>(x, w, partials, out, M, N, K, ldx, ldw, ldo, S)
   switch (mt) {
-    case 1: case 2: KVCM_ROWS(2, 4); break;
+    case 1: KVCM_ROWS(1, 4); break;
+    case 2: KVCM_ROWS(2, 4); break;
     case 3: KVCM_ROWS(3, 4); break;
     case 4: KVCM_ROWS(4, 4); break;
     case 5: case 6: KVCM_ROWS(6, 2); break;
@@ -429,7 +436,7 @@ int kvcm_gemm_skinny_splits(int M, int N, int K) {
 // Waves per workgroup that the shared-rows kernel runs a bfloat16 product of this shape with (0: another
 // kernel takes the shape).  swiglu: N is the activation's width, S is 1.
 int kvcm_gemm_skinny_waves(int M, int N, int K, int S, int swiglu) {
-  if (swiglu ? !(M > 16 && M <= kMaxSharedRows && N % 32 == 0) : !shares_rows(M, N)) return 0;
+  if (swiglu ? !swiglu_shares_rows(M, N) : !shares_rows(M, N)) return 0;
   if (K <= 0 || K % kUnit != 0 || S < 1) return 0;
   if (!swiglu && S == 1) return 4;
   return rows_waves(static_cast<long long>(N / (swiglu ? 8 : 16)) * row_blocks(M) * S, rows_tiles_m(M));
@@ -470,8 +477,10 @@ int kvcm_gemm_skinny(const void* X, const void* W, float* partials, void* out, i
 // May act = swiglu(X * [gate | up]^T) be computed in one launch?  I is the width of the result.
 int kvcm_gemm_skinny_swiglu_supported(int M, int I, int K) {
   if (!(M > 0 && I > 0 && I % 8 == 0 && K > 0 && K % kUnit == 0)) return 0;
-  // with too few workgroups a split product fills the chip better than this unsplit one
-  if (M > 16 && M <= kMaxSharedRows && I % 32 == 0) return (I / 32) * row_blocks(M) >= 160;
+  if (swiglu_shares_rows(M, I)) return 1;
+  // with too few workgroups a split product fills the chip better than an unsplit one; the kernel whose
+  // every tile reads the rows from L2 serves a few rows, or widths that are no multiple of 32
+  if (I % 32 == 0 && M > 16) return 0;
   return M <= 64 && I / 8 >= 320;
 }
 
@@ -487,7 +496,7 @@ int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dty
   const uint16_t* x = static_cast<const uint16_t*>(X);
   const uint16_t* w = static_cast<const uint16_t*>(W);
   const int mt = (M + 15) / 16;
-  if (M > 16 && M <= kMaxSharedRows && I % 32 == 0) {
+  if (swiglu_shares_rows(M, I)) {
     if (out_dtype == kBF16) launch_rows<bf16_t, true>(st, x, w, nullptr, static_cast<bf16_t*>(out), M, I, K, ldx, ldw, ldo, 1);
     else launch_rows<float, true>(st, x, w, nullptr, static_cast<float*>(out), M, I, K, ldx, ldw, ldo, 1);
     return launch_status("gemm_rows_swiglu");

@@ -67,8 +67,7 @@ int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dty
 int kvcm_gemm_f32(const float* X, const float* W, float* Y, int M, int N, int K, int ldx, int ldw, int ldy, hipStream_t s);
 int kvcm_gemm_bf16(const void* X, const void* W, void* Y, int out_dtype, int M, int N, int K, int ldx, int ldw, int ldy,
                    hipStream_t s);
-// Products of at most 16 rows with the RMS norm around them folded in (gemm_rows8.hip: one kernel for up to
-// 8 rows, one for 9 to 16).
+// Products of at most 8 rows with the RMS norm around them folded in (gemm_rows8.hip).
 int kvcm_gemm8_supported(int M, int N, int K);
 int kvcm_gemm8(const void* X, int ldx, const void* W, int ldw, int M, int N, int K, const float* ss_in, int tiles_in,
                float eps, void* out, int out_dtype, int ldo, int swiglu, hipStream_t stream);

@@ -90,7 +90,7 @@ class StepContext(StepView):
     def __init__(self, runner, layout: BatchLayout):
         self.runner, self.layout = runner, layout
         self.limits, self.attention_mode = runner.limits, runner.attn
-        self.fold_norms, self.tune_products = runner.fold_norms, runner.tune_products
+        self.fold_norms, self.fold_rows, self.tune_products = runner.fold_norms, runner.fold_rows, runner.tune_products
         self.recording = False
         L = layout
         self.rows, self.real_rows = L.rows_padded, L.rows
@@ -167,6 +167,7 @@ class ModelRunner:
         self.dtype, self.device, self.attn = dtype, device, attn
         self.fold_norms, self.tune_products = bool(fold_norms), tune_products
         self.ops = model.ctx.ops
+        self.fold_rows = self._fold_rows()
         self.workspace = Workspace(device, dtype, limits, self.ops)
         G = core.num_groups
         # (logits of every row may be asked for and fetched in portions: room for that many indices)
@@ -179,6 +180,19 @@ class ModelRunner:
         self._upload_done = torch.cuda.Event()
         self._upload_pending = False
         model.attach_caches(storages)
+
+    # Every workgroup of a folded product reads all of the step's rows from L2 (rows x K per 8 or 16 output
+    # columns), so a folded step's time grows with its rows by about a ninth of the layers' weight bytes at
+    # L2 speed, while the unfolded path (rows shared through LDS, two norm launches a layer more) costs the
+    # same from 1 to 16 rows.  Measured: at TinyLlama sizes (88 MB a layer) folding wins at every row count up
+    # to 8 (batch 8: 1.00 against 1.13 ms), at Llama-3-8B sizes (436 MB a layer) only up to 2 rows (batch 4:
+    # 4.15 against 3.97 ms, batch 8: 4.61 against 3.96).  Rows x bytes of a layer's weights up to this pay.
+    FOLD_ROWS_TIMES_LAYER_BYTES = 1.0e9
+
+    def _fold_rows(self) -> int:
+        layers = max(1, len(self.model.spec.schedule))
+        per_layer = max(1.0, self.model.step_bytes(1, 0) / layers)
+        return max(1, min(self.ops.FUSED_NORM_MAX_ROWS, int(self.FOLD_ROWS_TIMES_LAYER_BYTES // per_layer)))
 
     def host_buffer(self) -> np.ndarray:
         """The pinned metadata buffer, once the previous step's upload no longer reads it."""

@@ -270,9 +270,10 @@ class PartialSums:
         return self.out
 
 
-# Decode steps of at most this many rows fold their RMS norms into the products around them
-# (csrc/hip/gemm_rows8.hip).
-FUSED_NORM_MAX_ROWS = 16
+# Decode steps of at most this many rows may fold their RMS norms into the products around them
+# (csrc/hip/gemm_rows8.hip); how many rows of that a model's steps do fold is the engine's to say
+# (StepView.fold_rows).
+FUSED_NORM_MAX_ROWS = 8
 
 
 def gemm8_supported(M, N, K):
@@ -314,7 +315,7 @@ class NormedRows:
 
 def gemm_residual_norm(product, x, weight, eps, xg, ss, out):
     """x += round(product); returns NormedRows for the norm (weight, eps) that follows: the producer
-    half of the folded norm.  product: PendingProduct of at most 16 bfloat16 rows; x: the 32-bit residual
+    half of the folded norm.  product: PendingProduct of at most 8 bfloat16 rows; x: the 32-bit residual
     stream [rows, H]; xg [>= rows, H] bfloat16 and ss [>= rows, H / 8] float32 receive the result; out:
     where ``materialize`` would put ordinary normed rows."""
     a, w = product.x, product.w
@@ -335,7 +336,7 @@ def gemm_residual_norm(product, x, weight, eps, xg, ss, out):
 
 
 def _gemm8(x, w, out, N, swiglu):
-    """The product of at most 16 rows (gemm_rows8.hip); x: a tensor or NormedRows."""
+    """The product of at most 8 rows (gemm_rows8.hip); x: a tensor or NormedRows."""
     normed = isinstance(x, NormedRows)
     a = x.xg if normed else x
     M, K = a.shape

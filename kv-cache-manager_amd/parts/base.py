@@ -114,6 +114,8 @@ class StepView:
                                    call nothing but this package's kernels (ctx.ops) on device arrays
       fold_norms                   the engine option of that name: False keeps every norm a launch of its
                                    own, rounding exactly where the reference does
+      fold_rows                    the most rows a step may have for its norms to be folded (the engine's
+                                   estimate of where folding stops paying for this model's widths)
       tune_products                the engine option of that name ("off" | "heuristic" | "all"), handed to
                                    ops.gemm as ``tuning``
 
@@ -142,6 +144,7 @@ class StepView:
     recording = False
     attention_mode = "auto"
     fold_norms = True
+    fold_rows = 8
     tune_products = None
     max_run = 1
     limits = None

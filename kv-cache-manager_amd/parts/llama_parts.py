@@ -27,7 +27,7 @@ def _to_residual(ctx, step, x, w, name):
     rows it is handed on unrun (ops.PendingProduct): the norm that follows runs it with the addition
     and its own preparation in the epilogue.  Otherwise it runs here, split sums left un-added."""
     ops = ctx.ops
-    if (step.fold_norms and x.dtype == torch.bfloat16 and x.shape[0] <= ops.FUSED_NORM_MAX_ROWS
+    if (step.fold_norms and x.dtype == torch.bfloat16 and x.shape[0] <= min(ops.FUSED_NORM_MAX_ROWS, step.fold_rows)
             and ops.gemm8_supported(x.shape[0], w.shape[0], w.shape[1])):
         out = step.ws(name, (x.shape[0], w.shape[0]))
         return ops.PendingProduct(x, w, out, step.scratch(name, x.shape[0], w.shape[0], w.shape[1]))

@@ -734,12 +734,11 @@ def test_skinny_gemm_with_swiglu_epilogue_equals_product_then_swiglu(ops):
         ops.gemm(x, w, gu)                                   # unsplit: no scratch given
         ref = torch.zeros_like(act)
         ops.swiglu(gu, ref)
-        if M <= 16:
-            assert torch.equal(act, ref)
-        else:   # more than 16 rows: workgroups walk K from different starting points in the two launches
-            a, b = _np(act), _np(ref)
-            assert np.mean(a == b) > 0.98
-            np.testing.assert_allclose(a, b, rtol=2 ** -6, atol=2e-3)
+        # the two launches walk K in different orders (other kernels, or workgroups that start at different
+        # places): a sum may round to the neighbouring bfloat16 now and then
+        a, b = _np(act), _np(ref)
+        assert np.mean(a == b) > 0.98
+        np.testing.assert_allclose(a, b, rtol=2 ** -6, atol=2e-3)
     small = torch.zeros(8, 256, dtype=torch.bfloat16, device=DEV)      # too few columns to fill the chip unsplit
     assert not ops.gemm_swiglu(_t(rng.normal(size=(8, 64)), torch.bfloat16), _t(rng.normal(size=(512, 64)), torch.bfloat16), small)
     big = torch.zeros(65, 2560, dtype=torch.bfloat16, device=DEV)      # too many rows for the streaming kernel
@@ -1152,7 +1151,7 @@ def test_prefill_attention_longer_segments_when_the_launch_is_wide(ops, B):
         np.testing.assert_allclose(got[r], ref, atol=1e-2, rtol=0, err_msg=f"row {r}")
 
 
-# ------------------------------------- products of at most 16 rows with the norm folded in
+# ------------------------------------- products of at most 8 rows with the norm folded in
 def _folded_reference(a, wo, x, g, eps, w2):
     """What the producer and the consumer compute, in float64 with the same rounding points:
     x += round(a wo^T); xg = round(g round(x)); y = round((xg w2^T) rsqrt(mean x^2 + eps))."""
@@ -1162,14 +1161,13 @@ def _folded_reference(a, wo, x, g, eps, w2):
     return x_new, xg, (xg @ w2.T) * rstd
 
 
-@pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16])
+@pytest.mark.parametrize("M", [1, 3, 5, 8])
 @pytest.mark.parametrize("H,K,N2", [(2048, 2048, 2560), (2048, 5632, 512), (128, 64, 48), (320, 192, 32), (2048, 2112, 4128)])
 def test_products_with_the_norm_folded_in(ops, M, H, K, N2):
     """Producer (residual add + the norm's preparation in the epilogue) and consumer (the norm's scale on
     the finished sums) against the same arithmetic in float64, and against the reference's own form of
     the norm, whose two roundings fall at other places (kernels.cu:34-49): equal up to bfloat16 rounding.
-    Widths that are no power of two, K slices of unequal length, fewer rows than a tile holds; up to 8
-    rows and 9 to 16 rows are two kernels that leave and read the same sums of squares."""
+    Widths that are no power of two, K slices of unequal length, fewer rows than a tile holds."""
     rng = np.random.default_rng(M * 13 + H + K)
     a = _bf16_grid(rng.normal(size=(M, K)))
     wo = _bf16_grid(rng.normal(size=(H, K)) * 0.05)
@@ -1206,7 +1204,7 @@ def test_products_with_the_norm_folded_in(ops, M, H, K, N2):
     np.testing.assert_allclose(_np(h.materialize()), plain.rms_norm(got_x, g, eps, plain.round_bf16), rtol=2 ** -7, atol=1e-3)
 
 
-@pytest.mark.parametrize("M", [1, 5, 8, 11, 16])
+@pytest.mark.parametrize("M", [1, 5, 8])
 @pytest.mark.parametrize("H,I", [(2048, 5632), (192, 144), (64, 16)])
 def test_gate_up_product_with_the_norm_folded_in_applies_swiglu(ops, M, H, I):
     rng = np.random.default_rng(M + H + I)
@@ -1238,7 +1236,7 @@ def test_gate_up_product_with_the_norm_folded_in_applies_swiglu(ops, M, H, I):
     np.testing.assert_allclose(got, ref, rtol=0, atol=2e-2 * max(np.abs(ref).max(), 1e-3))
 
 
-@pytest.mark.parametrize("M", [1, 8, 10, 16])
+@pytest.mark.parametrize("M", [1, 6, 8])
 def test_small_product_plain_form_and_refusals(ops, M):
     """The same kernel without a norm in front (a tensor in x's place), float32 and bfloat16 results,
     one and two column groups per workgroup; shapes it does not take are refused by the entry."""
@@ -1251,11 +1249,11 @@ def test_small_product_plain_form_and_refusals(ops, M):
             ops._gemm8(_t(x, torch.bfloat16), _t(w, torch.bfloat16), out, N, False)
             tol = dict(rtol=2 ** -7, atol=1e-3) if dtype == torch.bfloat16 else dict(rtol=0, atol=2e-5 * math.sqrt(K))
             np.testing.assert_allclose(_np(out), plain.linear(x, w), **tol)
-    assert not ops.gemm8_supported(17, 2048, 2048) and not ops.gemm8_supported(4, 2044, 2048) and not ops.gemm8_supported(4, 2048, 96)
-    assert ops.gemm8_supported(8, 24, 64) and not ops.gemm8_supported(9, 24, 64)      # 9 to 16 rows: whole 16-column tiles
+    assert not ops.gemm8_supported(9, 2048, 2048) and not ops.gemm8_supported(4, 2044, 2048) and not ops.gemm8_supported(4, 2048, 96)
+    assert ops.gemm8_supported(8, 24, 64) and not ops.gemm8_supported(16, 32, 64)      # more than 8 rows: another kernel's
     with pytest.raises(ops.KernelError, match="unsupported shape"):
-        ops._gemm8(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(16, 64, dtype=torch.bfloat16, device=DEV),
-                   torch.zeros(17, 16, dtype=torch.bfloat16, device=DEV), 16, False)
+        ops._gemm8(torch.zeros(9, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(16, 64, dtype=torch.bfloat16, device=DEV),
+                   torch.zeros(9, 16, dtype=torch.bfloat16, device=DEV), 16, False)
 
 
 # ------------------------------------------------ where the order of rounding and multiplying shows
@@ -1304,7 +1302,7 @@ def test_norm_and_swiglu_kernels_round_where_the_reference_rounds(ops):
     fused = torch.zeros(rows_, I, dtype=torch.bfloat16, device=DEV)
     ops._gemm8(xt, wt, fused, I, True)                                   # the product of at most 8 rows
     np.testing.assert_array_equal(_np(fused), act_want)
-    for M in (rows_, 24):                                                # the weight-streaming products: up to 16 rows, and more
+    for M in (rows_, 24):                                                # the product whose waves share the rows
         Xm = np.zeros((M, K))
         Xm[:rows_] = X
         wide = 5632                                                      # wide enough for the one-launch form to be taken

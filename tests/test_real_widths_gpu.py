@@ -86,9 +86,9 @@ def test_real_widths_whole_tail_singly_and_mixed(real_width_setup, dtype):
 
 
 def test_real_widths_decode_through_the_engine_with_forced_tokens(real_width_setup):
-    """The scheduler's own decode steps at batch 3, 8 and 13 (graphs; the products that fold the norms in,
-    in their form for up to 8 rows and in the one for 9 to 16) and its prompt steps (the library's products),
-    teacher-forced: logits against the plain implementation."""
+    """The scheduler's own decode steps at batch 3, 8 and 13 (graphs; the products that fold the norms in at up
+    to 8 rows, the shared-rows products with norm launches of their own beyond) and its prompt steps (the
+    library's products), teacher-forced: logits against the plain implementation."""
     from kvcm_amd import Engine, EngineConfig
     from kvcm_amd.engine.replay import scheduled_replay
     cfg, tensors, reqs, ref = real_width_setup["bfloat16"]
@@ -148,9 +148,9 @@ def test_real_widths_bfloat16_error_distribution(real_width_setup):
 
 def test_real_widths_folded_norms_against_unfolded_and_against_steps_of_many_rows(real_width_setup):
     """The same positions computed three ways in bfloat16: in single-row steps with the norms folded into
-    the products (the default for up to 16 rows), in the same steps with every norm a launch of its own
+    the products (the default for up to 8 rows at these widths), in the same steps with every norm a launch of its own
     (EngineConfig.fold_norms=False), and in steps of 20 rows (20 requests decoding side by side: the
-    shared-rows products and norm launches that steps of 17 rows and more take).  Each stays inside the
+    shared-rows products and norm launches that steps of 9 rows and more take).  Each stays inside the
     tolerance against the plain implementation, and their distances from one another are reported and
     bounded: a position's logits depend on the kind of step it ran in by no more than they differ from
     the plain implementation anyway."""

@@ -65,12 +65,13 @@ def _noalloc(clib, x, w, out_dtype):
 
 
 # (M, N, K) pairs: a first call and a smaller second one.  The first of each pair splits K (the
-# column tiles alone do not fill the chip); both forms of the kernel: up to 16 rows, and rows
-# shared through LDS.
+# column tiles alone do not fill the chip); both forms of the kernel: the one whose waves share the
+# rows through LDS (widths that are multiples of 64), and the one whose every tile reads them itself.
 _PAIRS = [
     ((8, 2048, 2048), (3, 512, 1024)),
     ((64, 2048, 5632), (24, 1024, 512)),
     ((16, 2560, 2048), (1, 2560, 2048)),
+    ((8, 2064, 2048), (3, 528, 1024)),
 ]
 
 
