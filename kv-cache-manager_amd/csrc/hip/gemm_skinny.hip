@@ -1,8 +1,11 @@
-// Decode-shaped products: Y[M,N] = X[M,K] * W[N,K]^T with few rows (M <= 64) and a weight matrix
-// that has to be streamed from HBM once.  The reference leaves these to cuBLAS
-// (src/model/llama.cpp:45-52); here the point is to keep enough weight bytes in flight on 256 CUs.
+// Decode-shaped products: Y[M,N] = X[M,K] * W[N,K]^T with few rows and a weight matrix that has to be
+// streamed from HBM once.  The reference leaves these to cuBLAS (src/model/llama.cpp:45-52); here the
+// point is to keep enough weight bytes in flight on 256 CUs.  Two kernels: the first for up to 64 rows
+// and any width that is a multiple of 16, each tile reading the rows from L2 itself; the second, further
+// down, for up to 512 rows and widths that are multiples of 64, a workgroup's waves sharing the rows
+// through LDS.  Shapes both take go to the second.
 //
-// One workgroup (4 waves) owns 16 output columns and one slice of K ("split"); its waves divide
+// First kernel: one workgroup (4 waves) owns 16 output columns and one slice of K ("split"); its waves divide
 // the slice among themselves, each streaming its rows of W straight from global memory into
 // MFMA operand registers (every lane 32 contiguous bytes, four lanes one 128-byte line) and
 // multiplying with the matching pieces of X (v_mfma_f32_16x16x32_bf16).  The four waves' sums
