@@ -113,6 +113,34 @@ def _floor(nodes):
             g = 1e3 * e0.elapsed_time(e1) / (30 * nodes)
             rate = "%.2f" % (nbytes / g / 1e6) if nbytes else ""
             print("%-36s %10.2f %10.2f %12s" % (name, eager, g, rate))
+        # what a launch streams as a function of the CUs it covers and the waves on each: 46 MB (a gate/up matrix of
+        # TinyLlama sizes), every workgroup a contiguous share, consecutive launches consecutive regions
+        n = (46 << 20) // 4
+        print("\n46 MB read by one launch of G workgroups of W waves (a contiguous share each, 8 loads of 16 bytes on their"
+              "\nway per lane; 16 where said), launches of a graph one after the other: microseconds, TB/s")
+        print("%6s %4s %10s %10s" % ("G", "W", "us", "TB/s"))
+        for G, W, inflight in ((64, 4, 8), (128, 4, 8), (176, 4, 8), (176, 8, 8), (176, 4, 16), (235, 3, 8), (256, 2, 8), (256, 4, 8),
+                               (256, 8, 8), (512, 4, 8), (1024, 4, 8)):
+            def run_all():
+                for i in range(16):
+                    lo = (i * n) % (big.numel() - n)
+                    lo -= lo % 4
+                    ops.probe_stream(big[lo:lo + n], sink, G, W, inflight)
+            run_all()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                run_all()
+            for _ in range(3):
+                graph.replay()
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                graph.replay()
+            e1.record()
+            e1.synchronize()
+            us = 1e3 * e0.elapsed_time(e1) / (20 * 16)
+            print("%6d %4d %10.2f %10.2f%s" % (G, W, us, n * 4 / us / 1e6, "   (16 loads per lane)" if inflight == 16 else ""))
     return 0
 
 

@@ -343,8 +343,8 @@ static bool swiglu_shares_rows(int M, int I) {
 }
 
 // Waves per workgroup (each takes one column tile) so that tiles x splits x row blocks make about one
-// workgroup per CU and none is left out: a CU has only so many requests for weights on their way, so what
-// a launch streams per microsecond grows with the CUs it covers, not with the waves on each (measured:
+// workgroup per CU and none is left out: what this kernel streams per microsecond grows with the CUs it
+// covers, not with the waves on each (measured:
 // gate/up at TinyLlama sizes, 704 tiles, 32 rows: 176 workgroups of four waves 16.5 us, 235 of three
 // 13.2 us; at Llama-3-8B sizes, 1,792 tiles, 64 rows: 448 of four 63 us, 256 of seven 51 us).  One wave
 // more where that saves a staging pass (the workgroup's threads stage 16 rows per wave at a time: 64 rows

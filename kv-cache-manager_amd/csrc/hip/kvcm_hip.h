@@ -124,6 +124,8 @@ int kvcm_fill_index(int* out, long long n, uint64_t key, int modulus, hipStream_
 int kvcm_probe_empty(int grid, int block, hipStream_t s);
 int kvcm_probe_copy(const void* src, void* dst, long long bytes, int grid, hipStream_t s);      // moves 2 * bytes
 int kvcm_probe_read(const void* src, long long bytes, void* sink, int grid, hipStream_t s);
+// the same, every workgroup (of `waves` waves) reading a contiguous share with `inflight` 16-byte loads per lane on their way
+int kvcm_probe_stream(const void* src, long long bytes, void* sink, int grid, int waves, int inflight, hipStream_t s);
 int kvcm_probe_mfma(int iters, void* sink, int grid, hipStream_t s);   // grid * 4 waves * iters * 4 * 32768 flops
 // What it costs workgroups of one launch to depend on one another (every wait inside is bounded: flags[0] counts
 // workgroups that gave up, flags[1] wrong values): a barrier across G workgroups, `rounds` times; S sums per tile

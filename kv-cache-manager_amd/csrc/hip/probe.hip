@@ -34,6 +34,27 @@ __global__ void probe_read_kernel(const uint4* __restrict__ src, long long n, un
   if (acc == 0x9E3779B9u) sink[threadIdx.x] = acc;
 }
 
+// The same with a workgroup's share of the bytes contiguous (as a product's workgroup streams its own weight
+// rows) and a stated number of 16-byte loads on their way per lane: what a launch reads per microsecond
+// as a function of how many CUs it covers and how many waves each has.
+template <int INFLIGHT>
+__global__ void probe_stream_kernel(const uint4* __restrict__ src, long long n, unsigned* __restrict__ sink) {
+  const long long per = (n + gridDim.x - 1) / gridDim.x;
+  const long long lo = blockIdx.x * per, hi = lo + per < n ? lo + per : n;
+  unsigned acc = 0;
+  for (long long i = lo + threadIdx.x; i < hi; i += (long long)blockDim.x * INFLIGHT) {
+    uint4 v[INFLIGHT];
+#pragma unroll
+    for (int u = 0; u < INFLIGHT; ++u) {
+      const long long j = i + (long long)u * blockDim.x;
+      v[u] = src[j < hi ? j : hi - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < INFLIGHT; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  if (acc == 0x9E3779B9u) sink[threadIdx.x] = acc;
+}
+
 // `iters` rounds of four independent 32x32x16 bfloat16 matrix instructions per wave: 4 * 32768 flops a round
 __global__ void __launch_bounds__(256) probe_mfma_kernel(int iters, float* __restrict__ sink) {
   bf16x8 a, b;
@@ -232,6 +253,19 @@ int kvcm_probe_read(const void* src, long long bytes, void* sink, int grid, hipS
   KVCM_REQUIRE(src && sink && bytes > 0 && bytes % 16 == 0 && grid > 0, "probe_read: bad arguments");
   probe_read_kernel<<<grid, 256, 0, s>>>(static_cast<const uint4*>(src), bytes / 16, static_cast<unsigned*>(sink));
   return launch_status("probe_read");
+}
+
+// grid workgroups of `waves` waves, each workgroup an equal contiguous share of the bytes, `inflight` (4, 8 or
+// 16) loads of 16 bytes on their way per lane
+int kvcm_probe_stream(const void* src, long long bytes, void* sink, int grid, int waves, int inflight, hipStream_t s) {
+  KVCM_REQUIRE(src && sink && bytes > 0 && bytes % 16 == 0 && grid > 0 && waves >= 1 && waves <= 16, "probe_stream: bad arguments");
+  const uint4* p = static_cast<const uint4*>(src);
+  unsigned* k = static_cast<unsigned*>(sink);
+  if (inflight == 4) probe_stream_kernel<4><<<grid, waves * 64, 0, s>>>(p, bytes / 16, k);
+  else if (inflight == 8) probe_stream_kernel<8><<<grid, waves * 64, 0, s>>>(p, bytes / 16, k);
+  else if (inflight == 16) probe_stream_kernel<16><<<grid, waves * 64, 0, s>>>(p, bytes / 16, k);
+  else KVCM_REQUIRE(false, "probe_stream: 4, 8 or 16 loads in flight");
+  return launch_status("probe_stream");
 }
 
 // grid workgroups of four waves, each wave iters * 4 matrix instructions of 32768 flops

@@ -73,6 +73,7 @@ def _declare(lib):
     fn("kvcm_probe_empty", i, i, vp)
     fn("kvcm_probe_copy", vp, vp, C.c_longlong, i, vp)
     fn("kvcm_probe_read", vp, C.c_longlong, vp, i, vp)
+    fn("kvcm_probe_stream", vp, C.c_longlong, vp, i, i, i, vp)
     fn("kvcm_probe_mfma", i, vp, i, vp)
     fn("kvcm_probe_barrier", vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_probe_sums", vp, vp, vp, i, i, i, vp, vp)
@@ -786,6 +787,14 @@ def probe_read(src, sink, grid=2048, nbytes=None):
     n = src.numel() * src.element_size() if nbytes is None else int(nbytes)
     _need(src.is_contiguous() and n % 16 == 0 and n <= src.numel() * src.element_size() and sink.numel() * sink.element_size() >= 1024, "probe_read needs whole 16-byte pieces and a sink of 1 KiB")
     _check(lib().kvcm_probe_read(_ptr(src), n, _ptr(sink), int(grid), _stream()))
+
+
+def probe_stream(src, sink, grid, waves=4, inflight=8):
+    """``src`` read once by ``grid`` workgroups of ``waves`` waves, a contiguous share each."""
+    _dev(src, sink)
+    n = src.numel() * src.element_size()
+    _need(src.is_contiguous() and n % 16 == 0 and sink.numel() * sink.element_size() >= 1024, "probe_stream needs whole 16-byte pieces and a sink of 1 KiB")
+    _check(lib().kvcm_probe_stream(_ptr(src), n, _ptr(sink), int(grid), int(waves), int(inflight), _stream()))
 
 
 def probe_mfma(iters, sink, grid=2048):
