@@ -443,6 +443,21 @@ def add_residual(x, y):
 # package's kernels against 2.24 with the library's, 80 rows 2.05 / 2.26, 112 rows 2.83 / 2.61,
 # 176 rows 2.85 / 2.56, 336 rows 3.85 / 2.98.
 LIBRARY_GEMM_MIN_ROWS = 96
+# ... except that up to LIBRARY_LONG_K_MIN_ROWS - 1 rows this package's kernel keeps the products whose K is
+# at least their width and whose weights are at least LIBRARY_LONG_K_BYTES (the O and down projections of 7B /
+# 8B sizes): the library's first choice is slow there.  Measured at Llama-3-8B sizes, library against this
+# package's kernel: down 74.9 / 44.3 us at 128 rows, 102 / 69 at 192, 61.5 / 72.5 at 256; O 23.1 / 19.3 at 128,
+# 31.9 / 26.6 at 192, 21.9 / 28.6 at 256; a prompt step of 128 rows 7.15 -> 6.38 ms.  TinyLlama's down projection
+# (23 MB) is the library's at every row count from 96 on (12.9 / 16.4 us at 128 rows).
+LIBRARY_LONG_K_MIN_ROWS = 193
+LIBRARY_LONG_K_BYTES = 32 << 20
+
+
+def _library_takes(M, N, K):
+    """Does a bfloat16 product of M rows go to the vendor library?"""
+    if not LIBRARY_GEMM_MIN_ROWS or M < LIBRARY_GEMM_MIN_ROWS:
+        return False
+    return not (M < LIBRARY_LONG_K_MIN_ROWS and K >= N and 2 * N * K >= LIBRARY_LONG_K_BYTES)
 
 
 # Which of the library's algorithms a shape runs.  "off": the first choice of the library's heuristic.
@@ -514,7 +529,7 @@ def gemm(x, w, out, scratch=None, keep_partial=False, tuning=None):
         _call("kvcm_gemm_f32", _ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0), _stream())
         return out
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm operands must both be bfloat16")
-    library = bool(LIBRARY_GEMM_MIN_ROWS) and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 and out.is_contiguous()
+    library = _library_takes(M, N, K) and out.dtype == torch.bfloat16 and out.is_contiguous()
     S = skinny_splits(M, N, K) if (not library and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
                                    and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0) else 0
     if S > 1 and (scratch is None or scratch.numel() < S * M * N):

@@ -641,6 +641,25 @@ def test_gemm_shared_rows_with_every_number_of_waves(ops):
     assert seen == {2, 3, 4, 5, 6, 7, 8} and seen_act >= {3, 4, 5, 6, 7, 8}, (seen, seen_act)
 
 
+def test_long_k_products_of_wide_models_stay_with_this_packages_kernel_up_to_192_rows(ops):
+    """From 96 rows on a bfloat16 product is the vendor library's, except those whose K is at least their width and
+    whose weights are 32 MB or more, up to 192 rows: the shared-rows kernel takes them, split, and the result is right."""
+    assert ops._library_takes(128, 2048, 5632) and ops._library_takes(96, 6144, 4096)          # 23 MB; wider than K
+    assert not ops._library_takes(128, 4096, 4096) and not ops._library_takes(192, 4096, 14336)
+    assert ops._library_takes(193, 4096, 4096) and not ops._library_takes(95, 2048, 2048)
+    M, N, K = 150, 4096, 4096
+    rng = np.random.default_rng(5)
+    x = _bf16_grid(rng.normal(size=(M, K)))
+    w = _bf16_grid(rng.normal(size=(N, K)) * 0.03)
+    S = ops.skinny_splits(M, N, K)
+    assert S > 1
+    scratch = torch.zeros(S * M * N, dtype=torch.float32, device=DEV)
+    out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    got = ops.gemm(_t(x, torch.bfloat16), _t(w, torch.bfloat16), out, scratch=scratch, keep_partial=True)
+    assert isinstance(got, ops.PartialSums) and got.splits == S          # the library leaves no partial sums
+    np.testing.assert_allclose(_np(got.materialize()), plain.linear(x, w), rtol=2 ** -7, atol=2e-3)
+
+
 @pytest.mark.parametrize("mode", ["off", "heuristic", "all"])
 @pytest.mark.parametrize("M,N,K", [(96, 192, 320), (200, 2560, 512), (333, 328, 136)])
 def test_library_product_with_each_choice_of_algorithm(ops, mode, M, N, K):
