@@ -443,7 +443,7 @@ int kvcm_attention_decode_fused_info(int nh, int nkv, int hd, int* out) {
 // How a launch for T rows with contexts of at most max_context cuts them: one workgroup per
 // (kv head, row) while that fills the chip or contexts are short; else parts of whole chunks, about
 // one workgroup per CU in all.  Returns the number of parts, *part_chunks chunks of 256 tokens each.
-constexpr int kFusSingleMax = 1024;   // contexts up to this always run as one part
+constexpr int kFusSingleMax = 1024;   // contexts up to this run as one part, unless few workgroups read much each (below)
 constexpr int kFusTargetWorkgroups = 256;
 // A workgroup of eight waves has a CU to itself (registers).  From two workgroups per CU on, a
 // launch at head_dim 64 takes workgroups of four waves, each of which walks every chunk: two of
@@ -451,11 +451,19 @@ constexpr int kFusTargetWorkgroups = 256;
 // walk.  Measured inside decode steps of 512-token prompts: 128 rows 2.26 -> 2.16 ms, 256 rows
 // 3.45 -> 3.22 ms, 64 rows (256 workgroups) 1.61 -> 1.63 ms, hence the limit.
 constexpr long long kFusHalfFrom = 512;
-static int fused_parts(int T, int nkv, int max_context, int* part_chunks) {
+// A workgroup reads its context through one CU, which has only so many requests on their way: with few
+// workgroups and more than kFusFewBytes of keys and values each (512 tokens at head_dim 128), parts on CUs of
+// their own are worth the second launch that merges them (Llama-3-8B sizes, 512-token prompts, batch 1 / 4 / 8:
+// 3.86 / 3.95 / 3.96 -> 3.76 / 3.88 / 3.91 ms; batch 16, 128 workgroups: 4.01 -> 4.06, hence the limit; at
+// head_dim 64 the same cut at 512 to 768 tokens gained nothing: 0.905 -> 0.911 ms).
+constexpr int kFusFewWorkgroups = 64;
+constexpr int kFusFewBytes = 256 << 10;
+static int fused_parts(int T, int nkv, int hd, int max_context, int* part_chunks) {
   const int nchunks = max_context > 0 ? (max_context + kFusChunk - 1) / kFusChunk : 1;
   long long parts = 1;
-  if (max_context > kFusSingleMax) {
-    const long long wgs = static_cast<long long>(T) * nkv;
+  const long long wgs = static_cast<long long>(T) * nkv;
+  const bool few = wgs <= kFusFewWorkgroups && static_cast<long long>(max_context) * hd * 4 > kFusFewBytes;
+  if (max_context > kFusSingleMax || few) {
     parts = (kFusTargetWorkgroups + wgs - 1) / wgs;
     if (parts > nchunks) parts = nchunks;
     if (parts < 1) parts = 1;
@@ -469,7 +477,7 @@ static int fused_parts(int T, int nkv, int max_context, int* part_chunks) {
 // Floats of scratch a launch of these sizes needs (0: contexts are not cut).
 long long kvcm_attention_decode_fused_scratch(int T, int nh, int nkv, int hd, int max_context) {
   int pc;
-  const int parts = fused_parts(T, nkv, max_context, &pc);
+  const int parts = fused_parts(T, nkv, hd, max_context, &pc);
   return parts <= 1 ? 0 : static_cast<long long>(T) * nh * parts * (hd + 2);
 }
 
@@ -497,7 +505,7 @@ int kvcm_attention_decode_fused(const float* partials, int S, const void* qkv, i
                "attention_decode_fused: operands must be 16-byte aligned");
   const size_t pstride = size_t(T) * (nh + 2 * nkv) * hd;
   int part_chunks;
-  const int parts = fused_parts(T, nkv, max_context, &part_chunks);
+  const int parts = fused_parts(T, nkv, hd, max_context, &part_chunks);
   KVCM_REQUIRE(parts <= 65535, "attention_decode_fused: context too long");
   const long long need = kvcm_attention_decode_fused_scratch(T, nh, nkv, hd, max_context);
   KVCM_REQUIRE(need == 0 || (scratch != nullptr && scratch_floats >= need),
