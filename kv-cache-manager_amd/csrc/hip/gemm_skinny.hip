@@ -183,10 +183,12 @@ constexpr int kRowBlock = 128;
 template <int MT, int DEPTH, class TO, bool SWIGLU, int NWV>
 __global__ void __launch_bounds__(NWV * kWave)
     gemm_rows_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ partials,
-                     TO* __restrict__ out, int M, int N, int K, int ldx, int ldw, int ldo, int S) {
+                     TO* __restrict__ out, int M, int N, int K, int ldx, int ldw, int ldo, int S,
+                     const float* __restrict__ ss_in, int tiles_in, float eps) {
   constexpr int kPassRows = NWV * kWave / 4;                      // rows the workgroup's threads stage at a time (x 64 k)
   constexpr int RP = (MT * 16 + kPassRows - 1) / kPassRows;       // staging passes
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16][DEPTH * kUnit + kXPad];
+  __shared__ float rstd_s[MT * 16];   // ss_in: every row's 1 / sqrt(mean x^2 + eps), which the unsplit result is scaled by
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int r = lane % 16, kq = lane / 16;
   constexpr int kCols = SWIGLU ? 8 : 16;
@@ -270,9 +272,22 @@ __global__ void __launch_bounds__(NWV * kWave)
   // Two trips in registers: while one is multiplied, the next one's loads are on their way.  LDS
   // buffer i holds the X of the trip in register set i; a buffer is written one barrier after its
   // last read.
+  // X = round(g round(x)) of a norm folded into this product (gemm_rows8.hip): the rows' scales from their
+  // tiles' sums of squares, a wave per row, added in a fixed order while the first loads are on their way
+  auto scales = [&]() {
+    if (ss_in == nullptr) return;
+    for (int m = wave; m < MT * 16; m += NWV) {
+      const float* p = ss_in + size_t(row_base + m < M ? row_base + m : row_base) * tiles_in;
+      float part = 0.f;
+      for (int t = lane; t < tiles_in; t += kWave) part += p[t];
+      const float sum = wave_sum(part);
+      if (lane == 0) rstd_s[m] = rsqrtf(sum / float(tiles_in * 8) + eps);
+    }
+  };
   if (u_lo < u_hi) {
     Trip ta, tb;
     fetch(0, ta);
+    scales();
     for (int i = 0; i < trips; i += 2) {
       const int j0 = i * DEPTH;
       fetch(j0 + DEPTH, tb);
@@ -285,6 +300,15 @@ __global__ void __launch_bounds__(NWV * kWave)
       __syncthreads();
       multiply(1, j0 + DEPTH, tb);
     }
+  } else {
+    scales();
+  }
+  if (ss_in != nullptr) {   // (the same for the whole workgroup)
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[t][i] *= rstd_s[t * 16 + kq * 4 + i];
   }
   if (!col_on) return;
   // accumulator: column = r of the wave's tile, rows = 4 kq + i
@@ -380,12 +404,13 @@ static int rows_splits(int M, int N, int K) {
 // several), two k-depths: four units per trip up to 64 rows, two beyond (LDS holds rows x depth).
 template <class TO, bool SWIGLU, int NWV>
 static void launch_rows_n(hipStream_t st, const uint16_t* x, const uint16_t* w, float* partials, TO* out, int M, int N,
-                          int K, int ldx, int ldw, int ldo, int S) {
+                          int K, int ldx, int ldw, int ldo, int S, const float* ss_in, int tiles_in, float eps) {
   const int mt = rows_tiles_m(M);
   const int tiles = N / (SWIGLU ? 8 : 16);
   const dim3 grid((tiles + NWV - 1) / NWV, S, row_blocks(M));
 #define KVCM_ROWS(MT, DEPTH) \
-  gemm_rows_kernel<MT, DEPTH, TO, SWIGLU, NWV><<<grid, NWV * kWave, 0, st>>>(x, w, partials, out, M, N, K, ldx, ldw, ldo, S)
+  gemm_rows_kernel<MT, DEPTH, TO, SWIGLU, NWV><<<grid, NWV * kWave, 0, st>>>(x, w, partials, out, M, N, K, ldx, ldw, ldo, S, \
+                                                                             ss_in, tiles_in, eps)
   switch (mt) {
     case 1: KVCM_ROWS(1, 4); break;
     case 2: KVCM_ROWS(2, 4); break;
@@ -401,10 +426,10 @@ static void launch_rows_n(hipStream_t st, const uint16_t* x, const uint16_t* w, 
 // tiles) keeps four waves.
 template <class TO, bool SWIGLU>
 static void launch_rows(hipStream_t st, const uint16_t* x, const uint16_t* w, float* partials, TO* out, int M, int N, int K,
-                        int ldx, int ldw, int ldo, int S) {
+                        int ldx, int ldw, int ldo, int S, const float* ss_in = nullptr, int tiles_in = 0, float eps = 0.f) {
   const long long units = static_cast<long long>(N / (SWIGLU ? 8 : 16)) * row_blocks(M) * S;
   const int waves = sizeof(TO) == 4 || (S == 1 && !SWIGLU) ? 4 : rows_waves(units, rows_tiles_m(M));
-#define KVCM_WAVES(NWV) launch_rows_n<TO, SWIGLU, NWV>(st, x, w, partials, out, M, N, K, ldx, ldw, ldo, S)
+#define KVCM_WAVES(NWV) launch_rows_n<TO, SWIGLU, NWV>(st, x, w, partials, out, M, N, K, ldx, ldw, ldo, S, ss_in, tiles_in, eps)
   if constexpr (sizeof(TO) == 4) {
     KVCM_WAVES(4);
   } else {
@@ -514,6 +539,26 @@ int kvcm_gemm_skinny_swiglu(const void* X, const void* W, void* out, int out_dty
   }
 #undef KVCM_SKINNY
   return launch_status("gemm_skinny_swiglu");
+}
+
+// The same with a folded RMS norm in front (gemm_rows8.hip): X is xg = round(g round(x)) of the norm's producer,
+// ss_in its [M][tiles_in] sums of x^2 per 8-column tile, eps the norm's; the sums are scaled by
+// rsqrt(mean x^2 + eps) before they are rounded.  For the widths at which this kernel's few long-lived
+// workgroups stream the gate/up matrix faster than the 8-row kernel's many short ones (from 1,024 tiles on:
+// Llama-3-8B sizes, one row: 50.8 against 43.9 us).
+int kvcm_gemm_skinny_swiglu_normed_preferred(int M, int I, int K) {
+  return K > 0 && K % kUnit == 0 && swiglu_shares_rows(M, I) && I / 8 >= 4 * kRowsCUs;
+}
+int kvcm_gemm_skinny_swiglu_normed(const void* X, const void* W, const float* ss_in, int tiles_in, float eps, void* out,
+                                   int M, int I, int K, int ldx, int ldw, int ldo, hipStream_t st) {
+  KVCM_REQUIRE(K > 0 && K % kUnit == 0 && swiglu_shares_rows(M, I), "gemm_skinny_swiglu_normed: unsupported shape M=%d I=%d K=%d", M, I, K);
+  KVCM_REQUIRE(ss_in != nullptr && tiles_in > 0 && tiles_in * 8 == K, "gemm_skinny_swiglu_normed: %d tiles of sums for a width of %d", tiles_in, K);
+  KVCM_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0 && reinterpret_cast<uintptr_t>(X) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0,
+               "gemm_skinny_swiglu_normed: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
+  KVCM_REQUIRE(ldx >= K && ldw >= K && out != nullptr && ldo >= I, "gemm_skinny_swiglu_normed: leading dimensions too small");
+  launch_rows<bf16_t, true>(st, static_cast<const uint16_t*>(X), static_cast<const uint16_t*>(W), nullptr, static_cast<bf16_t*>(out),
+                            M, I, K, ldx, ldw, ldo, 1, ss_in, tiles_in, eps);
+  return launch_status("gemm_rows_swiglu_normed");
 }
 
 int kvcm_reduce_store(const float* partials, void* out, int out_dtype, int M, int N, int ldo, int S, hipStream_t st) {

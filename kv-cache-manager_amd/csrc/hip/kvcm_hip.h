@@ -27,6 +27,11 @@ int kvcm_reduce_store(const float* partials, void* out, int out_dtype, int M, in
 // Waves per workgroup of the shared-rows kernel for a bfloat16 product of this shape (0: another kernel takes it):
 // chosen so that column tiles x splits x row blocks come to about one workgroup per CU.
 int kvcm_gemm_skinny_waves(int M, int N, int K, int S, int swiglu);
+// act = swiglu(rstd * (xg * [gate | up]^T)) for the rows xg and tile sums ss_in that a folded norm's producer left
+// (kvcm_gemm8_residual_norm), by the shared-rows kernel; `preferred`: the widths at which it beats kvcm_gemm8.
+int kvcm_gemm_skinny_swiglu_normed_preferred(int M, int I, int K);
+int kvcm_gemm_skinny_swiglu_normed(const void* X, const void* W, const float* ss_in, int tiles_in, float eps, void* out,
+                                   int M, int I, int K, int ldx, int ldw, int ldo, hipStream_t stream);
 
 // The same product, whole (split where kvcm_gemm_skinny_splits says so, partial sums added up in
 // split order, result in `out`), for callers that cannot allocate device memory: code under HIP

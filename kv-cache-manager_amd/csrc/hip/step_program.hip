@@ -79,6 +79,7 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_gemm_skinny),
     KVCM_ENTRY(kvcm_reduce_store),
     KVCM_ENTRY(kvcm_gemm_skinny_swiglu),
+    KVCM_ENTRY(kvcm_gemm_skinny_swiglu_normed),
     KVCM_ENTRY(kvcm_gemm_f32),
     KVCM_ENTRY(kvcm_gemm_bf16),
     KVCM_ENTRY(kvcm_gemm_library),

@@ -46,6 +46,8 @@ def _declare(lib):
     fn("kvcm_gemm_skinny_swiglu", vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_gemm_skinny_splits", i, i, i)
     fn("kvcm_gemm_skinny_waves", i, i, i, i, i)
+    fn("kvcm_gemm_skinny_swiglu_normed_preferred", i, i, i)
+    fn("kvcm_gemm_skinny_swiglu_normed", vp, vp, vp, i, f, vp, i, i, i, i, i, i, vp)
     fn("kvcm_gemm_skinny", vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp)
     fn("kvcm_reduce_store", vp, vp, i, i, i, i, i, vp)
     fn("kvcm_swiglu", vp, vp, i, i, i, vp)
@@ -584,7 +586,11 @@ def gemm_swiglu(x, w_gate_up, out):
         if not (w_gate_up.dtype == out.dtype == torch.bfloat16 and tuple(w_gate_up.shape) == (2 * I, K) and out.shape[0] == M
                 and gemm8_supported(M, I, K) and w_gate_up.stride(0) % 8 == 0 and w_gate_up.data_ptr() % 16 == 0):
             return False          # the caller materializes the rows and comes again
-        _gemm8(x, w_gate_up, out, I, True)
+        if lib().kvcm_gemm_skinny_swiglu_normed_preferred(M, I, K) and x.xg.stride(0) % 8 == 0:
+            _call("kvcm_gemm_skinny_swiglu_normed", _ptr(x.xg), _ptr(w_gate_up), _ptr(x.ss), x.ss.shape[1], x.eps, _ptr(out),
+                  M, I, K, x.xg.stride(0), w_gate_up.stride(0), out.stride(0), _stream())
+        else:
+            _gemm8(x, w_gate_up, out, I, True)
         return True
     _dev(x, w_gate_up, out)
     for t, n in ((x, "x"), (w_gate_up, "w_gate_up"), (out, "out")):

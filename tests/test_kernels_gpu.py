@@ -1227,8 +1227,10 @@ def test_products_with_the_norm_folded_in(ops, M, H, K, N2):
 
 
 @pytest.mark.parametrize("M", [1, 5, 8])
-@pytest.mark.parametrize("H,I", [(2048, 5632), (192, 144), (64, 16)])
+@pytest.mark.parametrize("H,I", [(2048, 5632), (192, 144), (64, 16), (320, 8192 + 64)])
 def test_gate_up_product_with_the_norm_folded_in_applies_swiglu(ops, M, H, I):
+    """(the widest case goes through the shared-rows kernel's form of it, which very wide gate/up matrices take)"""
+    assert bool(ops.lib().kvcm_gemm_skinny_swiglu_normed_preferred(M, I, H)) == (I > 8192)
     rng = np.random.default_rng(M + H + I)
     x = (rng.normal(size=(M, H)) * 2).astype(np.float32).astype(np.float64)
     g = _bf16_grid(1 + 0.1 * rng.normal(size=H))
