@@ -200,6 +200,7 @@ __global__ void __launch_bounds__(kDecWaves* kWave)
 // in LDS, so that a long context (hundreds of partitions) costs a few trips to memory, not one
 // per partition.
 constexpr int kMergeThreads = 256;
+constexpr int kMergeFew = 8;       // parts up to which a thread merges its element alone
 
 template <int HD>
 __global__ void __launch_bounds__(kMergeThreads)
@@ -219,6 +220,28 @@ attention_decode_merge_kernel(const float* __restrict__ scratch, const int* __re
   }
   const int np = (ctx + part_tokens - 1) / part_tokens;
   const float* base = scratch + (size_t(row) * nh + head) * num_parts * (HD + 2);
+  if (np <= kMergeFew) {
+    // a few parts: every thread of the first group asks for all it needs at once (one trip to memory, no barrier)
+    if (g != 0) return;
+    float pm[kMergeFew], pl[kMergeFew], po[kMergeFew];
+#pragma unroll
+    for (int i = 0; i < kMergeFew; ++i) {
+      const float* part = base + size_t(i < np ? i : 0) * (HD + 2);
+      pm[i] = part[HD]; pl[i] = part[HD + 1]; po[i] = part[d];
+    }
+    float top = -FLT_MAX;
+#pragma unroll
+    for (int i = 0; i < kMergeFew; ++i) top = i < np ? fmaxf(top, pm[i]) : top;
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMergeFew; ++i) {
+      const float w = i < np ? pl[i] * expf(pm[i] - top) : 0.f;
+      num = fmaf(w, po[i], num);
+      den += w;
+    }
+    *o = float_to_bf16_bits(num / den);
+    return;
+  }
   float m = -FLT_MAX;
   for (int i = tid; i < np; i += kMergeThreads) m = fmaxf(m, base[i * (HD + 2) + HD]);
   m = wave_max(m);

@@ -277,10 +277,19 @@ __global__ void __launch_bounds__(NWV * kWave)
   auto scales = [&]() {
     if (ss_in == nullptr) return;
     for (int m = wave; m < MT * 16; m += NWV) {
-      const float* p = ss_in + size_t(row_base + m < M ? row_base + m : row_base) * tiles_in;
-      float part = 0.f;
-      for (int t = lane; t < tiles_in; t += kWave) part += p[t];
-      const float sum = wave_sum(part);
+      if (row_base + m >= M) {   // a row the block does not have: its sums are dropped at the store
+        if (lane == 0) rstd_s[m] = 1.f;
+        continue;
+      }
+      const float* p = ss_in + size_t(row_base + m) * tiles_in;
+      float part[4] = {0.f, 0.f, 0.f, 0.f};   // four loads on their way per lane
+      int t = lane;
+      for (; t + 3 * kWave < tiles_in; t += 4 * kWave) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) part[q] += p[t + q * kWave];
+      }
+      for (; t < tiles_in; t += kWave) part[0] += p[t];
+      const float sum = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
       if (lane == 0) rstd_s[m] = rsqrtf(sum / float(tiles_in * 8) + eps);
     }
   };
