@@ -185,10 +185,10 @@ class ModelRunner:
     # columns), so a folded step's time grows with its rows by about a ninth of the layers' weight bytes at
     # L2 speed, while the unfolded path (rows shared through LDS, two norm launches a layer more) costs the
     # same from 1 to 16 rows.  Measured: at TinyLlama sizes (88 MB a layer) folding wins at every row count up
-    # to 8 (batch 8: 1.00 against 1.13 ms), at Llama-3-8B sizes (436 MB a layer) a tie at 2 rows and a loss beyond
-    # (batch 4: 4.15 against 3.97 ms, batch 8: 4.61 against 3.96), at Llama-2-7B sizes (405 MB) a loss from 2 rows on
-    # (3.80 against 3.67 ms).  Rows x bytes of a layer's weights up to this pay.
-    FOLD_ROWS_TIMES_LAYER_BYTES = 0.8e9
+    # to 8 (batch 8: 1.00 against 1.13 ms), at Llama-3-8B sizes (436 MB a layer) up to 2 rows (3.61 against 3.89 ms; a tie
+    # at 4 rows, 3.92 both ways; batch 8: 4.61 against 3.96 when it still folded), at Llama-2-7B sizes (405 MB) the same
+    # (2 rows: 3.47 against 3.57 ms, 4 rows 3.71 both ways).  Rows x bytes of a layer's weights up to this pay.
+    FOLD_ROWS_TIMES_LAYER_BYTES = 1.0e9
 
     def _fold_rows(self) -> int:
         layers = max(1, len(self.model.spec.schedule))
