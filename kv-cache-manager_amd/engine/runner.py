@@ -190,10 +190,14 @@ class ModelRunner:
     # (2 rows: 3.47 against 3.57 ms, 4 rows 3.71 both ways).  Rows x bytes of a layer's weights up to this pay.
     FOLD_ROWS_TIMES_LAYER_BYTES = 1.0e9
 
+    @classmethod
+    def fold_rows_for(cls, layer_bytes: float, most_rows: int) -> int:
+        """The most rows a step may have for its norms to be folded, for layers of ``layer_bytes`` of weights."""
+        return max(1, min(int(most_rows), int(cls.FOLD_ROWS_TIMES_LAYER_BYTES // max(1.0, float(layer_bytes)))))
+
     def _fold_rows(self) -> int:
         layers = max(1, len(self.model.spec.schedule))
-        per_layer = max(1.0, self.model.step_bytes(1, 0) / layers)
-        return max(1, min(self.ops.FUSED_NORM_MAX_ROWS, int(self.FOLD_ROWS_TIMES_LAYER_BYTES // per_layer)))
+        return self.fold_rows_for(self.model.step_bytes(1, 0) / layers, self.ops.FUSED_NORM_MAX_ROWS)
 
     def host_buffer(self) -> np.ndarray:
         """The pinned metadata buffer, once the previous step's upload no longer reads it."""

@@ -222,3 +222,15 @@ def test_every_part_of_a_layer_that_needs_a_cache_gets_one_under_any_name():
         model([layer("a"), layer("r", {"look": "a.remember2"})])
     with pytest.raises(ValueError, match="does not have"):
         model([layer("a"), layer("r", {"lok": "a"})])
+
+
+def test_norms_fold_up_to_fewer_rows_the_wider_the_layers():
+    """Rows x a layer's weight bytes up to a constant fold: 8 rows at TinyLlama sizes, 2 at 7B / 8B sizes, never
+    fewer than one."""
+    from kvcm_amd.engine.runner import ModelRunner
+    tiny = 2 * (2560 * 2048 + 2048 * 2048 + 2 * 5632 * 2048 + 2048 * 5632)           # bfloat16 bytes of a layer
+    eight_b = 2 * (6144 * 4096 + 4096 * 4096 + 2 * 14336 * 4096 + 4096 * 14336)
+    seven_b = 2 * (3 * 4096 * 4096 + 4096 * 4096 + 3 * 11008 * 4096)
+    assert ModelRunner.fold_rows_for(tiny, 8) == 8 and ModelRunner.fold_rows_for(eight_b, 8) == 2
+    assert ModelRunner.fold_rows_for(seven_b, 8) == 2 and ModelRunner.fold_rows_for(5e9, 8) == 1
+    assert ModelRunner.fold_rows_for(1e6, 8) == 8 and ModelRunner.fold_rows_for(tiny, 4) == 4
